@@ -1,0 +1,72 @@
+// Shared device helpers for the gfx950 kernels: bfloat16 storage type, wave-wide reductions for
+// 64-lane wavefronts, and the error-reporting convention of the extern "C" entry points.
+//
+// Every entry point returns 0 on success. On a refused size or a failed launch it returns a
+// non-zero code and leaves a message that me_last_error() hands to the caller; nothing is
+// launched in that case, so a refused size never produces a wrong result.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define ME_WAVE 64
+
+extern "C" const char* me_last_error();
+int me_fail(const char* fmt, ...);
+int me_check_launch(const char* what);
+
+enum MeDtype { ME_F32 = 0, ME_BF16 = 1 };
+
+// ------------------------------------------------------------------ bfloat16 as raw 16 bits
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest, ties to even
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_float(float f);
+template <>
+__device__ __forceinline__ float from_float<float>(float f) {
+  return f;
+}
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
+  bf16_t r;
+  r.bits = f32_to_bf16_bits(f);
+  return r;
+}
+
+// ------------------------------------------------------------------ wave and block reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, ME_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, ME_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads. `scratch` holds 16 floats of LDS. Every thread gets
+// the result; the order of additions is fixed by the thread layout alone.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (ME_WAVE - 1), wave = threadIdx.x / ME_WAVE;
+  const int nwaves = (blockDim.x + ME_WAVE - 1) / ME_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}

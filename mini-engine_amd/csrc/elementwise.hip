@@ -1,0 +1,255 @@
+// Row-wise kernels around the matrix products: embedding lookup, residual add + RMSNorm,
+// SwiGLU, and the fused per-head q/k RMSNorm + rotary encoding + key/value page write.
+//
+// All arithmetic is float32; T is the storage type of activations (float or bf16_t). The residual
+// stream and the norm weights are float32 in both modes.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------- embedding
+// x[t, :] = table[ids[t], :] as float32. One block per token.
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ ids,
+                             int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // ids are validated on the host; never fault
+  const T* row = table + (size_t)id * hidden;
+  float* out = x + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_float(row[i]);
+}
+
+extern "C" int me_embed(void* x, const void* table, const int* ids, int num_tokens, int hidden, int vocab,
+                        int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (hidden <= 0 || vocab <= 0) return me_fail("me_embed: hidden=%d vocab=%d", hidden, vocab);
+  const int threads = hidden >= 256 ? 256 : 64;
+  if (dtype == ME_F32)
+    embed_kernel<float><<<num_tokens, threads, 0, stream>>>((float*)x, (const float*)table, ids, hidden, vocab);
+  else
+    embed_kernel<bf16_t><<<num_tokens, threads, 0, stream>>>((float*)x, (const bf16_t*)table, ids, hidden, vocab);
+  return me_check_launch("me_embed");
+}
+
+// ---------------------------------------------------------------------- residual add + RMSNorm
+// For output row r (input row src = rows ? rows[r] : r):
+//   s = x[src] + (delta ? delta[src] : 0);  if (write_x) x[src] = s;
+//   h[r] = s * rsqrt(mean(s^2) + eps) * w
+// One block per row; the sum of squares is reduced in a fixed order.
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ w,
+                                   T* __restrict__ h, const int* __restrict__ rows, int dim, float eps,
+                                   int write_x) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* xr = x + (size_t)src * dim;
+  const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    float s = xr[i];
+    if (dr) s += to_float(dr[i]);
+    if (write_x && dr) xr[i] = s;
+    ss += s * s;
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = rsqrtf(total / (float)dim + eps);
+  T* hr = h + (size_t)r * dim;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    float s = xr[i];
+    if (dr && !write_x) s += to_float(dr[i]);
+    hr[i] = from_float<T>(s * inv * w[i]);
+  }
+}
+
+extern "C" int me_add_rmsnorm(void* x, const void* delta, const float* w, void* h, const int* rows,
+                              int num_rows, int dim, float eps, int write_x, int dtype, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  if (dim <= 0) return me_fail("me_add_rmsnorm: dim=%d", dim);
+  const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
+  if (dtype == ME_F32)
+    add_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((float*)x, (const float*)delta, w, (float*)h, rows,
+                                                                dim, eps, write_x);
+  else
+    add_rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>((float*)x, (const bf16_t*)delta, w, (bf16_t*)h,
+                                                                 rows, dim, eps, write_x);
+  return me_check_launch("me_add_rmsnorm");
+}
+
+// Plain RMSNorm over rows of T (used by parts tests and by mixers that norm activations):
+// out[r] = in[r] * rsqrt(mean(in[r]^2) + eps) * w
+template <typename T>
+__global__ void rmsnorm_kernel(const T* __restrict__ in, const float* __restrict__ w, T* __restrict__ out, int dim,
+                               float eps) {
+  __shared__ float scratch[16];
+  const T* xr = in + (size_t)blockIdx.x * dim;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    const float s = to_float(xr[i]);
+    ss += s * s;
+  }
+  const float inv = rsqrtf(block_sum(ss, scratch) / (float)dim + eps);
+  T* o = out + (size_t)blockIdx.x * dim;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) o[i] = from_float<T>(to_float(xr[i]) * inv * w[i]);
+}
+
+extern "C" int me_rmsnorm(const void* in, const float* w, void* out, int num_rows, int dim, float eps, int dtype,
+                          hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  if (dim <= 0) return me_fail("me_rmsnorm: dim=%d", dim);
+  const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
+  if (dtype == ME_F32)
+    rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((const float*)in, w, (float*)out, dim, eps);
+  else
+    rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>((const bf16_t*)in, w, (bf16_t*)out, dim, eps);
+  return me_check_launch("me_rmsnorm");
+}
+
+// ------------------------------------------------------------------------------------ SwiGLU
+// act[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)).
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / inter;
+  const int i = (int)(idx - t * inter);
+  const float g = to_float(gu[t * 2 * inter + i]);
+  const float u = to_float(gu[t * 2 * inter + inter + i]);
+  act[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int me_swiglu(const void* gu, void* act, int num_tokens, int inter, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (inter <= 0) return me_fail("me_swiglu: intermediate=%d", inter);
+  const size_t total = (size_t)num_tokens * inter;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((total + threads - 1) / threads);
+  if (dtype == ME_F32)
+    swiglu_kernel<float><<<blocks, threads, 0, stream>>>((const float*)gu, (float*)act, inter, total);
+  else
+    swiglu_kernel<bf16_t><<<blocks, threads, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter, total);
+  return me_check_launch("me_swiglu");
+}
+
+// ------------------------------------------- per-head q/k RMSNorm + rotary + key/value page write
+// qkv is [T, (nh + 2*nkv) * d]: q heads, then k heads, then v heads. One wave per (token, head).
+//   q heads: optional RMSNorm over d with q_w, rotary, written to q_out [T, nh, d];
+//   k heads: optional RMSNorm with k_w, rotary, written to the key page   K[page, kvh, slot, d];
+//   v heads: copied to the transposed value page                          V[page, kvh, d, slot].
+// page = block_table[item, pos / bs], slot = pos % bs. Rotary: pairs (j, j + rd/2), j < rd/2, with
+// angle pos * inv_freq[j]; dims >= rd pass through. inv_freq == nullptr means no rotary.
+// write_kv == 0: qkv is [T, nh * d] and only q is processed (a layer that reads another layer's cache).
+#define ME_MAX_HEAD_DIM 256
+
+template <typename T>
+__global__ void qk_norm_rope_scatter_kernel(const T* __restrict__ qkv, const float* __restrict__ q_w,
+                                            const float* __restrict__ k_w, const float* __restrict__ inv_freq,
+                                            const int* __restrict__ positions, const int* __restrict__ token_item,
+                                            const int* __restrict__ block_table, int table_width,
+                                            T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                            int num_tokens, int nh, int nkv, int d, int rd, int bs, float eps,
+                                            int write_kv) {
+  __shared__ float stage[4][ME_MAX_HEAD_DIM];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int heads_total = write_kv ? nh + 2 * nkv : nh;
+  const long long unit = (long long)blockIdx.x * 4 + wave;
+  if (unit >= (long long)num_tokens * heads_total) return;
+  const int t = (int)(unit / heads_total), hd = (int)(unit % heads_total);
+  const int width = (write_kv ? nh + 2 * nkv : nh) * d;  // q-only rows when nothing is written
+  const T* src = qkv + (size_t)t * width + (size_t)hd * d;
+  const int pos = positions[t];
+  const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
+
+  float vals[ME_MAX_HEAD_DIM / ME_WAVE];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+    const int i = lane + k * ME_WAVE;
+    vals[k] = i < d ? to_float(src[i]) : 0.f;
+    ss += vals[k] * vals[k];
+  }
+  const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
+  if (w) {
+    const float inv = rsqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < d) vals[k] = vals[k] * inv * w[i];
+    }
+  }
+  if (kind != 2 && inv_freq) {
+    float* st = stage[wave];
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < d) st[i] = vals[k];
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS writes of this wave are visible
+    const int half = rd / 2;
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < rd) {
+        const int j = i < half ? i : i - half;
+        const float angle = (float)pos * inv_freq[j];
+        const float c = cosf(angle), s = sinf(angle);
+        vals[k] = i < half ? st[i] * c - st[i + half] * s : st[i] * c + st[i - half] * s;
+      }
+    }
+  }
+
+  if (kind == 0) {
+    T* dst = q_out + ((size_t)t * nh + hd) * d;
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < d) dst[i] = from_float<T>(vals[k]);
+    }
+    return;
+  }
+  const int item = token_item[t];
+  const int page = block_table[(size_t)item * table_width + pos / bs];
+  if (page < 0) return;
+  const int slot = pos % bs;
+  if (kind == 1) {
+    const int kvh = hd - nh;
+    T* dst = k_cache + (((size_t)page * nkv + kvh) * bs + slot) * d;
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < d) dst[i] = from_float<T>(vals[k]);
+    }
+  } else {
+    const int kvh = hd - nh - nkv;
+    T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + slot;
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < d) dst[(size_t)i * bs] = from_float<T>(vals[k]);
+    }
+  }
+}
+
+extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w, const float* inv_freq,
+                                       const int* positions, const int* token_item, const int* block_table,
+                                       int table_width, void* q_out, void* k_cache, void* v_cache, int num_tokens,
+                                       int nh, int nkv, int d, int rd, int bs, float eps, int write_kv, int dtype,
+                                       hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (d <= 0 || d > ME_MAX_HEAD_DIM || d % 2)
+    return me_fail("me_qk_norm_rope_scatter: head_dim=%d must be even and at most %d", d, ME_MAX_HEAD_DIM);
+  if (rd < 0 || rd > d || rd % 2) return me_fail("me_qk_norm_rope_scatter: rotary_dim=%d with head_dim=%d", rd, d);
+  if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
+    return me_fail("me_qk_norm_rope_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
+  const long long units = (long long)num_tokens * (write_kv ? nh + 2 * nkv : nh);
+  const unsigned blocks = (unsigned)((units + 3) / 4);
+  if (dtype == ME_F32)
+    qk_norm_rope_scatter_kernel<float><<<blocks, 256, 0, stream>>>(
+        (const float*)qkv, q_w, k_w, inv_freq, positions, token_item, block_table, table_width, (float*)q_out,
+        (float*)k_cache, (float*)v_cache, num_tokens, nh, nkv, d, rd, bs, eps, write_kv);
+  else
+    qk_norm_rope_scatter_kernel<bf16_t><<<blocks, 256, 0, stream>>>(
+        (const bf16_t*)qkv, q_w, k_w, inv_freq, positions, token_item, block_table, table_width, (bf16_t*)q_out,
+        (bf16_t*)k_cache, (bf16_t*)v_cache, num_tokens, nh, nkv, d, rd, bs, eps, write_kv);
+  return me_check_launch("me_qk_norm_rope_scatter");
+}

@@ -1,0 +1,290 @@
+"""Python entry points of the HIP kernels: each checks on the host that the operands have the
+shapes, dtypes and layout the kernel and its grid assume, then launches on torch's current stream.
+
+Tensors are torch CUDA tensors (torch is the allocator and the stream owner here); the kernels get
+raw device pointers. Nothing in this module computes anything on the CPU or through a torch op,
+except :func:`linear`, which hands large bfloat16 products to the GEMM library as the reference
+hands every projection to one (``src/mini_engine/model.py:97-100, 125-127, 168``).
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .library import check, lib
+
+_F32, _BF16 = 0, 1
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_f = ctypes.c_float
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype is torch.float32:
+        return _F32
+    if dtype is torch.bfloat16:
+        return _BF16
+    raise TypeError(f"kernels take float32 or bfloat16 activations, got {dtype}")
+
+
+def _p(t: torch.Tensor | None) -> _vp:
+    return _vp(None) if t is None else _vp(t.data_ptr())
+
+
+def _stream() -> _vp:
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _want(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: tuple | None = None) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be on the GPU")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype is not dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and s != g for s, g in zip(shape, t.shape)):
+            raise ValueError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+
+
+# ------------------------------------------------------------------------------------ row-wise ops
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``out[t] = float32(table[ids[t]])``; ids int32 [T], table [V, H]."""
+    _want(ids, "ids", torch.int32)
+    _want(table, "table", None, (None, None))
+    t, (v, h) = ids.numel(), table.shape
+    if out is None:
+        out = torch.empty((t, h), dtype=torch.float32, device=table.device)
+    _want(out, "out", torch.float32, (t, h))
+    check(lib().me_embed(_p(out), _p(table), _p(ids), _i(t), _i(h), _i(v), _i(_code(table.dtype)), _stream()))
+    return out
+
+
+def add_rmsnorm(
+    x: torch.Tensor,
+    delta: torch.Tensor | None,
+    weight: torch.Tensor,
+    eps: float,
+    dtype: torch.dtype,
+    out: torch.Tensor | None = None,
+    rows: torch.Tensor | None = None,
+    write_x: bool = True,
+) -> torch.Tensor:
+    """Residual add then RMSNorm. ``x`` float32 [T, D] is the residual stream (updated in place when
+    ``write_x``), ``delta`` [T, D] in ``dtype`` or None, ``weight`` float32 [D]. With ``rows`` (int32
+    [R]) only those rows are read and the result is [R, D]. Returns the normed rows in ``dtype``."""
+    _want(x, "x", torch.float32, (None, None))
+    t, d = x.shape
+    _want(weight, "weight", torch.float32, (d,))
+    if delta is not None:
+        _want(delta, "delta", dtype, (t, d))
+    n = t
+    if rows is not None:
+        _want(rows, "rows", torch.int32)
+        n = rows.numel()
+    if out is None:
+        out = torch.empty((n, d), dtype=dtype, device=x.device)
+    _want(out, "out", dtype, (n, d))
+    check(lib().me_add_rmsnorm(_p(x), _p(delta), _p(weight), _p(out), _p(rows), _i(n), _i(d), _f(eps),
+                               _i(1 if write_x else 0), _i(_code(dtype)), _stream()))
+    return out
+
+
+def rmsnorm(inp: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm over the last dim of ``inp`` [..., D]; weight float32 [D]."""
+    _want(inp, "inp")
+    d = inp.shape[-1]
+    _want(weight, "weight", torch.float32, (d,))
+    if out is None:
+        out = torch.empty_like(inp)
+    _want(out, "out", inp.dtype, tuple(inp.shape))
+    n = inp.numel() // d if d else 0
+    check(lib().me_rmsnorm(_p(inp), _p(weight), _p(out), _i(n), _i(d), _f(eps), _i(_code(inp.dtype)), _stream()))
+    return out
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I]."""
+    _want(gate_up, "gate_up", None, (None, None))
+    t, two_i = gate_up.shape
+    if two_i % 2:
+        raise ValueError(f"gate_up must have an even number of columns, got {two_i}")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((t, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _want(out, "out", gate_up.dtype, (t, inter))
+    check(lib().me_swiglu(_p(gate_up), _p(out), _i(t), _i(inter), _i(_code(gate_up.dtype)), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------------- attention
+
+
+def _check_cache(k_cache, v_cache, dtype, nkv, d, bs):
+    _want(k_cache, "k_cache", dtype, (None, nkv, bs, d))
+    _want(v_cache, "v_cache", dtype, (k_cache.shape[0], nkv, d, bs))
+
+
+def _check_step_index(positions, token_item, block_table, t):
+    _want(positions, "positions", torch.int32, (t,))
+    _want(token_item, "token_item", torch.int32, (t,))
+    _want(block_table, "block_table", torch.int32, (None, None))
+
+
+def qk_norm_rope_scatter(
+    qkv: torch.Tensor,
+    q_weight: torch.Tensor | None,
+    k_weight: torch.Tensor | None,
+    inv_freq: torch.Tensor | None,
+    positions: torch.Tensor,
+    token_item: torch.Tensor,
+    block_table: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    num_heads: int,
+    num_kv_heads: int,
+    head_dim: int,
+    eps: float,
+    write_kv: bool = True,
+    q_out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Per-head q/k RMSNorm (when weights are given), rotary encoding (when ``inv_freq`` float32
+    [rotary_dim/2] is given), and the write of keys and values into their pages.
+
+    qkv [T, (nh + 2 nkv) d] (or [T, nh d] with ``write_kv`` off: q only); k_cache [pages, nkv, bs, d]; v_cache [pages, nkv, d, bs];
+    block_table int32 [items, width]. Returns q [T, nh, d]."""
+    nh, nkv, d = num_heads, num_kv_heads, head_dim
+    _want(qkv, "qkv", None, (None, ((nh + 2 * nkv) if write_kv else nh) * d))
+    t, dtype = qkv.shape[0], qkv.dtype
+    _check_step_index(positions, token_item, block_table, t)
+    bs = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, dtype, nkv, d, bs)
+    for w, name in ((q_weight, "q_weight"), (k_weight, "k_weight")):
+        if w is not None:
+            _want(w, name, torch.float32, (d,))
+    rd = 0
+    if inv_freq is not None:
+        _want(inv_freq, "inv_freq", torch.float32, (None,))
+        rd = 2 * inv_freq.numel()
+    if q_out is None:
+        q_out = torch.empty((t, nh, d), dtype=dtype, device=qkv.device)
+    _want(q_out, "q_out", dtype, (t, nh, d))
+    check(lib().me_qk_norm_rope_scatter(
+        _p(qkv), _p(q_weight), _p(k_weight), _p(inv_freq), _p(positions), _p(token_item), _p(block_table),
+        _i(block_table.shape[1]), _p(q_out), _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(nkv), _i(d), _i(rd),
+        _i(bs), _f(eps), _i(1 if write_kv else 0), _i(_code(dtype)), _stream()))
+    return q_out
+
+
+def attention_general(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    positions: torch.Tensor,
+    token_item: torch.Tensor,
+    block_table: torch.Tensor,
+    scale: float,
+    window: int = 0,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Causal grouped-query attention of q [T, nh, d] over the paged cache; returns [T, nh * d]."""
+    _want(q, "q", None, (None, None, None))
+    t, nh, d = q.shape
+    nkv, bs = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, d, bs)
+    _check_step_index(positions, token_item, block_table, t)
+    if out is None:
+        out = torch.empty((t, nh * d), dtype=q.dtype, device=q.device)
+    _want(out, "out", q.dtype, (t, nh * d))
+    check(lib().me_attention_general(
+        _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]),
+        _p(out), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(_code(q.dtype)), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------ matrix products
+
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_f32(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """float32 ``x @ weight.T`` on the vector units, additions in ascending k for every element."""
+    _want(x, "x", torch.float32, (None, None))
+    m, k = x.shape
+    _want(weight, "weight", torch.float32, (None, k))
+    n = weight.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _want(out, "out", torch.float32, (m, n))
+    check(lib().me_gemm_f32(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _stream()))
+    return out
+
+
+def gemm_bf16_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                     out: torch.Tensor | None = None) -> torch.Tensor:
+    """bfloat16 ``x @ weight.T`` for at most 64 rows of x, float32 accumulation on the matrix cores."""
+    _want(x, "x", torch.bfloat16, (None, None))
+    m, k = x.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0]
+    if m > SKINNY_MAX_ROWS:
+        raise ValueError(f"gemm_bf16_skinny takes at most {SKINNY_MAX_ROWS} rows, got {m}")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _want(out, "out", out_dtype, (m, n))
+    check(lib().me_gemm_bf16_skinny(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(_code(out_dtype)), _stream()))
+    return out
+
+
+def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0)
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``x @ weight.T`` for x [M, K], weight [N, K].
+
+    float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16: the
+    skinny matrix-core kernel for up to 64 rows, else the GEMM library; rows are processed in
+    slices of 64 when a float32 result is wanted from bfloat16 inputs (logits)."""
+    out_dtype = out_dtype or x.dtype
+    if x.dtype is torch.float32:
+        if out_dtype is not torch.float32:
+            raise TypeError("the float32 path keeps float32 results")
+        return gemm_f32(x, weight)
+    if skinny_ok(x, weight):
+        return gemm_bf16_skinny(x, weight, out_dtype)
+    if out_dtype is torch.float32 and x.shape[1] % 8 == 0:
+        out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
+        for lo in range(0, x.shape[0], SKINNY_MAX_ROWS):
+            gemm_bf16_skinny(x[lo:lo + SKINNY_MAX_ROWS], weight, torch.float32, out[lo:lo + SKINNY_MAX_ROWS])
+        return out
+    y = torch.matmul(x, weight.t())
+    return y if out_dtype is y.dtype else y.to(out_dtype)
+
+
+# -------------------------------------------------------------------------------------- sampling
+
+
+def sample(logits: torch.Tensor, temperatures: torch.Tensor | None = None, keys: torch.Tensor | None = None,
+           out: torch.Tensor | None = None) -> torch.Tensor:
+    """One token per row of float32 logits [R, V]: argmax where the row's temperature is 0 (or no
+    temperatures are given), else a draw from softmax(logits / temperature) keyed by ``keys``
+    (int64 [R], any bit pattern)."""
+    _want(logits, "logits", torch.float32, (None, None))
+    r, v = logits.shape
+    if temperatures is not None:
+        _want(temperatures, "temperatures", torch.float32, (r,))
+        if keys is None:
+            raise ValueError("temperature sampling needs one key per row")
+        _want(keys, "keys", torch.int64, (r,))
+    if out is None:
+        out = torch.empty((r,), dtype=torch.int32, device=logits.device)
+    _want(out, "out", torch.int32, (r,))
+    check(lib().me_sample(_p(logits), _i(r), _i(v), _p(temperatures), _p(keys if temperatures is not None else None),
+                          _p(out), _stream()))
+    return out

@@ -1,0 +1,104 @@
+"""Grouped-query attention mixer over a paged key/value cache.
+
+Per step (reference: ``src/mini_engine/model.py:111-119`` and ``attention.py:104-175``):
+one product for q, k and v (the three weights are stacked at load time), then one fused kernel for
+the per-head q/k RMSNorm, the position encoding and the write of the new keys and values into their
+pages, then attention of every new token over the pages of its request (causal, optionally within a
+window), then the output projection.
+
+Sizes and constants all come from the spec: head counts, head size, score scale, eps of the q/k
+norm (None: no norm), window (0: none), position encoding (None: none), and ``cache_from`` (read
+another layer's pages and write none).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..ops import kernels as K
+from ..weights.loader import TensorWant
+from .base import MIXERS, POSITION_ENCODINGS, KVBinding, KVCacheNeed, Mixer
+
+MAX_HEAD_DIM = 256
+
+
+class Attention(Mixer):
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        s = spec
+        if s.num_heads % s.num_kv_heads:
+            raise ValueError(f"{s.num_heads} query heads are not a multiple of {s.num_kv_heads} key/value heads")
+        if s.head_dim % 16 or not 16 <= s.head_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"head_dim={s.head_dim} is not supported: the attention kernels take head sizes "
+                             f"from 16 to {MAX_HEAD_DIM} in steps of 16")
+        if s.window < 0:
+            raise ValueError(f"window={s.window} must be >= 0")
+        self.nh, self.nkv, self.d = s.num_heads, s.num_kv_heads, s.head_dim
+        self.position = None if s.position is None else POSITION_ENCODINGS.build(s.position, dtype, device)
+        self.q_norm_w = self.k_norm_w = None
+        self.w_qkv = self.w_o = None
+        self.binding: KVBinding | None = None
+
+    # ---- weights
+    def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
+        s = self.spec
+        wants = {
+            f"{prefix}.q_proj.weight": TensorWant((s.num_heads * s.head_dim, s.hidden_size)),
+            f"{prefix}.o_proj.weight": TensorWant((s.hidden_size, s.num_heads * s.head_dim)),
+        }
+        if s.cache_from is None:
+            wants[f"{prefix}.k_proj.weight"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
+            wants[f"{prefix}.v_proj.weight"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
+        if s.qk_norm_eps is not None:
+            wants[f"{prefix}.q_norm.weight"] = TensorWant((s.head_dim,), "vector")
+            if s.cache_from is None:
+                wants[f"{prefix}.k_norm.weight"] = TensorWant((s.head_dim,), "vector")
+        return wants
+
+    def load(self, tensors, prefix: str) -> None:
+        s = self.spec
+        q = tensors[f"{prefix}.q_proj.weight"]
+        if s.cache_from is None:
+            self.w_qkv = torch.cat((q, tensors[f"{prefix}.k_proj.weight"], tensors[f"{prefix}.v_proj.weight"]), dim=0)
+        else:
+            self.w_qkv = q.contiguous()
+        self.w_o = tensors[f"{prefix}.o_proj.weight"]
+        if s.qk_norm_eps is not None:
+            self.q_norm_w = tensors[f"{prefix}.q_norm.weight"]
+            self.k_norm_w = tensors.get(f"{prefix}.k_norm.weight")
+
+    # ---- cache
+    def cache_need(self):
+        if self.spec.cache_from is not None:
+            return None
+        return KVCacheNeed(self.nkv, self.d, self.spec.window)
+
+    def cache_source(self):
+        return self.spec.cache_from
+
+    def bind_cache(self, binding: KVBinding) -> None:
+        self.binding = binding
+
+    # ---- step
+    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
+        s, b = self.spec, self.binding
+        if b is None:
+            raise RuntimeError("attention mixer has no cache bound")
+        owns = s.cache_from is None
+        proj = K.linear(h, self.w_qkv)  # [T, (nh + 2 nkv) d] or [T, nh d]
+        table = batch.block_table(b.group)
+        inv_freq = None if self.position is None else self.position.tables()
+        eps = 0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps)
+        q = K.qk_norm_rope_scatter(
+            proj, self.q_norm_w, self.k_norm_w if owns else None, inv_freq, batch.positions, batch.token_item,
+            table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns)
+        out = self.attend(q, batch, table)
+        return K.linear(out, self.w_o)
+
+    def attend(self, q: torch.Tensor, batch, table: torch.Tensor) -> torch.Tensor:
+        b = self.binding
+        return K.attention_general(q, b.k_cache, b.v_cache, batch.positions, batch.token_item, table,
+                                   float(self.spec.scale), int(self.spec.window))
+
+
+MIXERS.register("attention", Attention)

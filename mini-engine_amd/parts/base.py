@@ -1,0 +1,125 @@
+"""Interfaces of the parts a decoder layer is assembled from, and the registries that map a spec's
+``kind`` to its implementation.
+
+A part is built from its spec alone (plus the compute dtype and device); it never learns which model
+it is in. The four interfaces:
+
+``Norm``               ``weight_wants(name)``, ``load(tensors, name)``, ``weight`` / ``eps`` used by the
+                       fused residual-add-and-norm of the block.
+``PositionEncoding``   ``tables(device)`` returns what the mixer's kernel needs (for rotary: inv_freq).
+``Mixer``              ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``cache_need()``,
+                       ``bind_cache(binding)``, ``forward(h, batch) -> [T, hidden]``.
+``FeedForward``        ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``forward(h, batch) -> [T, hidden]``.
+
+``h`` is the normed input [T, hidden] in the compute dtype, ``batch`` a ``StepBatch`` (token
+positions, item boundaries, block tables per cache group, state slots). A mixer states what it
+needs kept between steps through ``cache_need()``:
+
+* ``KVCacheNeed``: paged keys and values (heads, head size, window; 0 = all keys);
+* ``StateNeed``: a fixed-size tensor per live request (a slot);
+* ``None``: nothing.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable
+
+import torch
+
+from ..weights.loader import TensorWant
+
+
+@dataclass(frozen=True)
+class KVCacheNeed:
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0  # 0: every earlier key stays needed
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class KVBinding:
+    """What a mixer with paged keys/values is given: its cache group and this layer's pages."""
+
+    group: int
+    k_cache: torch.Tensor  # [pages, kv_heads, block_size, head_dim]
+    v_cache: torch.Tensor  # [pages, kv_heads, head_dim, block_size]
+    block_size: int
+
+
+@dataclass
+class StateBinding:
+    """What a mixer with per-request state is given: one row per slot (the last row is a spare)."""
+
+    state: torch.Tensor  # [slots + 1, *shape]
+
+
+class Part:
+    def __init__(self, spec: Any, dtype: torch.dtype, device: torch.device):
+        self.spec, self.dtype, self.device = spec, dtype, device
+
+    def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
+        return {}
+
+    def load(self, tensors: dict[str, torch.Tensor], prefix: str) -> None:
+        pass
+
+
+class Norm(Part):
+    weight: torch.Tensor
+    eps: float
+
+
+class PositionEncoding(Part):
+    def tables(self) -> Any:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self) -> KVCacheNeed | StateNeed | None:
+        return None
+
+    def cache_source(self) -> int | None:
+        """Index of another layer whose cache this mixer reads instead of owning one."""
+        return None
+
+    def bind_cache(self, binding: Any) -> None:
+        pass
+
+    def forward(self, h: torch.Tensor, batch: Any) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, batch: Any) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._by_kind: dict[str, Callable[..., Part]] = {}
+
+    def register(self, kind: str, factory: Callable[..., Part]) -> None:
+        self._by_kind[kind] = factory
+
+    def build(self, spec: Any, dtype: torch.dtype, device: torch.device) -> Part:
+        kind = getattr(spec, "kind", None)
+        if kind not in self._by_kind:
+            raise ValueError(f"no {self.what} registered for kind {kind!r}; known: {sorted(self._by_kind)}")
+        return self._by_kind[kind](spec, dtype, device)
+
+    def kinds(self) -> list[str]:
+        return sorted(self._by_kind)
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")

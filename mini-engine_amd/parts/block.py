@@ -1,0 +1,59 @@
+"""Arrangements of a mixer, a feed-forward and their norms into one residual block.
+
+``pre_norm`` (reference: ``src/mini_engine/model.py:142-151``)::
+
+    x = x + mixer(norm1(x));  x = x + ffn(norm2(x))
+
+The residual stream ``x`` is kept in float32 and every sum into it is a float32 sum. A block returns
+its feed-forward output unadded; the next norm kernel (of the next block, or the model's final norm)
+adds it while it norms, so each residual add costs no pass of its own.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..ops import kernels as K
+from .base import FEED_FORWARDS, MIXERS, NORMS
+
+
+class PreNormBlock:
+    def __init__(self, spec, dtype: torch.dtype, device: torch.device):
+        self.spec, self.dtype = spec, dtype
+        self.mixer = MIXERS.build(spec.mixer, dtype, device)
+        self.ffn = FEED_FORWARDS.build(spec.ffn, dtype, device)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
+        self.ffn_norm = NORMS.build(spec.ffn_norm, dtype, device)
+
+    def weight_wants(self):
+        s = self.spec
+        wants = {}
+        wants.update(self.mixer_norm.weight_wants(s.mixer_norm_name))
+        wants.update(self.mixer.weight_wants(s.mixer_prefix))
+        wants.update(self.ffn_norm.weight_wants(s.ffn_norm_name))
+        wants.update(self.ffn.weight_wants(s.ffn_prefix))
+        return wants
+
+    def load(self, tensors) -> None:
+        s = self.spec
+        self.mixer_norm.load(tensors, s.mixer_norm_name)
+        self.mixer.load(tensors, s.mixer_prefix)
+        self.ffn_norm.load(tensors, s.ffn_norm_name)
+        self.ffn.load(tensors, s.ffn_prefix)
+
+    def forward(self, x: torch.Tensor, pending: torch.Tensor | None, batch) -> torch.Tensor:
+        """``x`` float32 [T, H] residual stream (updated in place); ``pending`` is the previous
+        block's output that still has to be added. Returns this block's own pending output."""
+        h = K.add_rmsnorm(x, pending, self.mixer_norm.weight, self.mixer_norm.eps, self.dtype)
+        a = self.mixer.forward(h, batch)
+        h = K.add_rmsnorm(x, a, self.ffn_norm.weight, self.ffn_norm.eps, self.dtype)
+        return self.ffn.forward(h, batch)
+
+
+BLOCK_ARRANGEMENTS = {"pre_norm": PreNormBlock}
+
+
+def build_block(spec, dtype, device):
+    if spec.arrangement not in BLOCK_ARRANGEMENTS:
+        raise ValueError(f"unknown block arrangement {spec.arrangement!r}; known: {sorted(BLOCK_ARRANGEMENTS)}")
+    return BLOCK_ARRANGEMENTS[spec.arrangement](spec, dtype, device)

@@ -1,0 +1,89 @@
+"""The generic decoder: embedding, a list of blocks run in the plan's order, final norm, head.
+
+It is built from a :class:`~mini_engine_amd.config.specs.ModelPlan` alone. The forward pass takes a
+packed batch of new tokens (reference: ``src/mini_engine/model.py:172-188``) and returns float32
+logits for the wanted rows only; rows are selected before the final norm, as the reference does
+(``model.py:186``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import ModelPlan
+from ..ops import kernels as K
+from ..weights.loader import TensorWant, load_tensors
+from .base import NORMS
+from .block import build_block
+
+
+class Decoder:
+    def __init__(self, plan: ModelPlan, dtype: torch.dtype, device: torch.device | str = "cuda"):
+        self.plan, self.dtype, self.device = plan, dtype, torch.device(device)
+        self.blocks = [build_block(spec, dtype, self.device) for spec in plan.layers]
+        self.final_norm = NORMS.build(plan.final_norm, dtype, self.device)
+        self.embed_table: torch.Tensor | None = None
+        self.head: torch.Tensor | None = None
+        for i, blk in enumerate(self.blocks):
+            src = blk.mixer.cache_source()
+            if src is not None and not (0 <= src < len(self.blocks) and self.blocks[src].mixer.cache_source() is None):
+                raise ValueError(f"layer {i} reads the cache of layer {src}, which owns none")
+
+    # ---- weights
+    def weight_wants(self) -> dict[str, TensorWant]:
+        p = self.plan
+        wants = {p.embed_name: TensorWant((p.vocab_size, p.hidden_size))}
+        for blk in self.blocks:
+            wants.update(blk.weight_wants())
+        wants.update(self.final_norm.weight_wants(p.final_norm_name))
+        if not p.tie_word_embeddings:
+            wants[p.head_name] = TensorWant((p.vocab_size, p.hidden_size))
+        return wants
+
+    def load(self, source, progress=None) -> None:
+        """``source`` has ``shapes()`` and ``get(name)``. A stored head is ignored when the head is
+        tied to the embedding (reference: ``model.py:190-195``)."""
+        p = self.plan
+        ignorable = (p.head_name,) if p.tie_word_embeddings else ()
+        tensors = load_tensors(source, self.weight_wants(), self.dtype, self.device, ignorable, progress)
+        self.embed_table = tensors[p.embed_name]
+        self.head = self.embed_table if p.tie_word_embeddings else tensors[p.head_name]
+        for blk in self.blocks:
+            blk.load(tensors)
+        self.final_norm.load(tensors, p.final_norm_name)
+
+    def weight_bytes(self) -> int:
+        """Bytes of every distinct weight tensor a step reads (a tied head counts once)."""
+        seen, total = set(), 0
+        def add(t):
+            nonlocal total
+            if t is not None and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+        add(self.head)
+        add(self.final_norm.weight)
+        for i in set(self.plan.order):
+            for obj in (self.blocks[i].mixer, self.blocks[i].ffn, self.blocks[i].mixer_norm, self.blocks[i].ffn_norm):
+                for v in vars(obj).values():
+                    if isinstance(v, torch.Tensor):
+                        add(v)
+        return total
+
+    # ---- step
+    def forward(self, batch) -> torch.Tensor:
+        """Run the batch's tokens through every layer of ``plan.order``; logits float32 [R, V] for
+        ``batch.want_rows``."""
+        if self.embed_table is None:
+            raise RuntimeError("weights are not loaded")
+        x = K.embed(batch.token_ids, self.embed_table)
+        pending = None
+        for i in self.plan.order:
+            pending = self.blocks[i].forward(x, pending, batch)
+        return self.logits(x, pending, batch.want_rows)
+
+    def logits(self, x: torch.Tensor, pending: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
+        if rows.numel() == 0:
+            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
+        h = K.add_rmsnorm(x, pending, self.final_norm.weight, self.final_norm.eps, self.dtype, rows=rows,
+                          write_x=False)
+        return K.linear(h, self.head, torch.float32)

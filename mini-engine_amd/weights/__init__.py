@@ -1,0 +1,16 @@
+from .loader import FolderSource, TensorWant, WeightError, check_names_and_shapes, load_tensors
+from .random_init import RandomSource, write_model_folder
+from .safetensors_io import read_folder_header, read_header, write_file
+
+__all__ = [
+    "FolderSource",
+    "RandomSource",
+    "TensorWant",
+    "WeightError",
+    "check_names_and_shapes",
+    "load_tensors",
+    "read_folder_header",
+    "read_header",
+    "write_file",
+    "write_model_folder",
+]

@@ -1,0 +1,59 @@
+"""Shared fixtures: tiny Qwen3 configurations with seeded random weights, written to temporary
+model folders. Nothing is downloaded and nothing is committed."""
+
+from __future__ import annotations
+
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.dirname(os.path.abspath(__file__))):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a GPU (run with -m gpu on the GPU box)")
+
+
+def tiny_configs():
+    """Two configurations that differ in every size and option."""
+    from mini_engine_amd.models.qwen3 import Qwen3Config
+
+    a = Qwen3Config(vocab_size=256, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                    num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-6,
+                    rope_theta=10000.0, max_position_embeddings=512, tie_word_embeddings=True)
+    b = Qwen3Config(vocab_size=384, hidden_size=96, intermediate_size=160, num_hidden_layers=3,
+                    num_attention_heads=6, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-5,
+                    rope_theta=1e6, max_position_embeddings=1024, tie_word_embeddings=False)
+    return {"A": a, "B": b}
+
+
+BLOCK_SIZES = {"A": 16, "B": 8}
+
+
+def write_tiny(folder: str, cfg, seed: int = 0, std: float = 0.02, dtype=torch.bfloat16) -> str:
+    from mini_engine_amd.models.qwen3 import plan_from_config
+    from mini_engine_amd.parts.decoder import Decoder
+    from mini_engine_amd.weights import write_model_folder
+
+    wants = Decoder(plan_from_config(cfg), torch.float32, "cpu").weight_wants()
+    write_model_folder(folder, cfg.to_config_json(), wants, seed=seed, dtype=dtype, std=std)
+    return folder
+
+
+@pytest.fixture(scope="session")
+def tiny_folders(tmp_path_factory):
+    """{"A": folder, "B": folder} with bfloat16 weights (both engine dtypes read the same values)."""
+    out = {}
+    for name, cfg in tiny_configs().items():
+        out[name] = write_tiny(str(tmp_path_factory.mktemp(f"tiny_{name}")), cfg, seed=11 + len(out), std=0.05)
+    return out
+
+
+def random_prompt(length: int, vocab: int, seed: int) -> list[int]:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(1, vocab, (length,), generator=g).tolist()
