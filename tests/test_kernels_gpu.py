@@ -1,0 +1,311 @@
+"""Each HIP kernel alone against a plain float32 torch reference of the same op, at sizes other than
+the engine's tiny configurations (odd widths, vocabularies that are no power of two, several head
+sizes and group sizes), in float32 and bfloat16."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def K():
+    from mini_engine_amd.ops import kernels
+
+    return kernels
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype is torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def dev(t):
+    return t.cuda().contiguous()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,vocab", [(72, 301), (1024, 1000)])
+def test_embed(dtype, hidden, vocab):
+    table = torch.randn(vocab, hidden).to(dtype)
+    ids = torch.randint(0, vocab, (37,), dtype=torch.int32)
+    out = K().embed(dev(ids), dev(table))
+    assert out.dtype is torch.float32
+    assert torch.equal(out.cpu(), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,dim", [(5, 72), (3, 1000), (2, 5120), (1, 16)])
+def test_add_rmsnorm(dtype, rows, dim):
+    x, delta, w = torch.randn(rows, dim) * 3, torch.randn(rows, dim).to(dtype), 1 + 0.1 * torch.randn(dim)
+    xd = dev(x.clone())
+    h = K().add_rmsnorm(xd, dev(delta), dev(w), 1e-5, dtype)
+    s = x + delta.float()
+    torch.testing.assert_close(xd.cpu(), s, rtol=1e-6, atol=1e-6)  # the residual sum is a float32 sum
+    torch.testing.assert_close(h.float().cpu(), plain.rms_norm(s, w, 1e-5), **tol(dtype))
+    # no delta: x untouched; rows: gather without writing x
+    xd2 = dev(x.clone())
+    h2 = K().add_rmsnorm(xd2, None, dev(w), 1e-5, dtype)
+    assert torch.equal(xd2.cpu(), x)
+    torch.testing.assert_close(h2.float().cpu(), plain.rms_norm(x, w, 1e-5), **tol(dtype))
+    pick = torch.tensor([rows - 1, 0], dtype=torch.int32)
+    h3 = K().add_rmsnorm(xd2, dev(delta), dev(w), 1e-5, dtype, rows=dev(pick), write_x=False)
+    assert torch.equal(xd2.cpu(), x)
+    torch.testing.assert_close(h3.float().cpu(), plain.rms_norm(s[pick.long()], w, 1e-5), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_rows(dtype):
+    x, w = torch.randn(4, 3, 48).to(dtype), torch.randn(48)
+    out = K().rmsnorm(dev(x), dev(w), 1e-6)
+    torch.testing.assert_close(out.float().cpu(), plain.rms_norm(x.float(), w, 1e-6), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,inter", [(7, 160), (3, 1001)])
+def test_swiglu(dtype, tokens, inter):
+    gu = (torch.randn(tokens, 2 * inter) * 2).to(dtype)
+    out = K().swiglu(dev(gu))
+    g, u = gu.float()[:, :inter], gu.float()[:, inter:]
+    torch.testing.assert_close(out.float().cpu(), plain.silu(g) * u, **tol(dtype))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 50, 33), (5, 130, 72), (70, 64, 100), (129, 257, 48)])
+def test_gemm_f32(m, n, k):
+    x, w = torch.randn(m, k), torch.randn(n, k)
+    out = K().gemm_f32(dev(x), dev(w))
+    torch.testing.assert_close(out.cpu(), (x.double() @ w.double().T).float(), rtol=1e-5, atol=1e-5)
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch():
+    """The value of a row is bit-identical whatever other rows are in the product."""
+    x, w = torch.randn(90, 200), torch.randn(77, 200)
+    whole = K().gemm_f32(dev(x), dev(w)).cpu()
+    for lo, hi in [(0, 1), (63, 65), (89, 90), (10, 80)]:
+        assert torch.equal(K().gemm_f32(dev(x[lo:hi]), dev(w)).cpu(), whole[lo:hi])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 100, 72), (17, 1000, 1024), (64, 33, 160), (33, 151, 3072)])
+def test_gemm_bf16_skinny(m, n, k, out_dtype):
+    x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) * 0.05).bfloat16()
+    out = K().gemm_bf16_skinny(dev(x), dev(w), out_dtype)
+    want = (x.double() @ w.double().T).float()
+    t = dict(rtol=1e-4, atol=1e-4) if out_dtype is torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out.float().cpu(), want, **t)
+
+
+def test_gemm_bf16_skinny_refuses_what_it_cannot_do():
+    from mini_engine_amd.ops.library import KernelError
+
+    x, w = dev(torch.randn(4, 20).bfloat16()), dev(torch.randn(8, 20).bfloat16())
+    with pytest.raises(KernelError, match="multiple of 8"):
+        K().gemm_bf16_skinny(x, w)
+    with pytest.raises(ValueError, match="at most 64"):
+        K().gemm_bf16_skinny(dev(torch.randn(65, 16).bfloat16()), dev(torch.randn(8, 16).bfloat16()))
+
+
+@pytest.mark.parametrize("m,n,k", [(3, 40, 20), (200, 96, 72), (100, 70, 64)])
+def test_linear_bf16_takes_every_shape(m, n, k):
+    x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) * 0.1).bfloat16()
+    want = (x.double() @ w.double().T).float()
+    torch.testing.assert_close(K().linear(dev(x), dev(w)).float().cpu(), want, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(K().linear(dev(x), dev(w), torch.float32).cpu(), want, rtol=1e-2, atol=1e-2)
+
+
+# ------------------------------------------------- q/k norm + rotary + page write, and attention
+def make_paged(items, nkv, d, bs, dtype, num_pages=64, seed=0):
+    """items: list of (cached, new). Returns full k/v per item, scattered tables and the cache holding
+    the cached part of every item (pages used by nobody are filled with large garbage)."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    k_cache = torch.full((num_pages, nkv, bs, d), 50.0).to(dtype)
+    v_cache = torch.full((num_pages, nkv, d, bs), -70.0).to(dtype)
+    tables, ks, vs = [], [], []
+    for cached, new in items:
+        n = cached + new
+        table = [perm.pop() for _ in range(-(-n // bs))]
+        k, v = torch.randn(n, nkv, d, generator=g).to(dtype), torch.randn(n, nkv, d, generator=g).to(dtype)
+        for pos in range(cached):
+            k_cache[table[pos // bs], :, pos % bs, :] = k[pos]
+            v_cache[table[pos // bs], :, :, pos % bs] = v[pos]
+        tables.append(table)
+        ks.append(k)
+        vs.append(v)
+    width = max(len(t) for t in tables)
+    table_t = torch.tensor([t + [0] * (width - len(t)) for t in tables], dtype=torch.int32)
+    positions = torch.tensor([p for c, n in items for p in range(c, c + n)], dtype=torch.int32)
+    token_item = torch.tensor([i for i, (c, n) in enumerate(items) for _ in range(n)], dtype=torch.int32)
+    return k_cache, v_cache, tables, table_t, positions, token_item, ks, vs
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,bs,rd,norm", [(4, 2, 16, 4, 16, True), (6, 1, 32, 8, 32, True),
+                                                  (3, 3, 48, 16, 32, False), (16, 8, 128, 16, 128, True),
+                                                  (2, 1, 256, 32, 0, True)])
+def test_qk_norm_rope_scatter(dtype, nh, nkv, d, bs, rd, norm):
+    items = [(0, 7), (9, 1), (8, 5)]
+    k_cache, v_cache, tables, table_t, positions, token_item, _, _ = make_paged(items, nkv, d, bs, dtype)
+    t = positions.numel()
+    qkv = torch.randn(t, (nh + 2 * nkv) * d).to(dtype)
+    qw, kw = 1 + 0.2 * torch.randn(d), 1 + 0.2 * torch.randn(d)
+    theta, eps = 5000.0, 1e-5
+    inv_freq = (1.0 / (theta ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd))) if rd else None
+    kc, vc = dev(k_cache.clone()), dev(v_cache.clone())
+    q_out = K().qk_norm_rope_scatter(dev(qkv), dev(qw) if norm else None, dev(kw) if norm else None,
+                                     dev(inv_freq) if rd else None, dev(positions), dev(token_item), dev(table_t),
+                                     kc, vc, nh, nkv, d, eps)
+    f = qkv.float()
+    q, k, v = (f[:, : nh * d].view(t, nh, d), f[:, nh * d : (nh + nkv) * d].view(t, nkv, d),
+               f[:, (nh + nkv) * d :].view(t, nkv, d))
+    if norm:
+        q, k = plain.rms_norm(q, qw, eps), plain.rms_norm(k, kw, eps)
+    if rd:
+        cos, sin = plain.rope_tables(positions, rd, theta)
+        q = torch.cat((plain.apply_rope(q[..., :rd], cos, sin), q[..., rd:]), -1)
+        k = torch.cat((plain.apply_rope(k[..., :rd], cos, sin), k[..., rd:]), -1)
+    torch.testing.assert_close(q_out.float().cpu(), q, **tol(dtype))
+    kc, vc = kc.float().cpu(), vc.float().cpu()
+    touched = torch.zeros(k_cache.shape[0], bs, dtype=torch.bool)
+    for i in range(t):
+        table, pos = tables[token_item[i]], int(positions[i])
+        page, slot = table[pos // bs], pos % bs
+        touched[page, slot] = True
+        torch.testing.assert_close(kc[page, :, slot, :], k[i], **tol(dtype))
+        torch.testing.assert_close(vc[page, :, :, slot], v[i], **tol(dtype))
+    # every other slot keeps what it held
+    keep = ~touched
+    assert torch.equal(kc.permute(0, 2, 1, 3)[keep], k_cache.float().permute(0, 2, 1, 3)[keep])
+    assert torch.equal(vc.permute(0, 3, 1, 2)[keep], v_cache.float().permute(0, 3, 1, 2)[keep])
+
+
+def dense_reference(qs, ks, vs, items, scale, window):
+    outs = []
+    for q, k, v, (cached, new) in zip(qs, ks, vs, items):
+        outs.append(plain.grouped_causal_attention(q.float(), k.float(), v.float(), scale, window))
+    return torch.cat(outs).reshape(sum(n for _, n in items), -1)
+
+
+def fill_new(k_cache, v_cache, tables, ks, vs, items, bs):
+    for table, k, v, (cached, new) in zip(tables, ks, vs, items):
+        for pos in range(cached, cached + new):
+            k_cache[table[pos // bs], :, pos % bs, :] = k[pos]
+            v_cache[table[pos // bs], :, :, pos % bs] = v[pos]
+
+
+ATTN_SHAPES = [(4, 2, 16, 4), (6, 1, 32, 8), (5, 5, 48, 16), (16, 8, 128, 16), (8, 2, 64, 32), (4, 4, 256, 16)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,bs", ATTN_SHAPES)
+@pytest.mark.parametrize("window", [0, 5])
+def test_attention_general_mixed_batch(dtype, nh, nkv, d, bs, window):
+    """A fresh prompt, single decoded tokens at several context lengths and a continued portion in
+    one launch, with scattered tables (reference tests/test_attention.py:20 and test_gpu.py:29)."""
+    items = [(0, 7), (9, 1), (8, 5), (0, 1), (15, 1), (16, 1), (63, 2), (130, 1), (60, 70)]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=128)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(5)
+    qs = [torch.randn(n, nh, d, generator=g).to(dtype) for _, n in items]
+    scale = d**-0.5
+    out = K().attention_general(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(positions), dev(token_item),
+                                dev(table_t), scale, window)
+    want = dense_reference(qs, ks, vs, items, scale, window)
+    t = dict(rtol=1e-5, atol=1e-5) if dtype is torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(out.float().cpu(), want, **t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key_at_every_page_edge(dtype):
+    """One key's score is made to stand out by scaling it and the query; the output must be that
+    key's value. Places: first key, both sides of page and tile edges, the last key."""
+    nh, nkv, d, bs, ctx = 4, 2, 32, 16, 300
+    for hot in [0, 15, 16, 17, 63, 64, 65, 127, 128, 255, 256, 298, 299]:
+        items = [(ctx - 1, 1)]
+        k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, seed=hot)
+        direction = torch.randn(d)
+        direction /= direction.norm()
+        ks[0] = (ks[0].float() * 0.1).to(dtype)
+        ks[0][hot] = (direction * 8).to(dtype)
+        k_cache.fill_(0)
+        fill_new(k_cache, v_cache, tables, ks, vs, [(0, ctx)], bs)
+        q = (direction * 40).expand(1, nh, d).to(dtype)
+        out = K().attention_general(dev(q), dev(k_cache), dev(v_cache), dev(positions), dev(token_item), dev(table_t),
+                                    d**-0.5, 0)
+        want = vs[0][hot].float().repeat_interleave(nh // nkv, dim=0).reshape(1, -1)
+        torch.testing.assert_close(out.float().cpu(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_window_edge(dtype):
+    """The key just outside the window must be ignored even when it would dominate, and the key just
+    inside must be found."""
+    nh, nkv, d, bs, ctx, window = 2, 1, 16, 8, 100, 37
+    for hot, seen in [(ctx - window - 1, False), (ctx - window, True)]:
+        items = [(ctx - 1, 1)]
+        k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, seed=3)
+        direction = torch.zeros(d)
+        direction[3] = 1.0
+        ks[0] = (ks[0].float() * 0.05).to(dtype)
+        ks[0][hot] = (direction * 8).to(dtype)
+        fill_new(k_cache, v_cache, tables, ks, vs, [(0, ctx)], bs)
+        q = (direction * 40).expand(1, nh, d).to(dtype)
+        out = K().attention_general(dev(q), dev(k_cache), dev(v_cache), dev(positions), dev(token_item), dev(table_t),
+                                    d**-0.5, window).float().cpu()
+        hot_v = vs[0][hot].float().repeat_interleave(nh, dim=0).reshape(1, -1)
+        if seen:
+            torch.testing.assert_close(out, hot_v, rtol=1e-2, atol=1e-2)
+        else:
+            want = dense_reference([q], ks, vs, [(ctx - 1, 1)], d**-0.5, window)
+            torch.testing.assert_close(out, want, rtol=2e-2, atol=2e-2)
+            assert (out - hot_v).abs().max() > 0.3
+
+
+def test_attention_refuses_bad_sizes():
+    from mini_engine_amd.ops.library import KernelError
+
+    q = dev(torch.zeros(1, 3, 16))
+    kc, vc = dev(torch.zeros(2, 2, 4, 16)), dev(torch.zeros(2, 2, 16, 4))
+    idx = dev(torch.zeros(1, dtype=torch.int32))
+    with pytest.raises(KernelError, match="multiple"):
+        K().attention_general(q, kc, vc, idx, idx, dev(torch.zeros(1, 1, dtype=torch.int32)), 1.0)
+
+
+# -------------------------------------------------------------------------------------- sampling
+@pytest.mark.parametrize("vocab", [7, 384, 5000, 151936])
+def test_argmax_takes_the_first_maximum(vocab):
+    logits = torch.randn(5, vocab)
+    logits[1, vocab - 1] = 99.0
+    logits[2, 0] = 99.0
+    logits[3, vocab // 2] = 50.0
+    logits[3, vocab // 3] = 50.0  # two equal maxima: the lower index wins
+    out = K().sample(dev(logits)).cpu()
+    assert out.tolist() == logits.argmax(-1).tolist()
+    assert out[3] == vocab // 3
+
+
+def test_temperature_sampling_is_keyed_repeatable_and_follows_softmax():
+    from mini_engine_amd.sampling import draw_key
+
+    logits = torch.tensor([[2.0, 1.0, 0.0, -1.0, 0.5, -3.0, 1.5]])
+    n = 20000
+    rows = dev(logits.expand(n, -1).contiguous())
+    temps = dev(torch.full((n,), 0.8))
+    keys = dev(torch.tensor([draw_key(0, 5, i) for i in range(n)], dtype=torch.int64))
+    a = K().sample(rows, temps, keys).cpu()
+    b = K().sample(rows, temps, keys).cpu()
+    assert torch.equal(a, b)  # a draw is a function of its key
+    freq = torch.bincount(a.long(), minlength=7).float() / n
+    want = plain.temperature_probs(logits, 0.8)[0]
+    assert (freq - want).abs().max() < 4 * math.sqrt(0.25 / n) + 1e-3, (freq, want)
+    other = K().sample(rows, temps, dev(torch.tensor([draw_key(1, 5, i) for i in range(n)], dtype=torch.int64))).cpu()
+    assert not torch.equal(a, other)
+    # temperature 0 rows in the same launch are plain argmax; a tiny temperature acts as argmax too
+    mixed = dev(torch.tensor([0.0, 1e-7] * (n // 2)))
+    assert set(K().sample(rows, mixed, keys).cpu().tolist()) == {0}

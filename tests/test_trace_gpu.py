@@ -1,0 +1,151 @@
+"""Replay of the same requests under every way of cutting them, in float32 and bfloat16, on both
+tiny configurations, compared with the plain implementation position by position:
+whole; most in one step and the last 32 tokens one by one; portions of changing size down to two
+tokens; mixed with other requests in a pool so small that pages are used again."""
+
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import trace_helpers as th
+from conftest import BLOCK_SIZES, ROOT, random_prompt, tiny_configs
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [5, 17, 33, 70, 150, 64, 2, 41]
+
+
+def requests_for(name: str) -> dict[str, list[int]]:
+    vocab = tiny_configs()[name].vocab_size
+    return {f"r{i}": random_prompt(n, vocab, seed=100 * i + len(name)) for i, n in enumerate(LENGTHS)}
+
+
+_sessions = {}
+
+
+def session_for(folders, name: str, dtype: str, max_tokens: int):
+    from mini_engine_amd.engine.trace import TraceSession, build_session
+
+    key = (name, dtype, max_tokens)
+    if key not in _sessions:
+        _sessions[key] = TraceSession(build_session(folders[name], dtype, max_tokens, block_size=BLOCK_SIZES[name]))
+    return _sessions[key]
+
+
+_plain = {}
+
+
+def plain_for(folders, name):
+    if name not in _plain:
+        _plain[name] = th.plain_logits(folders[name], requests_for(name))
+    return _plain[name]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_replay_matches_plain(tiny_folders, name, dtype, mode):
+    reqs = requests_for(name)
+    max_tokens = 320  # 150 -> 192, plus two more 64s: a few requests live, pages used again and again
+    steps = {"whole": th.whole, "tail": th.tail_one_by_one, "portions": th.portions,
+             "mixed": lambda r: th.mixed(r, max_tokens, seed=7)}[mode](reqs)
+    if mode == "mixed":
+        assert max(len(s["entries"]) for s in steps) >= 3
+        assert any(len(e["tokens"]) == 1 for s in steps for e in s["entries"]) and any(
+            len(e["tokens"]) > 1 for s in steps if len(s["entries"]) > 1 for e in s["entries"])
+    session = session_for(tiny_folders, name, dtype, max_tokens)
+    got = th.collect(steps, th.replay_in_process(session, steps))
+    want = plain_for(tiny_folders, name)
+    for rid in reqs:
+        th.assert_logits_close(got[rid], want[rid], dtype, f"{name} {dtype} {mode} request {rid}")
+    bm = session.bm
+    assert all(len(p.free_pool) == p.num_blocks for p in bm.pools), "every page must be back in the pool"
+    assert session.engine.runner.graph_replays > 0 or mode in ("whole", "portions")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_modes_agree_with_each_other_beyond_rounding(tiny_folders, dtype):
+    """The logits at a position do not depend on the cut: compare the modes directly (tighter than
+    through the plain implementation in bfloat16, where both share the storage rounding)."""
+    name = "B"
+    reqs = requests_for(name)
+    session = session_for(tiny_folders, name, dtype, 320)
+    results = []
+    for build in (th.whole, th.tail_one_by_one, th.portions, lambda r: th.mixed(r, 320, seed=3)):
+        steps = build(reqs)
+        results.append(th.collect(steps, th.replay_in_process(session, steps)))
+    tol = 2e-5 if dtype == "float32" else 0.02
+    for other in results[1:]:
+        for rid in reqs:
+            err = (other[rid] - results[0][rid]).abs().max().item()
+            assert err < tol * max(1.0, results[0][rid].abs().max().item()), (rid, err)
+
+
+def test_first_tokens_of_a_sequence(tiny_folders):
+    """Positions 0 and 1 alone: a one-token prompt, then its second token."""
+    for name in ("A", "B"):
+        toks = requests_for(name)["r3"][:2]
+        steps = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:1], "want": [0]}], "end": []},
+                 {"step": 1, "entries": [{"id": "x", "tokens": toks[1:], "want": [0]}], "end": ["x"]}]
+        for dtype in ("float32", "bfloat16"):
+            session = session_for(tiny_folders, name, dtype, 320)
+            got = th.collect(steps, th.replay_in_process(session, steps))["x"]
+            want = th.plain_logits(tiny_folders[name], {"x": toks})["x"]
+            th.assert_logits_close(got, want, dtype, f"{name} {dtype} first tokens")
+
+
+def test_wanting_nothing_writes_nothing_and_still_fills_the_cache(tiny_folders):
+    name, dtype = "A", "float32"
+    toks = requests_for(name)["r2"]
+    session = session_for(tiny_folders, name, dtype, 320)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": toks[:20], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": toks[20:], "want": [len(toks) - 21]}], "end": ["q"]}]
+    assert session.run_step(steps[0]) is None
+    last = torch.from_numpy(session.run_step(steps[1]))
+    want = th.plain_logits(tiny_folders[name], {"q": toks})["q"][-1:]
+    th.assert_logits_close(last, want, dtype, "last row after a silent first portion")
+
+
+def test_trace_run_program(tiny_folders, tmp_path):
+    """The program itself, as a child process: stdin steps, `done <step>` lines, .f32 files."""
+    name = "A"
+    reqs = {k: v for k, v in list(requests_for(name).items())[:4]}
+    steps = th.mixed(reqs, 256, seed=1)
+    steps[0]["entries"][0]["want"] = []  # a step's entry may want nothing
+    silent_first = all(not e["want"] for e in steps[0]["entries"])
+    for dtype in ("float32", "bfloat16"):
+        out_dir = tmp_path / dtype
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", tiny_folders[name], "--dtype", dtype,
+             "--out", str(out_dir), "--max-tokens", "256"],
+            input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert proc.stdout.split("\n")[: len(steps)] == [f"done {s['step']}" for s in steps]
+        vocab = tiny_configs()[name].vocab_size
+        outputs = {}
+        for s in steps:
+            path = out_dir / f"{s['step']}.f32"
+            wanted = sum(len(e["want"]) for e in s["entries"])
+            assert path.exists() == (wanted > 0)
+            if wanted:
+                outputs[s["step"]] = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(wanted, vocab))
+        if silent_first:
+            assert 0 not in outputs
+        want = th.plain_logits(tiny_folders[name], reqs)
+        # compare every wanted row with the plain logits at its position
+        fed = {rid: 0 for rid in reqs}
+        for s in steps:
+            r = 0
+            for e in s["entries"]:
+                for w in e["want"]:
+                    th.assert_logits_close(outputs[s["step"]][r : r + 1], want[e["id"]][fed[e["id"]] + w][None], dtype,
+                                           f"program {dtype} step {s['step']} {e['id']}")
+                    r += 1
+                fed[e["id"]] += len(e["tokens"])
