@@ -288,3 +288,79 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor | None = None, keys:
     check(lib().me_sample(_p(logits), _i(r), _i(v), _p(temperatures), _p(keys if temperatures is not None else None),
                           _p(out), _stream()))
     return out
+
+
+# ------------------------------------------------------------- matrix-core attention (bfloat16)
+
+
+def attention_mfma_supported(head_dim: int, block_size: int, group: int = 1) -> bool:
+    """Whether the matrix-core attention kernels take this head size, page size and group size."""
+    return bool(lib().me_attention_mfma_supported(_i(head_dim), _i(block_size))) and group <= 16
+
+
+def decode_splits(items: int, kv_units: int, max_ctx: int, target_waves: int = 2048) -> tuple[int, int]:
+    """(keys per split, number of splits) for the decode kernel: enough waves to fill the chip,
+    splits of at least 64 keys, boundaries at multiples of 64."""
+    want = max(1, target_waves // max(1, items * kv_units))
+    splits = 1
+    while splits * 2 <= want and splits * 2 * 64 <= max(max_ctx, 64):
+        splits *= 2
+    split_keys = -(-max_ctx // splits)
+    split_keys = -(-split_keys // 64) * 64
+    return split_keys, -(-max_ctx // split_keys)
+
+
+def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: float, window: int, max_ctx: int,
+                          out: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention of one new token per item over its cached keys: q [items, nh, d] bfloat16,
+    item_ctx int32 [items] (keys per item, the new one included, each <= max_ctx)."""
+    _want(q, "q", torch.bfloat16, (None, None, None))
+    items, nh, d = q.shape
+    nkv, bs = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, torch.bfloat16, nkv, d, bs)
+    _want(item_ctx, "item_ctx", torch.int32, (items,))
+    _want(block_table, "block_table", torch.int32, (items, None))
+    if block_table.shape[1] * bs < max_ctx:
+        raise ValueError(f"block table of {block_table.shape[1]} pages cannot hold {max_ctx} keys")
+    chunks = -(-(nh // nkv) // 16)
+    split_keys, num_splits = decode_splits(items, nkv * chunks, max_ctx)
+    part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=q.device)
+    _want(out, "out", torch.bfloat16, (items, nh * d))
+    check(lib().me_attention_decode_bf16(
+        _p(q), _p(k_cache), _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out),
+        _p(part_o), _p(part_ml), _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys),
+        _i(num_splits), _i(max_ctx), _stream()))
+    return out
+
+
+def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: list[int], block_table, scale: float,
+                           window: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Causal attention of packed new tokens q [T, nh, d] bfloat16 over the paged cache (which already
+    holds the new tokens' keys and values). item_start int32 [items + 1] are the items' offsets into
+    the packed tokens, ``qlens`` the same lengths on the host (they size the grid)."""
+    _want(q, "q", torch.bfloat16, (None, None, None))
+    t, nh, d = q.shape
+    nkv, bs = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, torch.bfloat16, nkv, d, bs)
+    items = len(qlens)
+    if sum(qlens) != t:
+        raise ValueError(f"item lengths sum to {sum(qlens)}, but q has {t} tokens")
+    _want(positions, "positions", torch.int32, (t,))
+    _want(item_start, "item_start", torch.int32, (items + 1,))
+    _want(block_table, "block_table", torch.int32, (items, None))
+    group = nh // nkv
+    if group > 16:
+        raise ValueError(f"group size {group} exceeds what the matrix-core prefill kernel takes (16)")
+    tpb = 128 // group
+    num_blocks = sum(-(-n // tpb) for n in qlens)
+    if out is None:
+        out = torch.empty((t, nh * d), dtype=torch.bfloat16, device=q.device)
+    _want(out, "out", torch.bfloat16, (t, nh * d))
+    check(lib().me_attention_prefill_bf16(
+        _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(item_start), _i(items), _p(block_table),
+        _i(block_table.shape[1]), _p(out), _i(num_blocks), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
+        _stream()))
+    return out

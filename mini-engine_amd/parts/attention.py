@@ -96,9 +96,18 @@ class Attention(Mixer):
         return K.linear(out, self.w_o)
 
     def attend(self, q: torch.Tensor, batch, table: torch.Tensor) -> torch.Tensor:
-        b = self.binding
-        return K.attention_general(q, b.k_cache, b.v_cache, batch.positions, batch.token_item, table,
-                                   float(self.spec.scale), int(self.spec.window))
+        """bfloat16 with sizes the matrix-core kernels take: the split-context kernel when every item
+        brings one token, else the tiled prefill kernel. Everything else (float32, other head or page
+        sizes): the general kernel."""
+        b, s = self.binding, self.spec
+        scale, window = float(s.scale), int(s.window)
+        if self.dtype is torch.bfloat16 and K.attention_mfma_supported(self.d, b.block_size, self.nh // self.nkv):
+            if batch.decode_only:
+                return K.attention_decode_bf16(q, b.k_cache, b.v_cache, batch.item_ctx, table, scale, window,
+                                               batch.max_ctx)
+            return K.attention_prefill_bf16(q, b.k_cache, b.v_cache, batch.positions, batch.item_start, batch.qlens,
+                                            table, scale, window)
+        return K.attention_general(q, b.k_cache, b.v_cache, batch.positions, batch.token_item, table, scale, window)
 
 
 MIXERS.register("attention", Attention)

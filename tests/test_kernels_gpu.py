@@ -309,3 +309,91 @@ def test_temperature_sampling_is_keyed_repeatable_and_follows_softmax():
     # temperature 0 rows in the same launch are plain argmax; a tiny temperature acts as argmax too
     mixed = dev(torch.tensor([0.0, 1e-7] * (n // 2)))
     assert set(K().sample(rows, mixed, keys).cpu().tolist()) == {0}
+
+
+# -------------------------------------------------------- matrix-core attention kernels (bfloat16)
+MFMA_SHAPES = [(4, 2, 32, 16), (6, 1, 32, 16), (16, 8, 128, 16), (8, 8, 64, 32), (16, 1, 64, 16), (3, 1, 96, 48),
+               (2, 2, 256, 16), (40, 2, 32, 16)]
+
+
+@pytest.mark.parametrize("nh,nkv,d,bs", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_decode_mfma(nh, nkv, d, bs, window):
+    """One new token per item at context lengths around page, tile and split edges (reference
+    tests/test_gpu.py:29 uses [1, 16, 17, 33, 100, 255])."""
+    dtype = torch.bfloat16
+    ctxs = [1, 16, 17, 33, 100, 255, 64, 65, 700]
+    items = [(c - 1, 1) for c in ctxs]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=160)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(9)
+    qs = [torch.randn(1, nh, d, generator=g).to(dtype) for _ in items]
+    scale = d**-0.5
+    want = dense_reference(qs, ks, vs, items, scale, window)
+    item_ctx = torch.tensor(ctxs, dtype=torch.int32)
+    for max_ctx in (max(ctxs), 4096):  # a tight bound, and a graph's fixed bound with mostly empty splits
+        width = -(-max_ctx // bs)
+        wide = torch.zeros(len(items), max(width, table_t.shape[1]), dtype=torch.int32)
+        wide[:, : table_t.shape[1]] = table_t
+        out = K().attention_decode_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide),
+                                        scale, window, max_ctx)
+        torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,bs", [s for s in MFMA_SHAPES if s[0] // s[1] <= 16])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_prefill_mfma(nh, nkv, d, bs, window):
+    dtype = torch.bfloat16
+    items = [(0, 7), (9, 1), (8, 5), (0, 1), (15, 1), (16, 33), (63, 2), (130, 1), (60, 70), (0, 200), (300, 129)]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=256)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(5)
+    qs = [torch.randn(n, nh, d, generator=g).to(dtype) for _, n in items]
+    scale = d**-0.5
+    qlens = [n for _, n in items]
+    item_start = torch.tensor([0] + torch.tensor(qlens).cumsum(0).tolist(), dtype=torch.int32)
+    out = K().attention_prefill_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(positions), dev(item_start),
+                                     qlens, dev(table_t), scale, window)
+    want = dense_reference(qs, ks, vs, items, scale, window)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("kernel", ["decode", "prefill"])
+def test_mfma_attention_finds_one_far_key_and_respects_the_window_edge(kernel):
+    dtype, nh, nkv, d, bs, ctx = torch.bfloat16, 4, 2, 64, 16, 600
+    for hot, window in [(0, 0), (15, 0), (16, 0), (63, 0), (64, 0), (511, 0), (512, 0), (598, 0), (599, 0),
+                        (ctx - 100, 100), (ctx - 101, 100)]:
+        items = [(ctx - 1, 1)]
+        k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, seed=hot)
+        direction = torch.randn(d)
+        direction /= direction.norm()
+        ks[0] = (ks[0].float() * 0.05).to(dtype)
+        ks[0][hot] = (direction * 8).to(dtype)
+        fill_new(k_cache, v_cache, tables, ks, vs, [(0, ctx)], bs)
+        q = (direction * 40).expand(1, nh, d).to(dtype).contiguous()
+        if kernel == "decode":
+            out = K().attention_decode_bf16(dev(q), dev(k_cache), dev(v_cache), dev(torch.tensor([ctx], dtype=torch.int32)),
+                                            dev(table_t), d**-0.5, window, ctx)
+        else:
+            out = K().attention_prefill_bf16(dev(q), dev(k_cache), dev(v_cache), dev(positions),
+                                             dev(torch.tensor([0, 1], dtype=torch.int32)), [1], dev(table_t), d**-0.5, window)
+        out = out.float().cpu()
+        hot_v = vs[0][hot].float().repeat_interleave(nh // nkv, dim=0).reshape(1, -1)
+        seen = window == 0 or hot >= ctx - window
+        if seen:
+            torch.testing.assert_close(out, hot_v, rtol=2e-2, atol=2e-2)
+        else:
+            assert (out - hot_v).abs().max() > 0.3
+            torch.testing.assert_close(out, dense_reference([q], ks, vs, items, d**-0.5, window), rtol=2e-2, atol=2e-2)
+
+
+def test_mfma_attention_refuses_unsupported_sizes():
+    assert not K().attention_mfma_supported(16, 16)
+    assert not K().attention_mfma_supported(128, 8)
+    assert K().attention_mfma_supported(128, 16) and not K().attention_mfma_supported(128, 16, group=17)
+    from mini_engine_amd.ops.library import KernelError
+
+    q = dev(torch.zeros(1, 2, 16, dtype=torch.bfloat16))
+    kc, vc = dev(torch.zeros(2, 1, 16, 16, dtype=torch.bfloat16)), dev(torch.zeros(2, 1, 16, 16, dtype=torch.bfloat16))
+    with pytest.raises(KernelError, match="not supported"):
+        K().attention_decode_bf16(q, kc, vc, dev(torch.ones(1, dtype=torch.int32)), dev(torch.zeros(1, 1, dtype=torch.int32)), 1.0, 0, 16)
