@@ -52,6 +52,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--skip-prefill", action="store_true", help="profiling aid: do not measure the prefill")
+    ap.add_argument("--zero-context", action="store_true",
+                    help="profiling aid: allocate the context's pages without computing them (a decode step's "
+                         "time does not depend on the cached values); the line's 'data' says so")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
@@ -93,11 +97,13 @@ def main() -> int:
         engine.block_manager.free(seq)
         return dt
 
-    prefill_once(args.prefill_tokens)
-    prefill_s = min(prefill_once(args.prefill_tokens) for _ in range(3))
-    pf = prefill_flops(cfg, args.prefill_tokens)
-    prefill = {"value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
-               "ms": round(prefill_s * 1e3, 3), "frac": round(pf / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    prefill = None
+    if not args.skip_prefill:
+        prefill_once(args.prefill_tokens)
+        prefill_s = min(prefill_once(args.prefill_tokens) for _ in range(3))
+        pf = prefill_flops(cfg, args.prefill_tokens)
+        prefill = {"value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
+                   "ms": round(prefill_s * 1e3, 3), "frac": round(pf / prefill_s / PEAK_FLOPS[args.dtype], 4)}
 
     # ---- decode: B sequences at the benchmark context, K timed engine steps
     kv_per_token = engine.runner.storage.kv_bytes_per_token()
@@ -106,6 +112,14 @@ def main() -> int:
     def decode(batch):
         params = SamplingParams(max_tokens=k + w + 1, temperature=0.0, ignore_eos=True)
         seqs = [engine.add_request(prompt(prompt_len), params) for _ in range(batch)]
+        if args.zero_context:
+            from mini_engine_amd.engine.sequence import SequenceStatus
+
+            for s in seqs:  # admit by hand: pages for the whole prompt, all but its last token "computed"
+                engine.scheduler.waiting.remove(s)
+                assert engine.block_manager.try_allocate(s, prompt_len)
+                s.status, s.num_computed_tokens = SequenceStatus.RUNNING, prompt_len - 1
+                engine.scheduler.running.append(s)
         while any(s.num_output_tokens == 0 for s in seqs):
             engine.step()
         for _ in range(w - 1):
@@ -130,7 +144,8 @@ def main() -> int:
         "metric": "decode tok/s at batch 8 (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights",
+        "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights"
+                + (" (context pages allocated, not computed)" if args.zero_context else ""),
         "config": {"model": "Qwen3-0.6B shape", "layers": cfg.num_hidden_layers, "layers_of_config": 28,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,

@@ -174,33 +174,68 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   }
 }
 
-// out[item, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One wave per (item, head).
-__global__ __launch_bounds__(64) void attention_decode_combine_kernel(const float* __restrict__ part_o,
-                                                                      const float* __restrict__ part_ml,
-                                                                      bf16_t* __restrict__ out, int num_splits, int d) {
+// out[item, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One block of 256 threads per
+// (item, head): the weights of all splits first (every split's statistics are loaded at once), then
+// the weighted sum with thread -> (four output elements, one of 256 / (d/4) groups of splits), so
+// that the loads of different splits are independent of each other.
+#define ME_MAX_SPLITS 1024
+__global__ __launch_bounds__(256) void attention_decode_combine_kernel(const float* __restrict__ part_o,
+                                                                       const float* __restrict__ part_ml,
+                                                                       bf16_t* __restrict__ out, int num_splits, int d) {
+  __shared__ float wgt[ME_MAX_SPLITS];
+  __shared__ float red_max[4], red_sum[4];
+  __shared__ float4_t partial[256];
   const size_t unit = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & (ME_WAVE - 1), wave = tid / ME_WAVE;
   const float* ml = part_ml + unit * num_splits * 2;
   float big = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) big = fmaxf(big, ml[s * 2]);
-  float denom = 0.f;
-  float accv[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < num_splits; ++s) {
+  for (int s = tid; s < num_splits; s += 256)
+    if (ml[s * 2 + 1] > 0.f) big = fmaxf(big, ml[s * 2]);
+  big = wave_max(big);
+  if (lane == 0) red_max[wave] = big;
+  __syncthreads();
+  big = fmaxf(fmaxf(red_max[0], red_max[1]), fmaxf(red_max[2], red_max[3]));
+  float part_denom = 0.f;
+  for (int s = tid; s < num_splits; s += 256) {
     const float l = ml[s * 2 + 1];
-    if (l <= 0.f) continue;  // an empty split wrote no usable sum
-    const float wgt = fast_exp2(ml[s * 2] - big);
-    denom += wgt * l;
-    const float* po = part_o + (unit * num_splits + s) * d;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int i = threadIdx.x + k * ME_WAVE;
-      if (i < d) accv[k] += wgt * po[i];
+    const float w = l > 0.f ? fast_exp2(ml[s * 2] - big) : 0.f;  // an empty split has no weight
+    wgt[s] = w;
+    part_denom += w * l;
+  }
+  part_denom = wave_sum(part_denom);
+  if (lane == 0) red_sum[wave] = part_denom;
+  __syncthreads();
+  const float denom = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]);
+
+  const int quads = d / 4;          // d is a multiple of 32, so quads <= 64
+  const int groups = 256 / quads;   // groups of splits handled side by side
+  const int qd = tid % quads, grp = tid / quads;
+  float4_t accv = {0.f, 0.f, 0.f, 0.f};
+  if (grp < groups) {
+    const float* po = part_o + unit * num_splits * d + qd * 4;
+    for (int s = grp; s < num_splits; s += groups) {
+      const float w = wgt[s];
+      const float4_t v = *reinterpret_cast<const float4_t*>(po + (size_t)s * d);
+      accv[0] += w * v[0];
+      accv[1] += w * v[1];
+      accv[2] += w * v[2];
+      accv[3] += w * v[3];
     }
   }
-  const float inv = 1.f / denom;
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int i = threadIdx.x + k * ME_WAVE;
-    if (i < d) out[unit * d + i] = from_float<bf16_t>(accv[k] * inv);
+  partial[tid] = accv;
+  __syncthreads();
+  if (tid < quads) {
+    float4_t total = partial[tid];
+    for (int gi = 1; gi < groups; ++gi) {
+      const float4_t v = partial[gi * quads + tid];
+      total[0] += v[0];
+      total[1] += v[1];
+      total[2] += v[2];
+      total[3] += v[3];
+    }
+    const float inv = 1.f / denom;
+    *reinterpret_cast<short4_t*>(out + unit * d + tid * 4) =
+        pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
   }
 }
 
@@ -235,6 +270,7 @@ extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, cons
     return me_fail("me_attention_decode_bf16: %d splits of %d keys do not cover %d keys", num_splits, split_keys, max_ctx);
   if (table_width * bs < max_ctx)
     return me_fail("me_attention_decode_bf16: block table of %d pages of %d cannot hold %d keys", table_width, bs, max_ctx);
+  if (num_splits > ME_MAX_SPLITS) return me_fail("me_attention_decode_bf16: %d splits exceed %d", num_splits, ME_MAX_SPLITS);
   if (num_splits > 65535 || nkv * ((nh / nkv + 15) / 16) > 65535) return me_fail("me_attention_decode_bf16: grid too large");
   const float sl = scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
@@ -253,7 +289,7 @@ extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, cons
   }
 #undef ME_DECODE_CASE
   if (me_check_launch("me_attention_decode_bf16")) return 1;
-  attention_decode_combine_kernel<<<items * nh, 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d);
+  attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d);
   return me_check_launch("me_attention_decode_combine");
 }
 

@@ -88,7 +88,7 @@ union Frag16 {
   short4_t h[2];
 };
 
-template <int MT, typename OutT>
+template <int MT, int U, typename OutT>
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
                                                                const bf16_t* __restrict__ W,
                                                                OutT* __restrict__ C, int M, int N, int K) {
@@ -103,21 +103,34 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
+  // U chunks of 32 k per round: all loads of a round are issued before the first product, so a
+  // wave keeps U weight loads in flight instead of one
   const int chunks = (K + 31) / 32;
-  for (int c = wave; c < chunks; c += 4) {
-    const int k = c * 32 + g * 8;
-    Frag16 a;
-    a.u = make_uint4(0, 0, 0, 0);
-    if (n_ok && k < K) a.u = *reinterpret_cast<const uint4*>(wrow + k);  // K % 8 == 0 is checked on the host
+  for (int c0 = wave; c0 < chunks; c0 += 4 * U) {
+    Frag16 a[U], b[U][MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int m = t * 16 + r;
-      Frag16 b;
-      b.u = make_uint4(0, 0, 0, 0);
-      if (m < M && k < K) b.u = *reinterpret_cast<const uint4*>(X + (size_t)m * K + k);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.h[0], b.h[0], acc[t], 0, 0, 0);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.h[1], b.h[1], acc[t], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int k = (c0 + 4 * u) * 32 + g * 8;
+      a[u].u = make_uint4(0, 0, 0, 0);
+      if (n_ok && k < K) a[u].u = *reinterpret_cast<const uint4*>(wrow + k);  // K % 8 == 0 is checked on the host
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (c0 + 4 * u) * 32 + g * 8;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r;
+        b[u][t].u = make_uint4(0, 0, 0, 0);
+        if (m < M && k < K) b[u][t].u = *reinterpret_cast<const uint4*>(X + (size_t)m * K + k);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a[u].h[0], b[u][t].h[0], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a[u].h[1], b[u][t].h[1], acc[t], 0, 0, 0);
+      }
   }
 #pragma unroll
   for (int t = 0; t < MT; ++t)
@@ -143,10 +156,10 @@ static int launch_skinny(const bf16_t* X, const bf16_t* W, OutT* C, int M, int N
   const unsigned blocks = (N + 15) / 16;
   const int mt = (M + 15) / 16;
   switch (mt) {
-    case 1: gemm_bf16_skinny_kernel<1, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
-    case 2: gemm_bf16_skinny_kernel<2, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
-    case 3: gemm_bf16_skinny_kernel<3, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
-    default: gemm_bf16_skinny_kernel<4, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
+    case 1: gemm_bf16_skinny_kernel<1, 8, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
+    case 2: gemm_bf16_skinny_kernel<2, 4, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
+    case 3: gemm_bf16_skinny_kernel<3, 4, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
+    default: gemm_bf16_skinny_kernel<4, 4, OutT><<<blocks, 256, 0, stream>>>(X, W, C, M, N, K); break;
   }
   return me_check_launch("me_gemm_bf16_skinny");
 }

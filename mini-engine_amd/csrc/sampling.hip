@@ -22,35 +22,50 @@ __device__ __forceinline__ float gumbel_noise(uint64_t key, int i) {
   return -logf(-logf(uc));
 }
 
-__global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits, int vocab,
-                                                      const float* __restrict__ temperatures,
-                                                      const uint64_t* __restrict__ keys, int* __restrict__ out) {
-  __shared__ float best_v[16];
-  __shared__ int best_i[16];
-  const int row = blockIdx.x;
-  const float* lr = logits + (size_t)row * vocab;
-  const float temp = temperatures ? temperatures[row] : 0.f;
-  const uint64_t key = keys ? keys[row] : 0;
-  const float inv_t = temp > 0.f ? 1.f / fmaxf(temp, 1e-5f) : 1.f;
-  float bv = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    float v = lr[i];
-    if (temp > 0.f) v = v * inv_t + gumbel_noise(key, i);
-    if (v > bv || (v == bv && i < bi)) {
-      bv = v;
-      bi = i;
-    }
+// Stage 1: block (row, chunk) scans a contiguous slice of the vocabulary and writes its best
+// (value, index). Stage 2: one wave per row picks the best of the chunks. Ties go to the lowest index
+// at both stages, so the result is that of a single scan.
+struct Best {
+  float v;
+  int i;
+};
+
+__device__ __forceinline__ void take_better(float& bv, int& bi, float ov, int oi) {
+  if (ov > bv || (ov == bv && oi < bi)) {
+    bv = ov;
+    bi = oi;
   }
+}
+
+__device__ __forceinline__ void wave_best(float& bv, int& bi) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(bv, off, ME_WAVE);
     const int oi = __shfl_xor(bi, off, ME_WAVE);
-    if (ov > bv || (ov == bv && oi < bi)) {
-      bv = ov;
-      bi = oi;
-    }
+    take_better(bv, bi, ov, oi);
   }
+}
+
+__global__ __launch_bounds__(256) void sample_stage1_kernel(const float* __restrict__ logits, int vocab,
+                                                            const float* __restrict__ temperatures,
+                                                            const uint64_t* __restrict__ keys, Best* __restrict__ part,
+                                                            int chunks, int chunk_len) {
+  __shared__ float best_v[4];
+  __shared__ int best_i[4];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const float* lr = logits + (size_t)row * vocab;
+  const float temp = temperatures ? temperatures[row] : 0.f;
+  const uint64_t key = keys ? keys[row] : 0;
+  const float inv_t = temp > 0.f ? 1.f / fmaxf(temp, 1e-5f) : 1.f;
+  const int begin = chunk * chunk_len, end = min(vocab, begin + chunk_len);
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
+    float v = lr[i];
+    if (temp > 0.f) v = v * inv_t + gumbel_noise(key, i);
+    take_better(bv, bi, v, i);
+  }
+  wave_best(bv, bi);
   const int lane = threadIdx.x & (ME_WAVE - 1), wave = threadIdx.x / ME_WAVE;
   if (lane == 0) {
     best_v[wave] = bv;
@@ -58,21 +73,39 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int nwaves = blockDim.x / ME_WAVE;
-    for (int w = 1; w < nwaves; ++w)
-      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
-        bv = best_v[w];
-        bi = best_i[w];
-      }
-    out[row] = bi == 0x7fffffff ? 0 : bi;  // a row of NaNs picks token 0 rather than an invalid id
+    for (int w = 1; w < 4; ++w) take_better(bv, bi, best_v[w], best_i[w]);
+    part[(size_t)row * chunks + chunk].v = bv;
+    part[(size_t)row * chunks + chunk].i = bi;
   }
 }
 
+__global__ __launch_bounds__(64) void sample_stage2_kernel(const Best* __restrict__ part, int chunks,
+                                                           int* __restrict__ out) {
+  const int row = blockIdx.x;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += ME_WAVE) take_better(bv, bi, part[(size_t)row * chunks + c].v,
+                                                                  part[(size_t)row * chunks + c].i);
+  wave_best(bv, bi);
+  if (threadIdx.x == 0) out[row] = bi == 0x7fffffff ? 0 : bi;  // a row of NaNs picks token 0, not an invalid id
+}
+
+// Number of vocabulary slices per row; the workspace holds rows * chunks (float, int) pairs.
+extern "C" int me_sample_chunks(int vocab) {
+  const int c = (vocab + 2047) / 2048;
+  return c < 1 ? 1 : (c > 128 ? 128 : c);
+}
+
 extern "C" int me_sample(const float* logits, int num_rows, int vocab, const float* temperatures,
-                         const uint64_t* keys, int* out, hipStream_t stream) {
+                         const uint64_t* keys, int* out, void* workspace, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   if (vocab <= 0) return me_fail("me_sample: vocab=%d", vocab);
-  const int threads = vocab >= 8192 ? 1024 : (vocab >= 1024 ? 256 : 64);
-  sample_kernel<<<num_rows, threads, 0, stream>>>(logits, vocab, temperatures, keys, out);
-  return me_check_launch("me_sample");
+  if (num_rows > 65535) return me_fail("me_sample: %d rows exceed the grid", num_rows);
+  const int chunks = me_sample_chunks(vocab);
+  const int chunk_len = (vocab + chunks - 1) / chunks;
+  sample_stage1_kernel<<<dim3(num_rows, chunks), 256, 0, stream>>>(logits, vocab, temperatures, keys, (Best*)workspace,
+                                                                   chunks, chunk_len);
+  if (me_check_launch("me_sample stage 1")) return 1;
+  sample_stage2_kernel<<<num_rows, 64, 0, stream>>>((const Best*)workspace, chunks, out);
+  return me_check_launch("me_sample stage 2");
 }

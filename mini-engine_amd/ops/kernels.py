@@ -285,8 +285,10 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor | None = None, keys:
     if out is None:
         out = torch.empty((r,), dtype=torch.int32, device=logits.device)
     _want(out, "out", torch.int32, (r,))
+    chunks = lib().me_sample_chunks(_i(v))
+    workspace = torch.empty((r * chunks * 2,), dtype=torch.float32, device=logits.device)
     check(lib().me_sample(_p(logits), _i(r), _i(v), _p(temperatures), _p(keys if temperatures is not None else None),
-                          _p(out), _stream()))
+                          _p(out), _p(workspace), _stream()))
     return out
 
 
