@@ -1,8 +1,9 @@
-"""Device storage behind the page tables: for every cache group one tensor of key pages and one of
-value pages per layer, and one tensor of state rows for every layer with per-request state.
+"""Device storage behind the page tables: for every run of a layer (a position in the model's
+order) that owns a cache, one tensor of key pages and one of value pages, or one tensor of state
+rows for a mixer with per-request state.
 
-Layers whose mixers state the same need (heads, head size, window) form one group and share one
-block table per request. A page id indexes every layer of its group at once. Each group has one page
+Runs whose mixers state the same need (heads, head size, window) form one group and share one
+block table per request. A page id indexes every run of its group at once. Each group has one page
 more than the manager hands out: rows that pad a replayed graph write there.
 
 Layout of a layer's pages: keys ``[pages, kv_heads, block_size, head_dim]`` and values transposed,
@@ -24,21 +25,23 @@ from .block_manager import GroupSpec
 class CacheLayout:
     groups: list[GroupSpec]
     group_needs: list[KVCacheNeed]
-    layer_group: dict[int, int]  # layer index -> group index, for layers that own pages
-    state_layers: dict[int, StateNeed]
+    layer_group: dict[int, int]  # run (position in the order) -> group index, for runs that own pages
+    state_layers: dict[int, StateNeed]  # run -> its state need
 
     @property
     def has_state(self) -> bool:
         return bool(self.state_layers)
 
 
-def plan_layout(blocks) -> CacheLayout:
-    """Group the layers of a decoder by what their mixers need."""
+def plan_layout(decoder) -> CacheLayout:
+    """Group the runs of a decoder by what their mixers need."""
     needs: list[KVCacheNeed] = []
     layer_group: dict[int, int] = {}
     state_layers: dict[int, StateNeed] = {}
-    for i, blk in enumerate(blocks):
-        need = blk.mixer.cache_need()
+    for i, layer in enumerate(decoder.plan.order):
+        if decoder.cache_owner[i] != i:
+            continue
+        need = decoder.blocks[layer].mixer.cache_need()
         if isinstance(need, KVCacheNeed):
             if need not in needs:
                 needs.append(need)
@@ -52,7 +55,7 @@ def plan_layout(blocks) -> CacheLayout:
 
 
 class CacheStorage:
-    def __init__(self, blocks, layout: CacheLayout, num_blocks: int, block_size: int, num_state_slots: int,
+    def __init__(self, decoder, layout: CacheLayout, num_blocks: int, block_size: int, num_state_slots: int,
                  dtype: torch.dtype, device: torch.device):
         self.layout, self.block_size, self.dtype = layout, block_size, dtype
         self.spare_block = num_blocks  # never handed out by the manager
@@ -66,17 +69,15 @@ class CacheStorage:
             self.kv[i] = (k, v)
         for i, need in layout.state_layers.items():
             self.state[i] = torch.zeros((num_state_slots + 1, *need.shape), dtype=need.dtype, device=device)
-        for i, blk in enumerate(blocks):
-            src = blk.mixer.cache_source()
-            owner = i if src is None else src
+        for r, owner in enumerate(decoder.cache_owner):
             if owner in self.kv:
                 k, v = self.kv[owner]
-                blk.mixer.bind_cache(KVBinding(layout.layer_group[owner], k, v, block_size))
-            elif i in self.state:
-                blk.mixer.bind_cache(StateBinding(self.state[i]))
+                decoder.bindings[r] = KVBinding(layout.layer_group[owner], k, v, block_size)
+            elif r in self.state:
+                decoder.bindings[r] = StateBinding(self.state[r])
 
     def kv_bytes_per_token(self) -> int:
-        """Bytes of keys and values one token occupies over all layers that own pages."""
+        """Bytes of keys and values one token occupies over all runs that own pages."""
         elem = torch.empty((), dtype=self.dtype).element_size()
         return sum(2 * self.layout.group_needs[g].num_kv_heads * self.layout.group_needs[g].head_dim * elem
                    for g in self.layout.layer_group.values())

@@ -146,3 +146,16 @@ def validate_items(items: list[StepItem], vocab_size: int, block_size: int, grou
             for page in table[first_key // block_size : need]:
                 if page < 0:
                     raise ValueError(f"group {g}: a page the step reads or writes was already given back")
+
+
+def make_batch(items: list[StepItem], num_groups: int, device, spare_block: int = 0, spare_slot: int = 0) -> StepBatch:
+    """Pack ``items`` and upload them: the batch an eager step runs on."""
+    arr, t, b, r, widths = pack_host(items, num_groups, spare_block=spare_block, spare_slot=spare_slot)
+    batch = StepBatch(torch.from_numpy(arr).to(device), t, b, r, widths)
+    batch.starts = [it.start for it in items]
+    batch.qlens = [len(it.tokens) for it in items]
+    batch.slots_host = [it.seq.state_slot for it in items]
+    batch.max_qlen = max(batch.qlens)
+    batch.max_ctx = max(s + q for s, q in zip(batch.starts, batch.qlens))
+    batch.decode_only = batch.max_qlen == 1
+    return batch

@@ -33,11 +33,12 @@ class EngineStats:
 
 
 def kv_cache_bytes_per_token(plan: ModelPlan, dtype: str) -> int:
-    """``2 * layers * kv_heads * head_dim * element size`` summed over the layers that own a cache
-    (reference: ``engine.py:54-56``)."""
+    """``2 * kv_heads * head_dim * element size`` summed over the runs of attention layers that own
+    a cache (reference: ``engine.py:54-56``, where that is ``2 * layers * kv_heads * head_dim``)."""
     elem = 4 if dtype == "float32" else 2
-    return sum(2 * l.mixer.num_kv_heads * l.mixer.head_dim * elem for l in plan.layers
-               if getattr(l.mixer, "kind", "") == "attention" and l.mixer.cache_from is None)
+    runs = [plan.layers[i].mixer for i in plan.order]
+    return sum(2 * m.num_kv_heads * m.head_dim * elem for m in runs
+               if getattr(m, "kind", "") == "attention" and m.cache_from is None)
 
 
 class LLMEngine:

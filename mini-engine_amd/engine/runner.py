@@ -17,7 +17,7 @@ from ..cache.block_manager import BlockManager
 from ..cache.storage import CacheStorage, plan_layout
 from ..config.engine_config import EngineConfig
 from ..parts.decoder import Decoder
-from .batch import StepBatch, StepItem, pack_host, section_offsets, validate_items
+from .batch import StepBatch, StepItem, make_batch, pack_host, section_offsets, validate_items
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
@@ -35,8 +35,8 @@ class ModelRunner:
         self.decoder, self.config = decoder, config
         self.device = decoder.device
         self.dtype = decoder.dtype
-        self.layout = plan_layout(decoder.blocks)
-        self.storage = CacheStorage(decoder.blocks, self.layout, config.num_blocks, config.block_size,
+        self.layout = plan_layout(decoder)
+        self.storage = CacheStorage(decoder, self.layout, config.num_blocks, config.block_size,
                                     config.max_num_seqs, self.dtype, self.device)
         self.num_groups = len(self.layout.groups)
         self.max_blocks_per_seq = -(-config.max_model_len // config.block_size)
@@ -64,21 +64,8 @@ class ModelRunner:
         if self._graph_eligible(items):
             return self._replay(items)
         self.eager_steps += 1
-        arr, t, b, r, widths = pack_host(items, self.num_groups, spare_block=self.storage.spare_block,
-                                         spare_slot=self.storage.spare_slot)
-        buf = torch.from_numpy(arr).to(self.device, non_blocking=False)
-        batch = StepBatch(buf, t, b, r, widths)
-        self._describe(batch, items)
+        batch = make_batch(items, self.num_groups, self.device, self.storage.spare_block, self.storage.spare_slot)
         return self.decoder.forward(batch)
-
-    @staticmethod
-    def _describe(batch: StepBatch, items: list[StepItem]) -> None:
-        batch.starts = [it.start for it in items]
-        batch.qlens = [len(it.tokens) for it in items]
-        batch.slots_host = [it.seq.state_slot for it in items]
-        batch.max_qlen = max(batch.qlens)
-        batch.max_ctx = max(s + q for s, q in zip(batch.starts, batch.qlens))
-        batch.decode_only = batch.max_qlen == 1
 
     # ---------------------------------------------------------------------------------- graphs
     def _graph_eligible(self, items: list[StepItem]) -> bool:

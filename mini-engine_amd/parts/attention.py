@@ -37,7 +37,6 @@ class Attention(Mixer):
         self.position = None if s.position is None else POSITION_ENCODINGS.build(s.position, dtype, device)
         self.q_norm_w = self.k_norm_w = None
         self.w_qkv = self.w_o = None
-        self.binding: KVBinding | None = None
 
     # ---- weights
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
@@ -76,14 +75,11 @@ class Attention(Mixer):
     def cache_source(self):
         return self.spec.cache_from
 
-    def bind_cache(self, binding: KVBinding) -> None:
-        self.binding = binding
-
     # ---- step
-    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
-        s, b = self.spec, self.binding
+    def forward(self, h: torch.Tensor, batch, cache: KVBinding | None = None) -> torch.Tensor:
+        s, b = self.spec, cache
         if b is None:
-            raise RuntimeError("attention mixer has no cache bound")
+            raise RuntimeError("attention mixer was given no cache")
         owns = s.cache_from is None
         proj = K.linear(h, self.w_qkv)  # [T, (nh + 2 nkv) d] or [T, nh d]
         table = batch.block_table(b.group)
@@ -92,14 +88,14 @@ class Attention(Mixer):
         q = K.qk_norm_rope_scatter(
             proj, self.q_norm_w, self.k_norm_w if owns else None, inv_freq, batch.positions, batch.token_item,
             table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns)
-        out = self.attend(q, batch, table)
+        out = self.attend(q, batch, table, b)
         return K.linear(out, self.w_o)
 
-    def attend(self, q: torch.Tensor, batch, table: torch.Tensor) -> torch.Tensor:
+    def attend(self, q: torch.Tensor, batch, table: torch.Tensor, b: KVBinding) -> torch.Tensor:
         """bfloat16 with sizes the matrix-core kernels take: the split-context kernel when every item
         brings one token, else the tiled prefill kernel. Everything else (float32, other head or page
         sizes): the general kernel."""
-        b, s = self.binding, self.spec
+        s = self.spec
         scale, window = float(s.scale), int(s.window)
         if self.dtype is torch.bfloat16 and K.attention_mfma_supported(self.d, b.block_size, self.nh // self.nkv):
             if batch.decode_only:

@@ -8,12 +8,14 @@ it is in. The four interfaces:
                        fused residual-add-and-norm of the block.
 ``PositionEncoding``   ``tables(device)`` returns what the mixer's kernel needs (for rotary: inv_freq).
 ``Mixer``              ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``cache_need()``,
-                       ``bind_cache(binding)``, ``forward(h, batch) -> [T, hidden]``.
+                       ``forward(h, batch, cache) -> [T, hidden]``.
 ``FeedForward``        ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``forward(h, batch) -> [T, hidden]``.
 
 ``h`` is the normed input [T, hidden] in the compute dtype, ``batch`` a ``StepBatch`` (token
-positions, item boundaries, block tables per cache group, state slots). A mixer states what it
-needs kept between steps through ``cache_need()``:
+positions, item boundaries, block tables per cache group, state slots), ``cache`` the binding
+(``KVBinding`` / ``StateBinding`` / None) of this run of the layer: a layer that the order names
+twice has a cache for each run. A mixer states what it needs kept between steps through
+``cache_need()``:
 
 * ``KVCacheNeed``: paged keys and values (heads, head size, window; 0 = all keys);
 * ``StateNeed``: a fixed-size tensor per live request (a slot);
@@ -89,10 +91,7 @@ class Mixer(Part):
         """Index of another layer whose cache this mixer reads instead of owning one."""
         return None
 
-    def bind_cache(self, binding: Any) -> None:
-        pass
-
-    def forward(self, h: torch.Tensor, batch: Any) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch: Any, cache: Any = None) -> torch.Tensor:
         raise NotImplementedError
 
 

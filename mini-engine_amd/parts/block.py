@@ -41,11 +41,12 @@ class PreNormBlock:
         self.ffn_norm.load(tensors, s.ffn_norm_name)
         self.ffn.load(tensors, s.ffn_prefix)
 
-    def forward(self, x: torch.Tensor, pending: torch.Tensor | None, batch) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, pending: torch.Tensor | None, batch, cache=None) -> torch.Tensor:
         """``x`` float32 [T, H] residual stream (updated in place); ``pending`` is the previous
-        block's output that still has to be added. Returns this block's own pending output."""
+        block's output that still has to be added; ``cache`` is the binding of this run of the
+        layer. Returns this block's own pending output."""
         h = K.add_rmsnorm(x, pending, self.mixer_norm.weight, self.mixer_norm.eps, self.dtype)
-        a = self.mixer.forward(h, batch)
+        a = self.mixer.forward(h, batch, cache)
         h = K.add_rmsnorm(x, a, self.ffn_norm.weight, self.ffn_norm.eps, self.dtype)
         return self.ffn.forward(h, batch)
 

@@ -24,10 +24,20 @@ class Decoder:
         self.final_norm = NORMS.build(plan.final_norm, dtype, self.device)
         self.embed_table: torch.Tensor | None = None
         self.head: torch.Tensor | None = None
-        for i, blk in enumerate(self.blocks):
-            src = blk.mixer.cache_source()
-            if src is not None and not (0 <= src < len(self.blocks) and self.blocks[src].mixer.cache_source() is None):
-                raise ValueError(f"layer {i} reads the cache of layer {src}, which owns none")
+        # One cache per run (position in plan.order), not per layer: a layer named twice keeps the
+        # keys of each run apart. cache_owner[r] is the run whose cache run r uses: itself, or the
+        # latest earlier run of the layer its mixer names as its cache source.
+        self.cache_owner: list[int] = []
+        for r, i in enumerate(plan.order):
+            src = self.blocks[i].mixer.cache_source()
+            if src is None:
+                self.cache_owner.append(r)
+                continue
+            earlier = [q for q in range(r) if plan.order[q] == src and self.blocks[src].mixer.cache_source() is None]
+            if not earlier:
+                raise ValueError(f"layer {i} reads the cache of layer {src}, which has not run before it or owns none")
+            self.cache_owner.append(earlier[-1])
+        self.bindings: list = [None] * len(plan.order)  # filled by the cache storage
 
     # ---- weights
     def weight_wants(self) -> dict[str, TensorWant]:
@@ -77,8 +87,8 @@ class Decoder:
             raise RuntimeError("weights are not loaded")
         x = K.embed(batch.token_ids, self.embed_table)
         pending = None
-        for i in self.plan.order:
-            pending = self.blocks[i].forward(x, pending, batch)
+        for r, i in enumerate(self.plan.order):
+            pending = self.blocks[i].forward(x, pending, batch, self.bindings[r])
         return self.logits(x, pending, batch.want_rows)
 
     def logits(self, x: torch.Tensor, pending: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:

@@ -1,0 +1,266 @@
+"""Generation through the entry point (LLMEngine.generate) against the plain implementation: each
+request alone, batched, with prefix-cache hits, under preemption, with a 7-token budget, with EOS,
+long decoding through replayed graphs, temperature sampling, and the command line. The shapes of
+these tests follow the reference's tests/test_parity.py (cited per test)."""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from conftest import BLOCK_SIZES, ROOT, random_prompt, tiny_configs, write_tiny
+
+pytestmark = pytest.mark.gpu
+
+MAX_NEW = 16
+
+
+@pytest.fixture(scope="module")
+def peaked(tmp_path_factory):
+    """Both tiny configurations with a wide init (std 0.2), so that logits are peaked and float32
+    rounding cannot flip an argmax (the reference's precaution, tests/conftest.py:25-27)."""
+    out = {}
+    for name, cfg in tiny_configs().items():
+        folder = write_tiny(str(tmp_path_factory.mktemp(f"peaked_{name}")), cfg, seed=3, std=0.2, dtype=torch.float32)
+        out[name] = (folder, plain.read_config(folder), plain.read_weights(folder))
+    return out
+
+
+def prompts_for(name: str, n: int = 8, lo: int = 1, hi: int = 45, seed: int = 1) -> list[list[int]]:
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(lo, hi + 1, (n,), generator=g).tolist()
+    vocab = tiny_configs()[name].vocab_size
+    return [torch.randint(1, vocab, (k,), generator=g).tolist() for k in lens]
+
+
+def engine(folder, name, **over):
+    from mini_engine_amd import EngineConfig, LLMEngine
+
+    cfg = {"block_size": 4 if name == "A" else 8, "num_blocks": 256, "dtype": "float32", **over}
+    return LLMEngine.from_pretrained(folder, EngineConfig(**cfg))
+
+
+_reference = {}
+
+
+def reference(peaked, name):
+    if name not in _reference:
+        folder, pcfg, w = peaked[name]
+        _reference[name] = [plain.greedy_generate(w, pcfg, p, MAX_NEW) for p in prompts_for(name)]
+    return _reference[name]
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_unbatched_and_batched(peaked, name):  # test_parity.py:80-89
+    from mini_engine_amd import SamplingParams
+
+    want = reference(peaked, name)
+    eng = engine(peaked[name][0], name, enable_prefix_caching=False)
+    assert [eng.generate([p], SamplingParams(max_tokens=MAX_NEW))[0] for p in prompts_for(name)] == want
+    eng = engine(peaked[name][0], name)
+    assert eng.generate(prompts_for(name), SamplingParams(max_tokens=MAX_NEW)) == want
+    assert max(eng.stats.step_batch_sizes) == 8
+    assert eng.stats.generated_tokens == 8 * MAX_NEW and eng.runner.graph_replays > 0
+    assert all(rc == 0 for rc in eng.block_manager.ref_counts)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_prefix_cache_hits_keep_parity(peaked, name):  # test_parity.py:92-104
+    from mini_engine_amd import SamplingParams
+
+    folder, pcfg, w = peaked[name]
+    bs = 4 if name == "A" else 8
+    system = prompts_for(name, 1, 23, 23, seed=7)[0]
+    tails = prompts_for(name, 5, 1, 12, seed=8)
+    prompts = [system + t for t in tails] + [system]
+    want = [plain.greedy_generate(w, pcfg, p, MAX_NEW) for p in prompts]
+    eng = engine(folder, name)
+    first = eng.generate(prompts[:1], SamplingParams(max_tokens=MAX_NEW))
+    rest = eng.generate(prompts[1:], SamplingParams(max_tokens=MAX_NEW))
+    assert first + rest == want
+    # every later prompt reuses the full blocks of the shared prefix; the bare system prompt too,
+    # because its last token is the one that is recomputed
+    assert eng.scheduler.num_cached_tokens == 5 * bs * ((23 - 1) // bs)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_preemption_keeps_parity(peaked, name):  # test_parity.py:107-112
+    from mini_engine_amd import SamplingParams
+
+    eng = engine(peaked[name][0], name, num_blocks=20 if name == "A" else 12)
+    assert eng.generate(prompts_for(name), SamplingParams(max_tokens=MAX_NEW)) == reference(peaked, name)
+    assert eng.scheduler.num_preemptions > 0
+    assert all(rc == 0 for rc in eng.block_manager.ref_counts)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_chunked_prefill_keeps_parity(peaked, name):  # test_parity.py:115-119
+    from mini_engine_amd import SamplingParams
+
+    eng = engine(peaked[name][0], name, max_num_batched_tokens=7)
+    assert eng.generate(prompts_for(name), SamplingParams(max_tokens=MAX_NEW)) == reference(peaked, name)
+    assert eng.stats.steps > 30
+
+
+def test_engine_stops_at_eos(peaked):  # test_parity.py:122-129
+    from mini_engine_amd import SamplingParams
+
+    name = "A"
+    want = reference(peaked, name)
+    eos = want[0][3]
+    eng = engine(peaked[name][0], name, num_blocks=64)
+    eng.scheduler.eos_token_ids = {eos}
+    out = eng.generate([prompts_for(name)[0]], SamplingParams(max_tokens=MAX_NEW))[0]
+    assert out == want[0][: want[0].index(eos) + 1]
+    out = eng.generate([prompts_for(name)[0]], SamplingParams(max_tokens=MAX_NEW, ignore_eos=True))[0]
+    assert out == want[0]
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_long_decoding(peaked, graphs):
+    """300 tokens from a short prompt: many pages, several 64-key tiles, every step a replay."""
+    from mini_engine_amd import SamplingParams
+
+    name = "B"
+    folder, pcfg, w = peaked[name]
+    prompt = prompts_for(name)[2][:5]
+    want = plain.greedy_generate(w, pcfg, prompt, 300)
+    eng = engine(folder, name, cuda_graphs=graphs, max_model_len=512)
+    got = eng.generate([prompt], SamplingParams(max_tokens=300))[0]
+    assert got == want
+    assert (eng.runner.graph_replays > 250) == graphs
+
+
+def test_bfloat16_generation_stays_close(peaked):
+    """bfloat16 cannot promise equal tokens (near-ties flip, reference DECISIONS.md:80-82): the first
+    tokens agree, and each engine token is one the plain logits rank near the top."""
+    from mini_engine_amd import SamplingParams
+
+    for name in ("A", "B"):
+        folder, pcfg, w = peaked[name]
+        eng = engine(folder, name, dtype="bfloat16", block_size=16)
+        prompts = prompts_for(name)
+        got = eng.generate(prompts, SamplingParams(max_tokens=MAX_NEW))
+        want = reference(peaked, name)
+        assert sum(g[0] == e[0] for g, e in zip(got, want)) >= 7
+        for p, g in zip(prompts, got):
+            logits = plain.forward_logits(w, pcfg, p + g)[len(p) - 1 : -1]
+            chosen = logits.gather(1, torch.tensor(g)[:, None])[:, 0]
+            assert ((logits.max(-1).values - chosen) < 0.05 * logits.abs().max()).all()
+
+
+def test_tiny_b_workload_with_temperature_and_shared_prefix(peaked):
+    """Prompt lengths 1/9/16/31/50, two sharing a 16-token prefix (staged so that the second hits
+    it), 12 tokens at temperature 0.8 from a fixed seed. A request's samples are keyed on (seed,
+    request, token index), so the same tokens come out alone, batched, chunked and preempted."""
+    from mini_engine_amd import EngineConfig, LLMEngine, SamplingParams
+    from mini_engine_amd.engine.sequence import Sequence
+
+    name = "B"
+    folder, pcfg, w = peaked[name]
+    vocab = tiny_configs()[name].vocab_size
+    shared = random_prompt(16, vocab, 50)
+    prompts = [random_prompt(1, vocab, 51), random_prompt(9, vocab, 52), shared,
+               shared + random_prompt(15, vocab, 53), random_prompt(50, vocab, 54)]
+    params = SamplingParams(max_tokens=12, temperature=0.8)
+
+    def run(stage, **over):
+        import mini_engine_amd.engine.sequence as seqmod
+        import itertools
+
+        seqmod._seq_counter = itertools.count(1000)  # the same request ids in every run
+        eng = LLMEngine.from_pretrained(folder, EngineConfig(**{"block_size": 8, "dtype": "float32", "seed": 5, **over}))
+        outs = []
+        for group in stage:
+            outs += eng.generate([prompts[i] for i in group], params)
+        return eng, [outs[sum(stage, []).index(i)] for i in range(5)]
+
+    eng, base = run([[0, 1, 2], [3, 4]], num_blocks=64)
+    assert all(len(o) == 12 for o in base)  # a sampled request yields exactly max_tokens tokens
+    assert eng.scheduler.num_cached_tokens == 16  # request 3 hit the two full pages of request 2
+    assert base != [plain.greedy_generate(w, pcfg, p, 12) for p in prompts]  # it does sample
+    for p, o in zip(prompts, base):  # every sampled token is plausible under the plain distribution
+        probs = plain.temperature_probs(plain.forward_logits(w, pcfg, p + o)[len(p) - 1 : -1], 0.8)
+        assert (probs.gather(1, torch.tensor(o)[:, None]) > 1e-4).all()
+    _, again = run([[0, 1, 2], [3, 4]], num_blocks=64)
+    assert again == base  # fixed seed: repeatable
+    _, chunked = run([[0, 1, 2], [3, 4]], num_blocks=64, max_num_batched_tokens=7)
+    assert chunked == base
+    eng, squeezed = run([[0, 1, 2], [3, 4]], num_blocks=11, max_num_batched_tokens=24)
+    assert squeezed == base and eng.scheduler.num_preemptions > 0
+    _, other_seed = run([[0, 1, 2], [3, 4]], num_blocks=64, seed=6)
+    assert other_seed != base
+    greedy = LLMEngine.from_pretrained(folder, EngineConfig(block_size=8, dtype="float32", num_blocks=64))
+    assert greedy.generate(prompts, SamplingParams(max_tokens=12)) == [plain.greedy_generate(w, pcfg, p, 12) for p in prompts]
+
+
+def test_tiny_a_workload(peaked):
+    """Prompts 5/17/33, 8 greedy tokens; whole, token by token, in 7-token portions, mixed."""
+    from mini_engine_amd import SamplingParams
+
+    name = "A"
+    folder, pcfg, w = peaked[name]
+    vocab = tiny_configs()[name].vocab_size
+    prompts = [random_prompt(n, vocab, 60 + n) for n in (5, 17, 33)]
+    want = [plain.greedy_generate(w, pcfg, p, 8) for p in prompts]
+    for over in ({}, {"max_num_batched_tokens": 1}, {"max_num_batched_tokens": 7}, {"max_num_seqs": 2}):
+        eng = engine(folder, name, block_size=16, **over)
+        assert eng.generate(prompts, SamplingParams(max_tokens=8)) == want, over
+
+
+def test_requests_that_cannot_fit_are_refused(peaked):
+    from mini_engine_amd import SamplingParams
+
+    eng = engine(peaked["A"][0], "A", num_blocks=4, max_model_len=64)
+    with pytest.raises(ValueError, match="KV blocks"):
+        eng.add_request([1] * 14, SamplingParams(max_tokens=8))
+    with pytest.raises(ValueError, match="max_model_len"):
+        eng.add_request([1] * 60, SamplingParams(max_tokens=8))
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([1, 100000], SamplingParams(max_tokens=2))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    """No fallback: when the kernels can be neither found nor built, the first op raises."""
+    import mini_engine_amd.ops.library as library
+
+    monkeypatch.setattr(library, "_lib", None)
+
+    def broken():
+        class M:
+            LIB_NAME = "x.so"
+
+            @staticmethod
+            def default_lib_path():
+                return "/nonexistent/libmini_engine_hip.so"
+
+            @staticmethod
+            def is_current(p):
+                return False
+
+            @staticmethod
+            def build():
+                raise RuntimeError("hipcc not found: the HIP kernels cannot be compiled")
+
+        return M
+
+    monkeypatch.setattr(library, "_build_module", broken)
+    with pytest.raises(RuntimeError, match="cannot be compiled"):
+        library.lib()
+
+
+def test_command_line(peaked):
+    folder = peaked["A"][0]
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "examples", "generate.py"), "--model", folder,
+                           "--max-tokens", "6", "--dtype", "float32", "--prompt-ids", "5,6,7,8,9", "--prompt-ids", "5,6,7,8,9,10,11"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    _, pcfg, w = peaked["A"]
+    lines = [l for l in proc.stdout.splitlines() if l.startswith("A: ")]
+    assert lines[0] == "A: " + " ".join(map(str, plain.greedy_generate(w, pcfg, [5, 6, 7, 8, 9], 6)))
+    assert "tokens in" in proc.stdout and "served from prefix cache" in proc.stdout

@@ -1,0 +1,193 @@
+"""A toy mixer with state of its own, defined here, is registered, built into a model and stepped
+without a change to the framework's files. It keeps, per request, the running sum of its inputs
+(a fixed-size state in a slot) and returns the running mean through a projection:
+
+    s_t = s_{t-1} + h_t;   y_t = W (s_t / (t + 1))
+
+The state must be carried from portion to portion, start from zero for a new request in a used slot,
+and not leak between requests that share a batch. A toy feed-forward with routing (two experts, top-1
+by a float32 router) and a toy position encoding (none; the mixer is order-aware by itself) show the
+other registries. None of this is a model of anyone's."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@dataclass(frozen=True)
+class RunningMeanSpec:
+    hidden_size: int
+    kind: str = "toy_running_mean"
+
+
+@dataclass(frozen=True)
+class Top1ExpertsSpec:
+    hidden_size: int
+    num_experts: int
+    kind: str = "toy_top1_experts"
+
+
+def register_toys():
+    from mini_engine_amd.parts import FEED_FORWARDS, MIXERS, FeedForward, Mixer, StateNeed
+    from mini_engine_amd.weights import TensorWant
+
+    class RunningMean(Mixer):
+        def weight_wants(self, prefix):
+            h = self.spec.hidden_size
+            return {f"{prefix}.out.weight": TensorWant((h, h))}
+
+        def load(self, tensors, prefix):
+            self.w = tensors[f"{prefix}.out.weight"]
+
+        def cache_need(self):
+            return StateNeed((self.spec.hidden_size,), torch.float32)
+
+        def forward(self, h, batch, cache=None):
+            out = torch.empty_like(h)
+            cursor = 0
+            for start, n, slot in zip(batch.starts, batch.qlens, batch.slots_host):
+                seg = h[cursor : cursor + n].float()
+                running = cache.state[slot] + seg.cumsum(0)
+                counts = torch.arange(start + 1, start + n + 1, device=h.device, dtype=torch.float32)[:, None]
+                out[cursor : cursor + n] = ((running / counts) @ self.w.float().T).to(h.dtype)
+                cache.state[slot] = running[-1]
+                cursor += n
+            return out
+
+    class Top1Experts(FeedForward):
+        def weight_wants(self, prefix):
+            h, e = self.spec.hidden_size, self.spec.num_experts
+            wants = {f"{prefix}.router.weight": TensorWant((e, h), "vector")}  # kept in float32
+            for i in range(e):
+                wants[f"{prefix}.experts.{i}.weight"] = TensorWant((h, h))
+            return wants
+
+        def load(self, tensors, prefix):
+            self.router = tensors[f"{prefix}.router.weight"]
+            self.experts = [tensors[f"{prefix}.experts.{i}.weight"] for i in range(self.spec.num_experts)]
+
+        def forward(self, h, batch=None):
+            choice = (h.float() @ self.router.T).argmax(-1)  # router logits in float32
+            out = torch.zeros_like(h)
+            for i, w in enumerate(self.experts):
+                rows = (choice == i).nonzero()[:, 0]
+                if rows.numel():
+                    out[rows] = (h[rows].float() @ w.float().T).to(h.dtype)
+            return out
+
+    MIXERS.register("toy_running_mean", RunningMean)
+    FEED_FORWARDS.register("toy_top1_experts", Top1Experts)
+
+
+def toy_plan():
+    """Layer 0: the toy mixer + routed toy feed-forward. Layer 1: attention + dense gated MLP."""
+    from mini_engine_amd.config import AttentionSpec, GatedMlpSpec, LayerSpec, ModelPlan, NormSpec, RotarySpec
+
+    h = 48
+    norm = NormSpec(dim=h, eps=1e-5)
+    layers = (
+        LayerSpec(mixer=RunningMeanSpec(h), ffn=Top1ExpertsSpec(h, 2), mixer_norm=norm, ffn_norm=norm,
+                  mixer_prefix="toy.0.mix", ffn_prefix="toy.0.moe", mixer_norm_name="toy.0.n1", ffn_norm_name="toy.0.n2"),
+        LayerSpec(mixer=AttentionSpec(hidden_size=h, num_heads=3, num_kv_heads=1, head_dim=16, scale=0.25,
+                                      qk_norm_eps=None, position=RotarySpec(16, 1e4)),
+                  ffn=GatedMlpSpec(hidden_size=h, intermediate_size=80), mixer_norm=norm, ffn_norm=norm,
+                  mixer_prefix="toy.1.attn", ffn_prefix="toy.1.mlp", mixer_norm_name="toy.1.n1", ffn_norm_name="toy.1.n2"),
+    )
+    return ModelPlan(architecture="ToyForTests", vocab_size=97, hidden_size=h, layers=layers, order=(0, 1),
+                     final_norm=norm, embed_name="toy.embed", final_norm_name="toy.norm", head_name="toy.head",
+                     tie_word_embeddings=False, max_position_embeddings=256)
+
+
+def plain_toy(w, tokens):
+    import plain_qwen3 as plain
+
+    x = w["toy.embed"][torch.tensor(tokens)]
+    t = len(tokens)
+    h = plain.rms_norm(x, w["toy.0.n1"], 1e-5)
+    x = x + (h.cumsum(0) / torch.arange(1, t + 1)[:, None]) @ w["toy.0.mix.out.weight"].T
+    h = plain.rms_norm(x, w["toy.0.n2"], 1e-5)
+    choice = (h @ w["toy.0.moe.router.weight"].T).argmax(-1)
+    moe = torch.stack([h[i] @ w[f"toy.0.moe.experts.{int(choice[i])}.weight"].T for i in range(t)])
+    x = x + moe
+    h = plain.rms_norm(x, w["toy.1.n1"], 1e-5)
+    q = (h @ w["toy.1.attn.q_proj.weight"].T).view(t, 3, 16)
+    k = (h @ w["toy.1.attn.k_proj.weight"].T).view(t, 1, 16)
+    v = (h @ w["toy.1.attn.v_proj.weight"].T).view(t, 1, 16)
+    cos, sin = plain.rope_tables(torch.arange(t), 16, 1e4)
+    a = plain.grouped_causal_attention(plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin), v, 0.25)
+    x = x + a.reshape(t, -1) @ w["toy.1.attn.o_proj.weight"].T
+    h = plain.rms_norm(x, w["toy.1.n2"], 1e-5)
+    x = x + plain.swiglu_mlp(h, w, "toy.1.mlp")
+    return plain.rms_norm(x, w["toy.norm"], 1e-5) @ w["toy.head"].T
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped():
+    from mini_engine_amd import EngineConfig
+    from mini_engine_amd.engine.batch import StepItem
+    from mini_engine_amd.engine.runner import ModelRunner
+    from mini_engine_amd.engine.sequence import Sequence
+    from mini_engine_amd.parts import Decoder
+    from mini_engine_amd.weights import RandomSource
+
+    register_toys()
+    plan = toy_plan()
+    dec = Decoder(plan, torch.float32, "cuda")
+    wants = dec.weight_wants()
+    assert "toy.0.mix.out.weight" in wants and "toy.0.moe.experts.1.weight" in wants
+    src = RandomSource(wants, seed=2, std=0.2, norm_std=0.1, device="cpu")
+    weights = {n: src.get(n) for n in wants}
+    weights["toy.0.moe.router.weight"] = torch.randn(2, 48, generator=torch.Generator().manual_seed(8))
+
+    class Source:
+        def shapes(self):
+            return {n: tuple(t.shape) for n, t in weights.items()}
+
+        def get(self, n):
+            return weights[n]
+
+    dec.load(Source())
+    runner = ModelRunner(dec, EngineConfig(block_size=8, num_blocks=32, max_num_seqs=2, dtype="float32",
+                                           max_model_len=128))
+    assert runner.layout.has_state and list(runner.layout.state_layers) == [0]
+    bm = runner.new_block_manager()
+    assert not bm.enable_prefix_caching  # state cannot be rebuilt from shared pages
+
+    g = torch.Generator().manual_seed(1)
+    reqs = {k: torch.randint(0, 97, (n,), generator=g).tolist() for k, n in (("a", 37), ("b", 21), ("c", 30))}
+    want = {k: plain_toy(weights, v) for k, v in reqs.items()}
+    assert len({int(c) for c in (want["a"].argmax(-1))}) > 1
+
+    def feed(schedule):
+        """schedule: list of steps, each a list of (request, number of tokens)."""
+        seqs, got = {}, {k: [] for k in reqs}
+        for step in schedule:
+            items = []
+            for k, n in step:
+                seq = seqs.setdefault(k, Sequence(reqs[k]))
+                lo = seq.num_computed_tokens
+                assert bm.try_allocate(seq, lo + n)
+                items.append((k, StepItem(seq, reqs[k][lo : lo + n], lo, list(range(n)))))
+            out = runner.step([it for _, it in items]).cpu()
+            r = 0
+            for k, it in items:
+                got[k].append(out[r : r + len(it.tokens)].clone())
+                r += len(it.tokens)
+                seqs[k].num_computed_tokens += len(it.tokens)
+                if seqs[k].num_computed_tokens == len(reqs[k]):
+                    bm.free(seqs.pop(k))
+        return {k: torch.cat(v) for k, v in got.items() if v}
+
+    # whole requests one after another: the second and third reuse a slot whose state is not zero
+    whole = feed([[("a", 37)], [("b", 21)], [("c", 30)]])
+    for k in reqs:
+        torch.testing.assert_close(whole[k], want[k], rtol=1e-4, atol=1e-4)
+    # portions and single tokens, two requests side by side, the third admitted when a slot frees
+    mixed = feed([[("a", 10), ("b", 1)], [("b", 19), ("a", 2)], [("a", 1)], [("a", 24), ("b", 1)], [("c", 29)], [("c", 1)]])
+    for k in reqs:
+        torch.testing.assert_close(mixed[k], want[k], rtol=1e-4, atol=1e-4)
+    assert bm.slots.in_use == set() and all(len(p.free_pool) == p.num_blocks for p in bm.pools)
