@@ -66,8 +66,9 @@ def build(out_dir: str | None = None, quiet: bool = False, jobs: int | None = No
     if not os.access(out_dir, os.W_OK):
         out_dir = os.path.join(tempfile.gettempdir(), f"mini_engine_hip_{os.getuid()}")
         os.makedirs(out_dir, exist_ok=True)
-    obj_dir = os.path.join(out_dir, "_build")
-    os.makedirs(obj_dir, exist_ok=True)
+    os.makedirs(os.path.join(out_dir, "_build"), exist_ok=True)
+    # objects of this build only: two processes that build at the same time do not share files
+    obj_dir = tempfile.mkdtemp(prefix="objs_", dir=os.path.join(out_dir, "_build"))
     srcs = sources()
     jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")), 16)
     env = dict(os.environ)
@@ -96,6 +97,7 @@ def build(out_dir: str | None = None, quiet: bool = False, jobs: int | None = No
     if r.returncode != 0:
         raise RuntimeError(f"linking {LIB_NAME} failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, lib)
+    shutil.rmtree(obj_dir, ignore_errors=True)
     _say(f"built {lib} in {time.time() - t0:.0f}s", quiet)
     return lib
 
