@@ -42,14 +42,24 @@ __device__ __forceinline__ short4_t pack_bf16x4(float a, float b, float c, float
   return r;
 }
 
-// max / sum over the four lanes that share a query column (l%16 fixed, l/16 = 0..3)
+// max / sum over the four lanes that share a query column (l%16 fixed, l/16 = 0..3). The row swaps
+// of gfx950 (v_permlane16_swap, v_permlane32_swap) hand every lane its partner's value at vector-ALU
+// speed: after a swap of a register with a copy of itself, the two results hold, in every lane, the
+// lane's own value and that of lane ^ 16 (resp. lane ^ 32), in one order or the other.
+typedef unsigned uint2v_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float column_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, ME_WAVE));
-  return fmaxf(v, __shfl_xor(v, 32, ME_WAVE));
+  unsigned u = __float_as_uint(v);
+  uint2v_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  u = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
 }
 __device__ __forceinline__ float column_sum(float v) {
-  v += __shfl_xor(v, 16, ME_WAVE);
-  return v + __shfl_xor(v, 32, ME_WAVE);
+  unsigned u = __float_as_uint(v);
+  uint2v_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  u = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+  a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(a[0]) + __uint_as_float(a[1]);
 }
 
 #define LOG2E 1.4426950408889634f
@@ -122,8 +132,9 @@ template <int D>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int bs, int window, float scale_log2,
-    int split_keys, int num_splits, int head_chunks) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int bs_shift, int window,
+    float scale_log2, int split_keys, int num_splits, int head_chunks) {
+  const int bs = 1 << bs_shift;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
   const int split = blockIdx.z;
@@ -152,9 +163,9 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const int qpos[1] = {ctx - 1};
     const int* table = block_table + (size_t)item * table_width;
     for (int key0 = begin; key0 < end; key0 += 16) {
-      int page = table[key0 / bs];
+      int page = table[key0 >> bs_shift];
       page = page < 0 ? 0 : page;
-      const int off = key0 % bs;
+      const int off = key0 & (bs - 1);
       const bf16_t* kbase = k_cache + (((size_t)page * nkv + kvh) * bs + off) * D;
       const bf16_t* vbase = v_cache + ((size_t)page * nkv + kvh) * D * bs + off;
       const bool need_mask = key0 < lo || key0 + 16 > ctx;
@@ -245,12 +256,16 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
                           float scale_log2, int split_keys, int num_splits, hipStream_t stream) {
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits);
-  attention_decode_kernel<D><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, nkv, bs,
-                                                      window, scale_log2, split_keys, num_splits, chunks);
+  int bs_shift = 0;
+  while ((1 << bs_shift) < bs) ++bs_shift;
+  attention_decode_kernel<D><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, nkv,
+                                                      bs_shift, window, scale_log2, split_keys, num_splits, chunks);
 }
 
+// Head sizes that are multiples of 32 (instantiated: 32, 64, 96, 128, 192, 256) and pages of a power
+// of two of at least 16 keys.
 extern "C" int me_attention_mfma_supported(int d, int bs) {
-  return (d == 32 || d == 64 || d == 96 || d == 128 || d == 192 || d == 256) && bs > 0 && bs % 16 == 0;
+  return (d == 32 || d == 64 || d == 96 || d == 128 || d == 192 || d == 256) && bs >= 16 && (bs & (bs - 1)) == 0;
 }
 
 // q [items, nh, d] (one token per item), item_ctx[i] = keys of item i including the new one,
@@ -297,106 +312,279 @@ extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, cons
 // Block = 4 waves; a block owns the query columns of `tokens_per_block = 128 / group` consecutive
 // new tokens of one item for one kv head (column c -> token c / group, head c % group); wave w owns
 // columns 32w .. 32w+31 as two blocks of 16. Blocks are numbered over all items: item i has
-// ceil(qlen_i / tokens_per_block) of them.
+// ceil(qlen_i / tokens_per_block) of them, the later (longer) tiles of an item first.
+//
+// Keys and values are staged through LDS in tiles of 64 keys, double-buffered: while the waves
+// multiply tile i out of one buffer, the global loads of tile i+1 are in flight and are written to
+// the other buffer afterwards; one barrier per tile. Products use v_mfma_f32_16x16x32_bf16 (the
+// full-rate bfloat16 instruction of gfx950; the 16x16x16 form runs at half its rate):
+//   S^T (16 keys x 16 columns) += K[16 keys, 32 d] . Q^T[32 d, 16 columns]
+//   O^T (16 d x 16 columns)   += V^T[16 d, 32 keys] . P^T[32 keys, 16 columns]
+// For the second product the 32 keys of a lane's B operand are the four keys it holds of each of two
+// 16-key score tiles (keys 4g..4g+3 and 16+4g..16+4g+3 of the 32); the A operand reads V^T in the
+// same order, so the contraction pairs up.
+//
+// LDS rows are padded (keys: +8 elements, values: +4) so that the 16-byte key reads and the 8-byte
+// value reads of a wave spread over all banks.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+
+#define PF_KT 64  // keys per LDS tile
+#define PF_PIECES(D, THREADS) ((8 * (D) + (THREADS) - 1) / (THREADS))  // 16-byte pieces of a tile per thread
+
 template <int D>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+struct PrefillLds {
+  static constexpr int KROW = D + 8;        // elements per key row
+  static constexpr int VROW = PF_KT + 4;    // elements per value row (one d, 64 keys)
+  static constexpr int K_ELEMS = PF_KT * KROW;
+  static constexpr int V_ELEMS = D * VROW;
+  static constexpr int BUF_ELEMS = K_ELEMS + V_ELEMS;
+  static constexpr int BYTES = 2 * BUF_ELEMS * 2;
+};
+
+// Global loads of one 64-key tile into registers: thread `tid` of THREADS fetches 8D/THREADS
+// 16-byte pieces of keys and as many of values. Keys: piece c -> row c / (D/8), 8 elements at column
+// (c % (D/8)) * 8. Values: piece c -> 16-key sub-tile c / (2D), then d = (c % 2D) / 2, half = c % 2,
+// which walks a transposed value page front to back. The page size is a power of two.
+template <int D, int THREADS>
+__device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)], uint4 (&vreg)[PF_PIECES(D, THREADS)], int key0,
+                                             int tid, const int* __restrict__ table, int table_width, int bs_shift,
+                                             int nkv, int kvh, const bf16_t* __restrict__ k_cache,
+                                             const bf16_t* __restrict__ v_cache) {
+  const int bs_mask = (1 << bs_shift) - 1;
+#pragma unroll
+  for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
+    const int c = tid + i * THREADS;
+    if ((8 * D) % THREADS != 0 && c >= 8 * D) break;  // only the last round can be partial
+    {
+      const int row = c / (D / 8), col = c % (D / 8);
+      const int key = key0 + row;
+      int page = table[min(key >> bs_shift, table_width - 1)];
+      page = page < 0 ? 0 : page;
+      kreg[i] = *reinterpret_cast<const uint4*>(k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + (key & bs_mask)) * D + col * 8);
+    }
+    {
+      const int sub = c / (2 * D), rem = c % (2 * D);
+      const int d = rem >> 1, half = rem & 1;
+      const int key = key0 + sub * 16 + half * 8;
+      int page = table[min(key >> bs_shift, table_width - 1)];
+      page = page < 0 ? 0 : page;
+      vreg[i] = *reinterpret_cast<const uint4*>(v_cache + ((((size_t)page * nkv + kvh) * D + d) << bs_shift) + (key & bs_mask));
+    }
+  }
+}
+
+template <int D, int THREADS>
+__device__ __forceinline__ void pf_store_tile(const uint4 (&kreg)[PF_PIECES(D, THREADS)], const uint4 (&vreg)[PF_PIECES(D, THREADS)],
+                                              bf16_t* ks, int tid) {
+  using L = PrefillLds<D>;
+  bf16_t* vs = ks + L::K_ELEMS;
+#pragma unroll
+  for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
+    const int c = tid + i * THREADS;
+    if ((8 * D) % THREADS != 0 && c >= 8 * D) break;
+    const int row = c / (D / 8), col = c % (D / 8);
+    *reinterpret_cast<uint4*>(ks + row * L::KROW + col * 8) = kreg[i];
+    const int sub = c / (2 * D), rem = c % (2 * D);
+    const int d = rem >> 1, half = rem & 1;
+    uint2* dst = reinterpret_cast<uint2*>(vs + d * L::VROW + sub * 16 + half * 8);
+    dst[0] = make_uint2(vreg[i].x, vreg[i].y);
+    dst[1] = make_uint2(vreg[i].z, vreg[i].w);
+  }
+}
+
+typedef unsigned uint4v_t __attribute__((ext_vector_type(4)));
+
+// 32 keys (two 16-key score tiles) against NB blocks of 16 query columns, out of one LDS buffer.
+// MASK is a compile-time switch: tiles that every column of the wave sees whole skip the compares.
+template <int D, int NB, bool MASK>
+__device__ __forceinline__ void pf_attend32(const bf16_t* __restrict__ ks, const bf16_t* __restrict__ vs, int kbase_row,
+                                            int key_base, int r, int g, const bf16x8_t (&qf)[NB][D / 32],
+                                            const int (&qpos)[NB], const int (&lo_col)[NB], float scale_log2,
+                                            float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16]) {
+  using L = PrefillLds<D>;
+  float4_t s0[NB], s1[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) s0[nb] = s1[nb] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < D / 32; ++c) {
+    const bf16x8_t k0 = *reinterpret_cast<const bf16x8_t*>(ks + (kbase_row + r) * L::KROW + c * 32 + g * 8);
+    const bf16x8_t k1 = *reinterpret_cast<const bf16x8_t*>(ks + (kbase_row + 16 + r) * L::KROW + c * 32 + g * 8);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      s0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[nb][c], s0[nb], 0, 0, 0);
+      s1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[nb][c], s1[nb], 0, 0, 0);
+    }
+  }
+  bf16x8_t pf[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    float sv[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sv[i] = s0[nb][i];
+      sv[4 + i] = s1[nb][i];
+    }
+    if (MASK) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int key = key_base + (i >> 2) * 16 + g * 4 + (i & 3);
+        if (key < lo_col[nb] || key > qpos[nb]) sv[i] = -INFINITY;
+      }
+    }
+    // statistics are kept in units of the raw score times scale*log2(e): one fused multiply-add per
+    // score feeds the exponential
+    float tmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+    tmax = column_max(tmax) * scale_log2;
+    const float m_new = fmaxf(m[nb], tmax);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // a column with no visible key so far
+    const float alpha = fast_exp2(m[nb] - m_ref);
+    float p[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(sv[i], scale_log2, -m_ref));
+    lsum[nb] = fmaf(lsum[nb], alpha, column_sum(((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))));
+    m[nb] = m_new;
+    // the running maximum rarely moves after the first tiles: skip the rescale of the accumulator
+    // when no column of the wave needs it
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) {
+        acc[nb][dt][0] *= alpha;
+        acc[nb][dt][1] *= alpha;
+        acc[nb][dt][2] *= alpha;
+        acc[nb][dt][3] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) pf[nb][i] = (__bf16)p[i];  // round to nearest even in hardware
+  }
+#pragma unroll
+  for (int dt = 0; dt < D / 16; ++dt) {
+    const bf16_t* vrow = vs + (dt * 16 + r) * L::VROW + kbase_row + g * 4;
+    const uint2 v0 = *reinterpret_cast<const uint2*>(vrow);
+    const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + 16);
+    const uint4v_t packed = {v0.x, v0.y, v1.x, v1.y};
+    const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, packed);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      acc[nb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[nb], acc[nb][dt], 0, 0, 0);
+  }
+}
+
+// WAVES waves per block, NB blocks of 16 query columns per wave: WAVES * NB * 16 = 128 columns.
+template <int D, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ item_start, int num_items,
-    const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int nh, int nkv, int bs,
+    const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
     int window, float scale_log2, int tokens_per_block) {
-  __shared__ int s_item, s_tile;
+  constexpr int THREADS = WAVES * 64;
+  static_assert(WAVES * NB * 16 == 128, "a block owns 128 query columns");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
+  using L = PrefillLds<D>;
+  __shared__ int s_item, s_tile, s_lo, s_hi;
   if (threadIdx.x == 0) {
-    int left = blockIdx.x, it = 0;
+    int left = blockIdx.x, it = 0, tiles = 0;
     for (; it < num_items; ++it) {
-      const int tiles = (item_start[it + 1] - item_start[it] + tokens_per_block - 1) / tokens_per_block;
+      tiles = (item_start[it + 1] - item_start[it] + tokens_per_block - 1) / tokens_per_block;
       if (left < tiles) break;
       left -= tiles;
     }
     s_item = it;
-    s_tile = left;
+    s_tile = tiles - 1 - left;  // long tiles first
+    if (it < num_items) {
+      const int tb = item_start[it] + s_tile * tokens_per_block;
+      const int te = min(item_start[it + 1], tb + tokens_per_block);
+      const int p_first = positions[tb], p_last = positions[te - 1];
+      s_lo = window > 0 ? max(p_first - window + 1, 0) : 0;
+      s_hi = p_last;
+    }
   }
   __syncthreads();
   const int item = s_item;
   if (item >= num_items) return;
   const int kvh = blockIdx.y;
   const int group = nh / nkv;
-  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int t_begin = item_start[item] + s_tile * tokens_per_block;
   const int t_end = min(item_start[item + 1], t_begin + tokens_per_block);
+  const int* table = block_table + (size_t)item * table_width;
 
-  // this lane's query column in each of the wave's two blocks
-  int tok[2], head[2], qpos[2];
-  bool col_ok[2];
+  // this lane's query column in each of the wave's blocks
+  int tok[NB], head[NB], qpos[NB], lo_col[NB];
+  bool col_ok[NB];
   int wave_max_pos = -1, wave_min_pos = 0x7fffffff;
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const int c = wave * 32 + nb * 16 + r;
+  for (int nb = 0; nb < NB; ++nb) {
+    const int c = (wave * NB + nb) * 16 + r;
     tok[nb] = t_begin + c / group;
     head[nb] = kvh * group + c % group;
     col_ok[nb] = c < tokens_per_block * group && tok[nb] < t_end;
     qpos[nb] = col_ok[nb] ? positions[tok[nb]] : -1;
+    lo_col[nb] = window > 0 ? max(qpos[nb] - window + 1, 0) : 0;
+    wave_max_pos = max(wave_max_pos, qpos[nb]);
+    if (col_ok[nb]) wave_min_pos = min(wave_min_pos, qpos[nb]);
   }
-  {
-    int mx = max(qpos[0], qpos[1]);
-    int mn = min(col_ok[0] ? qpos[0] : 0x7fffffff, col_ok[1] ? qpos[1] : 0x7fffffff);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      mx = max(mx, __shfl_xor(mx, off, ME_WAVE));
-      mn = min(mn, __shfl_xor(mn, off, ME_WAVE));
-    }
-    wave_max_pos = mx;
-    wave_min_pos = mn;
+  for (int off = 32; off > 0; off >>= 1) {
+    wave_max_pos = max(wave_max_pos, __shfl_xor(wave_max_pos, off, ME_WAVE));
+    wave_min_pos = min(wave_min_pos, __shfl_xor(wave_min_pos, off, ME_WAVE));
   }
-  if (wave_max_pos < 0) return;  // no column of this wave is in use
 
-  Frag8 qf[2][D / 32];
+  bf16x8_t qf[NB][D / 32];
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb)
+  for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) {
-      qf[nb][c].u = make_uint4(0, 0, 0, 0);
+      qf[nb][c] = bf16x8_t{};
       if (col_ok[nb])
-        qf[nb][c].u = *reinterpret_cast<const uint4*>(q + ((size_t)tok[nb] * nh + head[nb]) * D + c * 32 + g * 8);
+        qf[nb][c] = *reinterpret_cast<const bf16x8_t*>(q + ((size_t)tok[nb] * nh + head[nb]) * D + c * 32 + g * 8);
     }
-  float m[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
-  float4_t acc[2][D / 16];
+  float m[NB], lsum[NB];
+  float4_t acc[NB][D / 16];
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb)
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = -INFINITY;
+    lsum[nb] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < D / 16; ++dt) acc[nb][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  }
 
-  // every column of the wave sees keys from its own lo; the lowest one bounds the loop
-  const int lo_min = window > 0 ? max(wave_min_pos - window + 1, 0) : 0;
-  const int* table = block_table + (size_t)item * table_width;
-  // the four values a lane holds belong to one column, so the window's lower bound is per lane too
-  int lo_col[2];
+  // ---- global -> register -> LDS staging of one 64-key tile (pf_load_tile / pf_store_tile)
+  uint4 kreg[PF_PIECES(D, THREADS)], vreg[PF_PIECES(D, THREADS)];
+  const int first_tile = (s_lo / PF_KT) * PF_KT;
+  const int last_key = s_hi;
+  pf_load_tile<D, THREADS>(kreg, vreg, first_tile, tid, table, table_width, bs_shift, nkv, kvh, k_cache, v_cache);
+  pf_store_tile<D, THREADS>(kreg, vreg, lds, tid);
+  __syncthreads();
+  int buf = 0;
+  for (int key0 = first_tile; key0 <= last_key; key0 += PF_KT, buf ^= 1) {
+    // the next tile is fetched unconditionally (the page index is clamped to the table, so a tile
+    // past the last key reads valid memory that nobody uses): no control flow around the registers
+    pf_load_tile<D, THREADS>(kreg, vreg, key0 + PF_KT, tid, table, table_width, bs_shift, nkv, kvh, k_cache, v_cache);
+    if (key0 <= wave_max_pos) {
+      const bf16_t* ks = lds + (size_t)buf * L::BUF_ELEMS;
+      const bf16_t* vs = ks + L::K_ELEMS;
+      const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || window > 0;
+      if (need_mask) {
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) lo_col[nb] = window > 0 ? max(qpos[nb] - window + 1, 0) : 0;
-
-  for (int key0 = (lo_min / 16) * 16; key0 <= wave_max_pos; key0 += 16) {
-    int page = table[key0 / bs];
-    page = page < 0 ? 0 : page;
-    const int off = key0 % bs;
-    const bf16_t* kbase = k_cache + (((size_t)page * nkv + kvh) * bs + off) * D;
-    const bf16_t* vbase = v_cache + ((size_t)page * nkv + kvh) * D * bs + off;
-    const bool need_mask = key0 + 15 > wave_min_pos || window > 0;
-    if (window > 0) {
-      // per-column lower bounds differ: mask with the larger of the two inside attend_tile by
-      // passing lo = 0 and folding the bound into qpos is not possible, so do the tile per block
-      const int q0[1] = {qpos[0]}, q1[1] = {qpos[1]};
-      attend_tile<D, 1>(kbase, vbase, bs, key0, lo_col[0], q0, true, reinterpret_cast<const Frag8(&)[1][D / 32]>(qf[0]),
-                        scale_log2, reinterpret_cast<float(&)[1]>(m[0]), reinterpret_cast<float(&)[1]>(lsum[0]),
-                        reinterpret_cast<float4_t(&)[1][D / 16]>(acc[0]));
-      attend_tile<D, 1>(kbase, vbase, bs, key0, lo_col[1], q1, true, reinterpret_cast<const Frag8(&)[1][D / 32]>(qf[1]),
-                        scale_log2, reinterpret_cast<float(&)[1]>(m[1]), reinterpret_cast<float(&)[1]>(lsum[1]),
-                        reinterpret_cast<float4_t(&)[1][D / 16]>(acc[1]));
-    } else {
-      attend_tile<D, 2>(kbase, vbase, bs, key0, 0, qpos, need_mask, qf, scale_log2, m, lsum, acc);
+        for (int kg = 0; kg < PF_KT / 32; ++kg)
+          if (key0 + kg * 32 <= wave_max_pos)
+            pf_attend32<D, NB, true>(ks, vs, kg * 32, key0 + kg * 32, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
+      } else {
+#pragma unroll
+        for (int kg = 0; kg < PF_KT / 32; ++kg)
+          pf_attend32<D, NB, false>(ks, vs, kg * 32, key0 + kg * 32, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
+      }
     }
+    pf_store_tile<D, THREADS>(kreg, vreg, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, tid);
+    __syncthreads();
   }
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
+  for (int nb = 0; nb < NB; ++nb) {
     if (!col_ok[nb]) continue;
     const float inv = 1.f / lsum[nb];
     bf16_t* orow = out + ((size_t)tok[nb] * nh + head[nb]) * D;
@@ -407,6 +595,26 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       *reinterpret_cast<short4_t*>(orow + dt * 16 + g * 4) = o;
     }
   }
+}
+
+#define PF_NB 1
+#define PF_WAVES 8
+
+template <int D>
+static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* positions,
+                          const int* item_start, int num_items, const int* table, int width, bf16_t* out, int nh,
+                          int nkv, int bs_shift, int window, float sl, int tpb, hipStream_t stream) {
+  static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, PF_NB, PF_WAVES>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, PrefillLds<D>::BYTES);
+    if (e != hipSuccess) return me_fail("me_attention_prefill_bf16: cannot reserve %d bytes of LDS: %s",
+                                        PrefillLds<D>::BYTES, hipGetErrorString(e));
+    configured = true;
+  }
+  attention_prefill_kernel<D, PF_NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
+      q, kc, vc, positions, item_start, num_items, table, width, out, nh, nkv, bs_shift, window, sl, tpb);
+  return 0;
 }
 
 // q [T, nh, d]; item_start int [items + 1] (offsets of the items' tokens); positions int [T];
@@ -422,14 +630,18 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   const int group = nh / nkv;
   if (group > 16) return me_fail("me_attention_prefill_bf16: group size %d exceeds 16", group);
   if (nkv > 65535) return me_fail("me_attention_prefill_bf16: %d kv heads exceed the grid", nkv);
+  if (table_width <= 0) return me_fail("me_attention_prefill_bf16: empty block table");
   const int tpb = 128 / group;
   const float sl = scale * LOG2E;
+  int bs_shift = 0;
+  while ((1 << bs_shift) < bs) ++bs_shift;
   dim3 grid(num_blocks, nkv);
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
+  int rc = 0;
 #define ME_PREFILL_CASE(DD)                                                                                        \
   case DD:                                                                                                         \
-    attention_prefill_kernel<DD><<<grid, 256, 0, stream>>>(qq, kc, vc, positions, item_start, num_items, block_table, \
-                                                           table_width, (bf16_t*)out, nh, nkv, bs, window, sl, tpb); \
+    rc = launch_prefill<DD>(grid, qq, kc, vc, positions, item_start, num_items, block_table, table_width,          \
+                            (bf16_t*)out, nh, nkv, bs_shift, window, sl, tpb, stream);                             \
     break;
   switch (d) {
     ME_PREFILL_CASE(32)
@@ -440,5 +652,6 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
     ME_PREFILL_CASE(256)
   }
 #undef ME_PREFILL_CASE
+  if (rc) return rc;
   return me_check_launch("me_attention_prefill_bf16");
 }

@@ -105,33 +105,58 @@ extern "C" int me_rmsnorm(const void* in, const float* w, void* out, int num_row
 }
 
 // ------------------------------------------------------------------------------------ SwiGLU
-// act[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)).
+// act[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)). A thread handles VEC
+// consecutive i (16-byte loads when the row length allows it).
+template <typename T, int VEC>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t total_vec) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total_vec) return;
+  const int per_row = inter / VEC;
+  const size_t t = idx / per_row;
+  const int i = (int)(idx - t * per_row) * VEC;
+  struct alignas(sizeof(T) * VEC) Pack {
+    T v[VEC];
+  };
+  const Pack g = *reinterpret_cast<const Pack*>(gu + t * 2 * inter + i);
+  const Pack u = *reinterpret_cast<const Pack*>(gu + t * 2 * inter + inter + i);
+  Pack o;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    const float gf = to_float(g.v[k]);
+    o.v[k] = from_float<T>(gf / (1.f + expf(-gf)) * to_float(u.v[k]));
+  }
+  *reinterpret_cast<Pack*>(act + t * inter + i) = o;
+}
+
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t total) {
-  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= total) return;
-  const size_t t = idx / inter;
-  const int i = (int)(idx - t * inter);
-  const float g = to_float(gu[t * 2 * inter + i]);
-  const float u = to_float(gu[t * 2 * inter + inter + i]);
-  act[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
+static void launch_swiglu(const T* gu, T* act, int num_tokens, int inter, hipStream_t stream) {
+  constexpr int WIDE = 16 / sizeof(T);
+  const bool wide = inter % WIDE == 0 && ((uintptr_t)gu % 16 == 0) && ((uintptr_t)act % 16 == 0);
+  const int threads = 256;
+  if (wide) {
+    const size_t total = (size_t)num_tokens * (inter / WIDE);
+    swiglu_kernel<T, WIDE><<<(unsigned)((total + threads - 1) / threads), threads, 0, stream>>>(gu, act, inter, total);
+  } else {
+    const size_t total = (size_t)num_tokens * inter;
+    swiglu_kernel<T, 1><<<(unsigned)((total + threads - 1) / threads), threads, 0, stream>>>(gu, act, inter, total);
+  }
 }
 
 extern "C" int me_swiglu(const void* gu, void* act, int num_tokens, int inter, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (inter <= 0) return me_fail("me_swiglu: intermediate=%d", inter);
-  const size_t total = (size_t)num_tokens * inter;
-  const int threads = 256;
-  const unsigned blocks = (unsigned)((total + threads - 1) / threads);
   if (dtype == ME_F32)
-    swiglu_kernel<float><<<blocks, threads, 0, stream>>>((const float*)gu, (float*)act, inter, total);
+    launch_swiglu<float>((const float*)gu, (float*)act, num_tokens, inter, stream);
   else
-    swiglu_kernel<bf16_t><<<blocks, threads, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter, total);
+    launch_swiglu<bf16_t>((const bf16_t*)gu, (bf16_t*)act, num_tokens, inter, stream);
   return me_check_launch("me_swiglu");
 }
 
 // ------------------------------------------- per-head q/k RMSNorm + rotary + key/value page write
-// qkv is [T, (nh + 2*nkv) * d]: q heads, then k heads, then v heads. One wave per (token, head).
+// qkv is [T, (nh + 2*nkv) * d]: q heads, then k heads, then v heads. One block of four waves per
+// token: the cosines and sines of the token's angles are computed once into LDS (float32, the
+// accurate library routines: angles reach tens of thousands of radians), then each wave takes every
+// fourth head:
 //   q heads: optional RMSNorm over d with q_w, rotary, written to q_out [T, nh, d];
 //   k heads: optional RMSNorm with k_w, rotary, written to the key page   K[page, kvh, slot, d];
 //   v heads: copied to the transposed value page                          V[page, kvh, d, slot].
@@ -141,91 +166,96 @@ extern "C" int me_swiglu(const void* gu, void* act, int num_tokens, int inter, i
 #define ME_MAX_HEAD_DIM 256
 
 template <typename T>
-__global__ void qk_norm_rope_scatter_kernel(const T* __restrict__ qkv, const float* __restrict__ q_w,
-                                            const float* __restrict__ k_w, const float* __restrict__ inv_freq,
-                                            const int* __restrict__ positions, const int* __restrict__ token_item,
-                                            const int* __restrict__ block_table, int table_width,
-                                            T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                            int num_tokens, int nh, int nkv, int d, int rd, int bs, float eps,
-                                            int write_kv) {
+__global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
+    const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    const float* __restrict__ inv_freq, const int* __restrict__ positions, const int* __restrict__ token_item,
+    const int* __restrict__ block_table, int table_width, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, int nh, int nkv, int d, int rd, int bs, float eps, int write_kv) {
   __shared__ float stage[4][ME_MAX_HEAD_DIM];
+  __shared__ float cs[ME_MAX_HEAD_DIM / 2], sn[ME_MAX_HEAD_DIM / 2];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int t = blockIdx.x;
   const int heads_total = write_kv ? nh + 2 * nkv : nh;
-  const long long unit = (long long)blockIdx.x * 4 + wave;
-  if (unit >= (long long)num_tokens * heads_total) return;
-  const int t = (int)(unit / heads_total), hd = (int)(unit % heads_total);
-  const int width = (write_kv ? nh + 2 * nkv : nh) * d;  // q-only rows when nothing is written
-  const T* src = qkv + (size_t)t * width + (size_t)hd * d;
+  const int width = heads_total * d;  // q-only rows when nothing is written
   const int pos = positions[t];
-  const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
-
-  float vals[ME_MAX_HEAD_DIM / ME_WAVE];
-  float ss = 0.f;
-#pragma unroll
-  for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
-    const int i = lane + k * ME_WAVE;
-    vals[k] = i < d ? to_float(src[i]) : 0.f;
-    ss += vals[k] * vals[k];
-  }
-  const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
-  if (w) {
-    const float inv = rsqrtf(wave_sum(ss) / (float)d + eps);
-#pragma unroll
-    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
-      const int i = lane + k * ME_WAVE;
-      if (i < d) vals[k] = vals[k] * inv * w[i];
+  const int half = rd / 2;
+  if (inv_freq)
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      const float angle = (float)pos * inv_freq[j];
+      cs[j] = cosf(angle);
+      sn[j] = sinf(angle);
     }
+  __syncthreads();
+  int page = 0, slot = 0;
+  if (write_kv) {
+    page = block_table[(size_t)token_item[t] * table_width + pos / bs];
+    slot = pos % bs;
   }
-  if (kind != 2 && inv_freq) {
-    float* st = stage[wave];
+  for (int hd = wave; hd < heads_total; hd += 4) {
+    const T* src = qkv + (size_t)t * width + (size_t)hd * d;
+    const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
+    float vals[ME_MAX_HEAD_DIM / ME_WAVE];
+    float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
       const int i = lane + k * ME_WAVE;
-      if (i < d) st[i] = vals[k];
+      vals[k] = i < d ? to_float(src[i]) : 0.f;
+      ss += vals[k] * vals[k];
     }
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS writes of this wave are visible
-    const int half = rd / 2;
+    const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
+    if (w) {
+      const float inv = rsqrtf(wave_sum(ss) / (float)d + eps);
 #pragma unroll
-    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
-      const int i = lane + k * ME_WAVE;
-      if (i < rd) {
-        const int j = i < half ? i : i - half;
-        const float angle = (float)pos * inv_freq[j];
-        const float c = cosf(angle), s = sinf(angle);
-        vals[k] = i < half ? st[i] * c - st[i + half] * s : st[i] * c + st[i - half] * s;
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < d) vals[k] = vals[k] * inv * w[i];
       }
     }
-  }
-
-  if (kind == 0) {
-    T* dst = q_out + ((size_t)t * nh + hd) * d;
+    if (kind != 2 && inv_freq) {
+      float* st = stage[wave];
+      __builtin_amdgcn_wave_barrier();  // the previous head's reads of this wave's stage are done
 #pragma unroll
-    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
-      const int i = lane + k * ME_WAVE;
-      if (i < d) dst[i] = from_float<T>(vals[k]);
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < d) st[i] = vals[k];
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS writes of this wave are visible
+#pragma unroll
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < rd) {
+          const int j = i < half ? i : i - half;
+          const float c = cs[j], s = sn[j];
+          vals[k] = i < half ? st[i] * c - st[i + half] * s : st[i] * c + st[i - half] * s;
+        }
+      }
     }
-    return;
-  }
-  const int item = token_item[t];
-  const int page = block_table[(size_t)item * table_width + pos / bs];
-  if (page < 0) return;
-  const int slot = pos % bs;
-  if (kind == 1) {
-    const int kvh = hd - nh;
-    T* dst = k_cache + (((size_t)page * nkv + kvh) * bs + slot) * d;
+    if (kind == 0) {
+      T* dst = q_out + ((size_t)t * nh + hd) * d;
 #pragma unroll
-    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
-      const int i = lane + k * ME_WAVE;
-      if (i < d) dst[i] = from_float<T>(vals[k]);
-    }
-  } else {
-    const int kvh = hd - nh - nkv;
-    T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + slot;
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < d) dst[i] = from_float<T>(vals[k]);
+      }
+    } else if (page >= 0) {
+      if (kind == 1) {
+        const int kvh = hd - nh;
+        T* dst = k_cache + (((size_t)page * nkv + kvh) * bs + slot) * d;
 #pragma unroll
-    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
-      const int i = lane + k * ME_WAVE;
-      if (i < d) dst[(size_t)i * bs] = from_float<T>(vals[k]);
+        for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (i < d) dst[i] = from_float<T>(vals[k]);
+        }
+      } else {
+        const int kvh = hd - nh - nkv;
+        T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + slot;
+#pragma unroll
+        for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (i < d) dst[(size_t)i * bs] = from_float<T>(vals[k]);
+        }
+      }
     }
   }
 }
@@ -241,15 +271,13 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
   if (rd < 0 || rd > d || rd % 2) return me_fail("me_qk_norm_rope_scatter: rotary_dim=%d with head_dim=%d", rd, d);
   if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
     return me_fail("me_qk_norm_rope_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
-  const long long units = (long long)num_tokens * (write_kv ? nh + 2 * nkv : nh);
-  const unsigned blocks = (unsigned)((units + 3) / 4);
   if (dtype == ME_F32)
-    qk_norm_rope_scatter_kernel<float><<<blocks, 256, 0, stream>>>(
+    qk_norm_rope_scatter_kernel<float><<<num_tokens, 256, 0, stream>>>(
         (const float*)qkv, q_w, k_w, inv_freq, positions, token_item, block_table, table_width, (float*)q_out,
-        (float*)k_cache, (float*)v_cache, num_tokens, nh, nkv, d, rd, bs, eps, write_kv);
+        (float*)k_cache, (float*)v_cache, nh, nkv, d, rd, bs, eps, write_kv);
   else
-    qk_norm_rope_scatter_kernel<bf16_t><<<blocks, 256, 0, stream>>>(
+    qk_norm_rope_scatter_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
         (const bf16_t*)qkv, q_w, k_w, inv_freq, positions, token_item, block_table, table_width, (bf16_t*)q_out,
-        (bf16_t*)k_cache, (bf16_t*)v_cache, num_tokens, nh, nkv, d, rd, bs, eps, write_kv);
+        (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, rd, bs, eps, write_kv);
   return me_check_launch("me_qk_norm_rope_scatter");
 }

@@ -1,0 +1,209 @@
+// Skinny bfloat16 product y = x . W^T for decode-sized batches (M <= 64 rows) with what surrounds
+// it in a layer fused in, so that a decode step needs fewer, fatter kernels:
+//
+//   prologue NORM:   the input is the float32 residual stream. Every block forms
+//                    s = x_in + delta (float32), uses bf16(s * w_norm) as its operand, sums s^2 on the
+//                    way and multiplies its results by rsqrt(mean(s^2) + eps) at the end (the scale of
+//                    a row is a common factor of the whole row of the product). Block 0 also writes s
+//                    to x_out, the new residual stream; x_out must not alias x_in, since the other
+//                    blocks still read x_in.
+//   epilogue SWIGLU: W holds gate rows [0, N) and up rows [N, 2N); a block computes 16 gate columns and
+//                    the 16 matching up columns and writes silu(gate) * up.
+//
+// A block owns 16 output columns and all M rows; its WAVES waves split k in interleaved chunks of 32
+// and add their partial sums through LDS in wave order. Products use v_mfma_f32_16x16x32_bf16 with
+// the transposed arrangement (C^T[n, m] = sum_k W[n, k] X[m, k]): lane l feeds W[n0 + l%16][8 k] and
+// X[m0 + l%16][8 k] (k = 32 c + 8 (l/16) ..), both contiguous in memory, and receives
+// C^T[4 (l/16) .. +4][l%16]. All loads of a round of U chunks are issued before its products.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+template <int MT, int WAVES, int U, bool NORM, bool SWIGLU, typename OutT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
+    const bf16_t* __restrict__ X, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+    const float* __restrict__ w_norm, float eps, float* __restrict__ x_out, const bf16_t* __restrict__ W,
+    OutT* __restrict__ C, int M, int N, int K) {
+  constexpr int ACCS = SWIGLU ? 2 : 1;
+  __shared__ float red[WAVES][MT * ACCS][64][4];
+  __shared__ float ssq[WAVES][MT][64];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int n0 = blockIdx.x * 16;
+  const int r = lane & 15, g = lane >> 4;
+  const int n = n0 + r;
+  const bool n_ok = n < N;
+  const bf16_t* wrow = W + (size_t)(n_ok ? n : 0) * K;
+  const bf16_t* wrow_up = SWIGLU ? W + ((size_t)N + (n_ok ? n : 0)) * K : nullptr;
+  float4_t acc[MT][ACCS];
+  float ss[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    ss[t] = 0.f;
+#pragma unroll
+    for (int a = 0; a < ACCS; ++a) acc[t][a] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  }
+  const bool writes_x = NORM && delta != nullptr && blockIdx.x == 0;
+
+  const int chunks = (K + 31) / 32;
+  for (int c0 = wave; c0 < chunks; c0 += WAVES * U) {
+    bf16x8_t a[U][ACCS], b[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (c0 + WAVES * u) * 32 + g * 8;
+      const bool k_ok = k < K;  // K % 8 == 0 is checked on the host
+      a[u][0] = bf16x8_t{};
+      if (n_ok && k_ok) a[u][0] = *reinterpret_cast<const bf16x8_t*>(wrow + k);
+      if (SWIGLU) {
+        a[u][ACCS - 1] = bf16x8_t{};
+        if (n_ok && k_ok) a[u][ACCS - 1] = *reinterpret_cast<const bf16x8_t*>(wrow_up + k);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (c0 + WAVES * u) * 32 + g * 8;
+      const bool k_ok = k < K;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r;
+        b[u][t] = bf16x8_t{};
+        if (m < M && k_ok) {
+          if (NORM) {
+            const float4 x0 = *reinterpret_cast<const float4*>(x_in + (size_t)m * K + k);
+            const float4 x1 = *reinterpret_cast<const float4*>(x_in + (size_t)m * K + k + 4);
+            float s[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            if (delta) {
+              const uint4 dv = *reinterpret_cast<const uint4*>(delta + (size_t)m * K + k);
+              const uint32_t dw[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                s[2 * j] += __uint_as_float(dw[j] << 16);
+                s[2 * j + 1] += __uint_as_float(dw[j] & 0xffff0000u);
+              }
+              if (writes_x) {
+                *reinterpret_cast<float4*>(x_out + (size_t)m * K + k) = make_float4(s[0], s[1], s[2], s[3]);
+                *reinterpret_cast<float4*>(x_out + (size_t)m * K + k + 4) = make_float4(s[4], s[5], s[6], s[7]);
+              }
+            }
+            const float4 w0 = *reinterpret_cast<const float4*>(w_norm + k);
+            const float4 w1 = *reinterpret_cast<const float4*>(w_norm + k + 4);
+            const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              ss[t] = fmaf(s[j], s[j], ss[t]);
+              b[u][t][j] = (__bf16)(s[j] * wv[j]);
+            }
+          } else {
+            b[u][t] = *reinterpret_cast<const bf16x8_t*>(X + (size_t)m * K + k);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int aa = 0; aa < ACCS; ++aa)
+          acc[t][aa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][aa], b[u][t], acc[t][aa], 0, 0, 0);
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+#pragma unroll
+    for (int aa = 0; aa < ACCS; ++aa)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) red[wave][t * ACCS + aa][lane][j] = acc[t][aa][j];
+    if (NORM) ssq[wave][t][lane] = ss[t];
+  }
+  __syncthreads();
+  // thread -> (tile t, lane l): row m = 16 t + l % 16, columns n0 + 4 (l / 16) .. +4
+  for (int idx = threadIdx.x; idx < MT * 64; idx += WAVES * 64) {
+    const int t = idx / 64, l = idx % 64;
+    const int m = t * 16 + (l & 15);
+    const int nb = n0 + (l >> 4) * 4;
+    if (m >= M) continue;
+    float scale = 1.f;
+    if (NORM) {
+      // the row's sum of squares: every wave's lanes (l % 16) + 16 g hold a part of it
+      float total = 0.f;
+      for (int w = 0; w < WAVES; ++w)
+        total += (ssq[w][t][l & 15] + ssq[w][t][(l & 15) + 16]) + (ssq[w][t][(l & 15) + 32] + ssq[w][t][(l & 15) + 48]);
+      scale = rsqrtf(total / (float)K + eps);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v0 = 0.f, v1 = 0.f;
+      for (int w = 0; w < WAVES; ++w) {
+        v0 += red[w][t * ACCS][l][j];
+        if (SWIGLU) v1 += red[w][t * ACCS + 1][l][j];
+      }
+      v0 *= scale;
+      float y = v0;
+      if (SWIGLU) y = v0 / (1.f + expf(-v0)) * (v1 * scale);
+      if (nb + j < N) C[(size_t)m * N + nb + j] = from_float<OutT>(y);
+    }
+  }
+}
+
+template <int MT, int WAVES, int U, typename OutT>
+static void launch_variant(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
+                           const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
+                           hipStream_t stream) {
+  const unsigned blocks = (N + 15) / 16;
+#define ME_LAUNCH(NORM, SWI)                                                                                  \
+  gemm_small_kernel<MT, WAVES, U, NORM, SWI, OutT><<<blocks, WAVES * 64, 0, stream>>>(X, x_in, delta, w_norm, eps, \
+                                                                                      x_out, W, C, M, N, K)
+  if (norm && swiglu)
+    ME_LAUNCH(true, true);
+  else if (norm)
+    ME_LAUNCH(true, false);
+  else if (swiglu)
+    ME_LAUNCH(false, true);
+  else
+    ME_LAUNCH(false, false);
+#undef ME_LAUNCH
+}
+
+template <typename OutT>
+static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
+                         const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
+                         hipStream_t stream) {
+  const int mt = (M + 15) / 16;
+  if (mt == 1)
+    launch_variant<1, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else if (mt == 2)
+    launch_variant<2, 8, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else if (mt == 3)
+    launch_variant<3, 4, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else
+    launch_variant<4, 4, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+}
+
+// C[M, N] = epilogue(prologue(input) . W^T).
+//   norm == 0: input is X (bfloat16 [M, K]).  norm == 1: input is rmsnorm(x_in + delta) * w_norm, from the
+//   float32 residual stream x_in [M, K], delta (bfloat16 [M, K] or null), w_norm float32 [K]; when delta
+//   is given, x_in + delta is written to x_out (float32 [M, K], not aliasing x_in).
+//   swiglu == 0: W is [N, K].  swiglu == 1: W is [2 N, K] (gate rows, then up rows), C = silu(gate) * up.
+//   out_dtype: ME_BF16 or ME_F32. M <= 64, K % 8 == 0, pointers 16-byte aligned.
+extern "C" int me_gemm_bf16_small(const void* X, const float* x_in, const void* delta, const float* w_norm, float eps,
+                                  float* x_out, const void* W, void* C, int M, int N, int K, int norm, int swiglu,
+                                  int out_dtype, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64) return me_fail("me_gemm_bf16_small: M=%d exceeds 64 rows", M);
+  if (K <= 0 || K % 8) return me_fail("me_gemm_bf16_small: K=%d must be a positive multiple of 8", K);
+  if (norm) {
+    if (!x_in || !w_norm) return me_fail("me_gemm_bf16_small: the norm prologue needs x_in and w_norm");
+    if (delta && (!x_out || x_out == x_in)) return me_fail("me_gemm_bf16_small: x_out must be given and must not alias x_in");
+    if (((uintptr_t)x_in | (uintptr_t)delta | (uintptr_t)w_norm | (uintptr_t)x_out) & 15)
+      return me_fail("me_gemm_bf16_small: residual operands must be 16-byte aligned");
+  } else if (!X) {
+    return me_fail("me_gemm_bf16_small: X is null");
+  }
+  if (((uintptr_t)X | (uintptr_t)W) & 15) return me_fail("me_gemm_bf16_small: operands must be 16-byte aligned");
+  const bf16_t *x = (const bf16_t*)X, *d = (const bf16_t*)delta, *w = (const bf16_t*)W;
+  if (out_dtype == ME_F32)
+    launch_small<float>(norm, swiglu, x, x_in, d, w_norm, eps, x_out, w, (float*)C, M, N, K, stream);
+  else
+    launch_small<bf16_t>(norm, swiglu, x, x_in, d, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, stream);
+  return me_check_launch("me_gemm_bf16_small");
+}

@@ -208,9 +208,6 @@ def attention_general(
 
 # ------------------------------------------------------------------------------ matrix products
 
-SKINNY_MAX_ROWS = 64
-
-
 def gemm_f32(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """float32 ``x @ weight.T`` on the vector units, additions in ascending k for every element."""
     _want(x, "x", torch.float32, (None, None))
@@ -224,44 +221,121 @@ def gemm_f32(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = N
     return out
 
 
-def gemm_bf16_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                     out: torch.Tensor | None = None) -> torch.Tensor:
-    """bfloat16 ``x @ weight.T`` for at most 64 rows of x, float32 accumulation on the matrix cores."""
-    _want(x, "x", torch.bfloat16, (None, None))
+class NormedInput:
+    """``rmsnorm(x + delta) * weight`` not yet computed: what a block hands to a part that can take
+    the residual add and the norm as the prologue of its first matrix product.
+
+    ``x`` is the float32 residual stream [T, D], ``delta`` the pending addition in the compute dtype
+    (or None), ``spare`` a second float32 buffer of x's shape. Whoever consumes the input performs the
+    residual add; afterwards :attr:`residual` is the buffer that holds ``x + delta``."""
+
+    def __init__(self, x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                 dtype: torch.dtype, spare: torch.Tensor | None):
+        self.x, self.delta, self.weight, self.eps, self.dtype, self.spare = x, delta, weight, eps, dtype, spare
+        self.residual: torch.Tensor | None = None
+        self._tensor: torch.Tensor | None = None
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    def materialize(self) -> torch.Tensor:
+        """Run the add-and-norm kernel (once) and return the normed activations."""
+        if self._tensor is None:
+            if self.residual is not None:  # the add already happened in a fused product
+                self._tensor = add_rmsnorm(self.residual, None, self.weight, self.eps, self.dtype)
+            else:
+                self._tensor = add_rmsnorm(self.x, self.delta, self.weight, self.eps, self.dtype)
+                self.residual = self.x
+        return self._tensor
+
+    def fusable(self, weight: torch.Tensor) -> bool:
+        return (self.dtype is torch.bfloat16 and self._tensor is None and self.x.shape[0] <= SMALL_MAX_ROWS
+                and self.x.shape[1] % 8 == 0 and (self.delta is None or self.spare is not None)
+                and weight.dtype is torch.bfloat16)
+
+
+SMALL_MAX_ROWS = 64
+
+
+def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
+    """bfloat16 ``x @ weight.T`` for at most 64 rows on the matrix cores, float32 accumulation.
+
+    ``x`` is a bfloat16 tensor [M, K] or a :class:`NormedInput` (then the residual add and the RMSNorm
+    are the product's prologue). With ``swiglu`` the weight holds gate rows then up rows, [2N, K], and
+    the result is ``silu(gate) * up`` [M, N]."""
+    normed = isinstance(x, NormedInput)
     m, k = x.shape
     _want(weight, "weight", torch.bfloat16, (None, k))
     n = weight.shape[0]
-    if m > SKINNY_MAX_ROWS:
-        raise ValueError(f"gemm_bf16_skinny takes at most {SKINNY_MAX_ROWS} rows, got {m}")
+    if swiglu:
+        if n % 2:
+            raise ValueError(f"a gate/up weight needs an even number of rows, got {n}")
+        n //= 2
+    if m > SMALL_MAX_ROWS:
+        raise ValueError(f"gemm_bf16_small takes at most {SMALL_MAX_ROWS} rows, got {m}")
     if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        out = torch.empty((m, n), dtype=out_dtype, device=weight.device)
     _want(out, "out", out_dtype, (m, n))
-    check(lib().me_gemm_bf16_skinny(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(_code(out_dtype)), _stream()))
+    if normed:
+        _want(x.x, "residual stream", torch.float32, (m, k))
+        _want(x.weight, "norm weight", torch.float32, (k,))
+        x_out = None
+        if x.delta is not None:
+            _want(x.delta, "delta", torch.bfloat16, (m, k))
+            _want(x.spare, "spare residual buffer", torch.float32, (m, k))
+            if x.spare.data_ptr() == x.x.data_ptr():
+                raise ValueError("the spare residual buffer must not alias the residual stream")
+            x_out = x.spare
+        check(lib().me_gemm_bf16_small(_p(None), _p(x.x), _p(x.delta), _p(x.weight), _f(x.eps), _p(x_out), _p(weight),
+                                       _p(out), _i(m), _i(n), _i(k), _i(1), _i(1 if swiglu else 0),
+                                       _i(_code(out_dtype)), _stream()))
+        x.residual = x.x if x.delta is None else x.spare
+    else:
+        _want(x, "x", torch.bfloat16, (m, k))
+        check(lib().me_gemm_bf16_small(_p(x), _p(None), _p(None), _p(None), _f(0.0), _p(None), _p(weight), _p(out),
+                                       _i(m), _i(n), _i(k), _i(0), _i(1 if swiglu else 0), _i(_code(out_dtype)),
+                                       _stream()))
     return out
 
 
-def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    return (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
+def gemm_bf16_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                     out: torch.Tensor | None = None) -> torch.Tensor:
+    """The plain form of :func:`gemm_bf16_small` (no prologue, no epilogue)."""
+    return gemm_bf16_small(x, weight, out_dtype, False, out)
+
+
+def small_ok(x, weight: torch.Tensor) -> bool:
+    return (x.shape[0] <= SMALL_MAX_ROWS and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
             and weight.data_ptr() % 16 == 0)
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """``x @ weight.T`` for x [M, K], weight [N, K].
+def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False) -> torch.Tensor:
+    """``x @ weight.T`` for x [M, K], weight [N, K]; with ``gated`` the weight is [2N, K] (gate rows,
+    then up rows) and the result is ``silu(gate) * up``. ``x`` may be a :class:`NormedInput`.
 
     float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16: the
-    skinny matrix-core kernel for up to 64 rows, else the GEMM library; rows are processed in
-    slices of 64 when a float32 result is wanted from bfloat16 inputs (logits)."""
+    fused matrix-core kernel for up to 64 rows, else the GEMM library; rows are processed in slices
+    of 64 when a float32 result is wanted from bfloat16 inputs (logits)."""
+    if isinstance(x, NormedInput):
+        if x.fusable(weight):
+            return gemm_bf16_small(x, weight, out_dtype or x.dtype, gated)
+        x = x.materialize()
     out_dtype = out_dtype or x.dtype
     if x.dtype is torch.float32:
         if out_dtype is not torch.float32:
             raise TypeError("the float32 path keeps float32 results")
-        return gemm_f32(x, weight)
-    if skinny_ok(x, weight):
-        return gemm_bf16_skinny(x, weight, out_dtype)
+        y = gemm_f32(x, weight)
+        return swiglu(y) if gated else y
+    if small_ok(x, weight):
+        return gemm_bf16_small(x, weight, out_dtype, gated)
+    if gated:
+        return swiglu(linear(x, weight, out_dtype))
     if out_dtype is torch.float32 and x.shape[1] % 8 == 0:
         out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
-        for lo in range(0, x.shape[0], SKINNY_MAX_ROWS):
-            gemm_bf16_skinny(x[lo:lo + SKINNY_MAX_ROWS], weight, torch.float32, out[lo:lo + SKINNY_MAX_ROWS])
+        for lo in range(0, x.shape[0], SMALL_MAX_ROWS):
+            gemm_bf16_small(x[lo:lo + SMALL_MAX_ROWS], weight, torch.float32, False, out[lo:lo + SMALL_MAX_ROWS])
         return out
     y = torch.matmul(x, weight.t())
     return y if out_dtype is y.dtype else y.to(out_dtype)

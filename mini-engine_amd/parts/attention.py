@@ -76,7 +76,9 @@ class Attention(Mixer):
         return self.spec.cache_from
 
     # ---- step
-    def forward(self, h: torch.Tensor, batch, cache: KVBinding | None = None) -> torch.Tensor:
+    takes_normed_input = True
+
+    def forward(self, h, batch, cache: KVBinding | None = None) -> torch.Tensor:
         s, b = self.spec, cache
         if b is None:
             raise RuntimeError("attention mixer was given no cache")

@@ -11,6 +11,11 @@ it is in. The four interfaces:
                        ``forward(h, batch, cache) -> [T, hidden]``.
 ``FeedForward``        ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``forward(h, batch) -> [T, hidden]``.
 
+A mixer or feed-forward class may set ``takes_normed_input = True``; its ``forward`` is then handed a
+``NormedInput`` (the residual add and the norm not yet evaluated) instead of a tensor and passes it
+to ``ops.kernels.linear`` as the input of its first matrix product, which fuses both into that
+product for decode-sized batches (``h.materialize()`` gives the tensor where it is needed).
+
 ``h`` is the normed input [T, hidden] in the compute dtype, ``batch`` a ``StepBatch`` (token
 positions, item boundaries, block tables per cache group, state slots), ``cache`` the binding
 (``KVBinding`` / ``StateBinding`` / None) of this run of the layer: a layer that the order names

@@ -41,14 +41,26 @@ class PreNormBlock:
         self.ffn_norm.load(tensors, s.ffn_norm_name)
         self.ffn.load(tensors, s.ffn_prefix)
 
-    def forward(self, x: torch.Tensor, pending: torch.Tensor | None, batch, cache=None) -> torch.Tensor:
-        """``x`` float32 [T, H] residual stream (updated in place); ``pending`` is the previous
-        block's output that still has to be added; ``cache`` is the binding of this run of the
-        layer. Returns this block's own pending output."""
-        h = K.add_rmsnorm(x, pending, self.mixer_norm.weight, self.mixer_norm.eps, self.dtype)
-        a = self.mixer.forward(h, batch, cache)
-        h = K.add_rmsnorm(x, a, self.ffn_norm.weight, self.ffn_norm.eps, self.dtype)
-        return self.ffn.forward(h, batch)
+    def forward(self, x: torch.Tensor, pending: torch.Tensor | None, batch, cache=None, spare: torch.Tensor | None = None):
+        """``x`` float32 [T, H] is the residual stream, ``pending`` the previous block's output that
+        still has to be added, ``cache`` the binding of this run of the layer, ``spare`` a second
+        float32 buffer of x's shape. Returns ``(x, spare, pending)``: the buffer that now holds the
+        residual stream, the other one, and this block's own pending output.
+
+        A part whose class sets ``takes_normed_input`` is handed the add-and-norm unevaluated
+        (:class:`~mini_engine_amd.ops.kernels.NormedInput`) and may fuse it into its first matrix
+        product; any other part gets the normed activations."""
+        x, spare, a = self._run(self.mixer, self.mixer_norm, x, pending, spare, batch, (cache,))
+        return self._run(self.ffn, self.ffn_norm, x, a, spare, batch, ())
+
+    def _run(self, part, norm, x, pending, spare, batch, extra):
+        h = K.NormedInput(x, pending, norm.weight, norm.eps, self.dtype, spare)
+        out = part.forward(h if getattr(part, "takes_normed_input", False) else h.materialize(), batch, *extra)
+        if h.residual is None:  # the part never looked at its input: the add still has to happen
+            h.materialize()
+        if h.residual is not x:
+            x, spare = h.residual, x
+        return x, spare, out
 
 
 BLOCK_ARRANGEMENTS = {"pre_norm": PreNormBlock}

@@ -86,9 +86,10 @@ class Decoder:
         if self.embed_table is None:
             raise RuntimeError("weights are not loaded")
         x = K.embed(batch.token_ids, self.embed_table)
+        spare = torch.empty_like(x)  # the residual stream alternates between two buffers
         pending = None
         for r, i in enumerate(self.plan.order):
-            pending = self.blocks[i].forward(x, pending, batch, self.bindings[r])
+            x, spare, pending = self.blocks[i].forward(x, pending, batch, self.bindings[r], spare)
         return self.logits(x, pending, batch.want_rows)
 
     def logits(self, x: torch.Tensor, pending: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:

@@ -30,9 +30,10 @@ class GatedMlp(FeedForward):
         self.w_gate_up = torch.cat((tensors[f"{prefix}.gate_proj.weight"], tensors[f"{prefix}.up_proj.weight"]), dim=0)
         self.w_down = tensors[f"{prefix}.down_proj.weight"]
 
-    def forward(self, h: torch.Tensor, batch=None) -> torch.Tensor:
-        gate_up = K.linear(h, self.w_gate_up)
-        act = K.swiglu(gate_up)
+    takes_normed_input = True
+
+    def forward(self, h, batch=None) -> torch.Tensor:
+        act = K.linear(h, self.w_gate_up, gated=True)
         return K.linear(act, self.w_down)
 
 

@@ -101,6 +101,48 @@ def test_gemm_bf16_skinny(m, n, k, out_dtype):
     torch.testing.assert_close(out.float().cpu(), want, **t)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 96, 72), (16, 1000, 1024), (33, 64, 160), (64, 160, 3072)])
+@pytest.mark.parametrize("with_delta", [True, False])
+@pytest.mark.parametrize("gated", [True, False])
+def test_gemm_bf16_small_with_norm_prologue_and_swiglu_epilogue(m, n, k, with_delta, gated):
+    """The fused form against its unfused definition: rmsnorm(x + delta) * w, product, silu(gate) * up;
+    the residual stream comes out in the second buffer and the first is left untouched."""
+    g = torch.Generator().manual_seed(m * 1000 + n)
+    x = torch.randn(m, k, generator=g) * 2
+    delta = torch.randn(m, k, generator=g).bfloat16() if with_delta else None
+    wn = 1 + 0.2 * torch.randn(k, generator=g)
+    w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
+    xd, spare = dev(x.clone()), dev(torch.full((m, k), 7.0))
+    h = K().NormedInput(xd, None if delta is None else dev(delta), dev(wn), 1e-5, torch.bfloat16, spare)
+    assert h.fusable(dev(w))
+    out = K().linear(h, dev(w), gated=gated).float().cpu()
+    s = x + (delta.float() if with_delta else 0)
+    y = plain.rms_norm(s, wn, 1e-5) @ w.float().T
+    want = plain.silu(y[:, :n]) * y[:, n:] if gated else y
+    torch.testing.assert_close(out, want, rtol=2e-2, atol=2e-2 * max(1.0, want.abs().max().item()))
+    assert torch.equal(xd.cpu(), x)  # the input buffer is only read
+    if with_delta:
+        assert h.residual is spare
+        torch.testing.assert_close(spare.cpu(), s, rtol=1e-6, atol=1e-6)  # a float32 sum
+    else:
+        assert h.residual is xd and torch.equal(spare.cpu(), torch.full((m, k), 7.0))
+
+
+def test_normed_input_falls_back_to_the_separate_kernels():
+    """More than 64 rows or float32: the add-and-norm kernel runs, in place, and the product follows."""
+    for dtype, m in ((torch.bfloat16, 100), (torch.float32, 5)):
+        x, delta = torch.randn(m, 64), torch.randn(m, 64).to(dtype)
+        wn, w = 1 + 0.1 * torch.randn(64), (torch.randn(48, 64) * 0.1).to(dtype)
+        xd = dev(x.clone())
+        h = K().NormedInput(xd, dev(delta), dev(wn), 1e-6, dtype, dev(torch.zeros(m, 64)))
+        out = K().linear(h, dev(w), gated=True).float().cpu()
+        s = x + delta.float()
+        y = plain.rms_norm(s, wn, 1e-6) @ w.float().T
+        torch.testing.assert_close(out, plain.silu(y[:, :24]) * y[:, 24:], **tol(dtype))
+        assert h.residual is xd
+        torch.testing.assert_close(xd.cpu(), s, rtol=1e-6, atol=1e-6)
+
+
 def test_gemm_bf16_skinny_refuses_what_it_cannot_do():
     from mini_engine_amd.ops.library import KernelError
 
@@ -312,7 +354,7 @@ def test_temperature_sampling_is_keyed_repeatable_and_follows_softmax():
 
 
 # -------------------------------------------------------- matrix-core attention kernels (bfloat16)
-MFMA_SHAPES = [(4, 2, 32, 16), (6, 1, 32, 16), (16, 8, 128, 16), (8, 8, 64, 32), (16, 1, 64, 16), (3, 1, 96, 48),
+MFMA_SHAPES = [(4, 2, 32, 16), (6, 1, 32, 16), (16, 8, 128, 16), (8, 8, 64, 32), (16, 1, 64, 16), (3, 1, 96, 64),
                (2, 2, 256, 16), (40, 2, 32, 16)]
 
 
@@ -389,7 +431,7 @@ def test_mfma_attention_finds_one_far_key_and_respects_the_window_edge(kernel):
 
 def test_mfma_attention_refuses_unsupported_sizes():
     assert not K().attention_mfma_supported(16, 16)
-    assert not K().attention_mfma_supported(128, 8)
+    assert not K().attention_mfma_supported(128, 8) and not K().attention_mfma_supported(128, 48)
     assert K().attention_mfma_supported(128, 16) and not K().attention_mfma_supported(128, 16, group=17)
     from mini_engine_amd.ops.library import KernelError
 
