@@ -152,46 +152,60 @@ extern "C" int me_swiglu(const void* gu, void* act, int num_tokens, int inter, i
   return me_check_launch("me_swiglu");
 }
 
+// ------------------------------------------------------------------- rotary cos/sin table
+// table[pos, 0, j] = cos(pos * inv_freq[j]), table[pos, 1, j] = sin(pos * inv_freq[j]) in float32, with
+// the accurate library routines (angles reach tens of thousands of radians). Computed once per model;
+// every kernel that rotates reads it, so all of them see the same bits for a position.
+__global__ void rope_table_kernel(float* __restrict__ table, const float* __restrict__ inv_freq, int half,
+                                  int num_positions) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= num_positions * half) return;
+  const int pos = idx / half, j = idx % half;
+  const float angle = (float)pos * inv_freq[j];
+  table[((size_t)pos * 2) * half + j] = cosf(angle);
+  table[((size_t)pos * 2 + 1) * half + j] = sinf(angle);
+}
+
+extern "C" int me_rope_table(float* table, const float* inv_freq, int half, int num_positions, hipStream_t stream) {
+  if (half <= 0 || num_positions <= 0) return me_fail("me_rope_table: half=%d positions=%d", half, num_positions);
+  const long long total = (long long)half * num_positions;
+  rope_table_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(table, inv_freq, half, num_positions);
+  return me_check_launch("me_rope_table");
+}
+
 // ------------------------------------------- per-head q/k RMSNorm + rotary + key/value page write
-// qkv is [T, (nh + 2*nkv) * d]: q heads, then k heads, then v heads. One block of four waves per
-// token: the cosines and sines of the token's angles are computed once into LDS (float32, the
-// accurate library routines: angles reach tens of thousands of radians), then each wave takes every
-// fourth head:
+// qkv is [T, (nh + 2*nkv) * d]: q heads, then k heads, then v heads. Grid (token, group of heads),
+// four waves per block, a wave per head at a time:
 //   q heads: optional RMSNorm over d with q_w, rotary, written to q_out [T, nh, d];
 //   k heads: optional RMSNorm with k_w, rotary, written to the key page   K[page, kvh, slot, d];
 //   v heads: copied to the transposed value page                          V[page, kvh, d, slot].
 // page = block_table[item, pos / bs], slot = pos % bs. Rotary: pairs (j, j + rd/2), j < rd/2, with
-// angle pos * inv_freq[j]; dims >= rd pass through. inv_freq == nullptr means no rotary.
+// cos/sin of pos * inv_freq[j] read from rope_table [positions, 2, rd/2]; dims >= rd pass through.
+// rope_table == nullptr means no rotary.
 // write_kv == 0: qkv is [T, nh * d] and only q is processed (a layer that reads another layer's cache).
 #define ME_MAX_HEAD_DIM 256
 
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
-    const float* __restrict__ inv_freq, const int* __restrict__ positions, const int* __restrict__ token_item,
+    const float* __restrict__ rope_table, const int* __restrict__ positions, const int* __restrict__ token_item,
     const int* __restrict__ block_table, int table_width, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, int nh, int nkv, int d, int rd, int bs, float eps, int write_kv) {
+    T* __restrict__ v_cache, int nh, int nkv, int d, int rd, int bs, float eps, int write_kv, int heads_per_block) {
   __shared__ float stage[4][ME_MAX_HEAD_DIM];
-  __shared__ float cs[ME_MAX_HEAD_DIM / 2], sn[ME_MAX_HEAD_DIM / 2];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int t = blockIdx.x;
   const int heads_total = write_kv ? nh + 2 * nkv : nh;
   const int width = heads_total * d;  // q-only rows when nothing is written
   const int pos = positions[t];
   const int half = rd / 2;
-  if (inv_freq)
-    for (int j = threadIdx.x; j < half; j += blockDim.x) {
-      const float angle = (float)pos * inv_freq[j];
-      cs[j] = cosf(angle);
-      sn[j] = sinf(angle);
-    }
-  __syncthreads();
+  const float* cs = rope_table ? rope_table + (size_t)pos * rd : nullptr;  // [2, half] of this position
   int page = 0, slot = 0;
   if (write_kv) {
     page = block_table[(size_t)token_item[t] * table_width + pos / bs];
     slot = pos % bs;
   }
-  for (int hd = wave; hd < heads_total; hd += 4) {
+  const int hd_end = min(heads_total, (int)(blockIdx.y + 1) * heads_per_block);
+  for (int hd = blockIdx.y * heads_per_block + wave; hd < hd_end; hd += 4) {
     const T* src = qkv + (size_t)t * width + (size_t)hd * d;
     const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
     float vals[ME_MAX_HEAD_DIM / ME_WAVE];
@@ -211,7 +225,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
         if (i < d) vals[k] = vals[k] * inv * w[i];
       }
     }
-    if (kind != 2 && inv_freq) {
+    if (kind != 2 && cs) {
       float* st = stage[wave];
       __builtin_amdgcn_wave_barrier();  // the previous head's reads of this wave's stage are done
 #pragma unroll
@@ -226,8 +240,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
         const int i = lane + k * ME_WAVE;
         if (i < rd) {
           const int j = i < half ? i : i - half;
-          const float c = cs[j], s = sn[j];
-          vals[k] = i < half ? st[i] * c - st[i + half] * s : st[i] * c + st[i - half] * s;
+          const float c = cs[j], sn = cs[half + j];
+          vals[k] = i < half ? st[i] * c - st[i + half] * sn : st[i] * c + st[i - half] * sn;
         }
       }
     }
@@ -260,7 +274,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
   }
 }
 
-extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w, const float* inv_freq,
+// rope_table: float32 [num_positions, 2, rd / 2] or null; every position of the step must be below
+// num_positions (checked by the caller against the engine's length limit).
+extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table,
                                        const int* positions, const int* token_item, const int* block_table,
                                        int table_width, void* q_out, void* k_cache, void* v_cache, int num_tokens,
                                        int nh, int nkv, int d, int rd, int bs, float eps, int write_kv, int dtype,
@@ -271,13 +287,18 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
   if (rd < 0 || rd > d || rd % 2) return me_fail("me_qk_norm_rope_scatter: rotary_dim=%d with head_dim=%d", rd, d);
   if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
     return me_fail("me_qk_norm_rope_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
+  const int heads_total = write_kv ? nh + 2 * nkv : nh;
+  // few tokens: spread the heads over many blocks; many tokens: a block per token keeps its table rows hot
+  const int hpb = num_tokens >= 512 ? heads_total : 4;
+  dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
+  if (grid.y > 65535) return me_fail("me_qk_norm_rope_scatter: too many heads");
   if (dtype == ME_F32)
-    qk_norm_rope_scatter_kernel<float><<<num_tokens, 256, 0, stream>>>(
-        (const float*)qkv, q_w, k_w, inv_freq, positions, token_item, block_table, table_width, (float*)q_out,
-        (float*)k_cache, (float*)v_cache, nh, nkv, d, rd, bs, eps, write_kv);
+    qk_norm_rope_scatter_kernel<float><<<grid, 256, 0, stream>>>(
+        (const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (float*)q_out,
+        (float*)k_cache, (float*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb);
   else
-    qk_norm_rope_scatter_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
-        (const bf16_t*)qkv, q_w, k_w, inv_freq, positions, token_item, block_table, table_width, (bf16_t*)q_out,
-        (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, rd, bs, eps, write_kv);
+    qk_norm_rope_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+        (const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (bf16_t*)q_out,
+        (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb);
   return me_check_launch("me_qk_norm_rope_scatter");
 }

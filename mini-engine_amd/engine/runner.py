@@ -58,7 +58,8 @@ class ModelRunner:
 
         After a replayed step the result is a view of the graph's output buffer: read it before the
         next step."""
-        validate_items(items, self.decoder.plan.vocab_size, self.config.block_size, self.layout.groups)
+        validate_items(items, self.decoder.plan.vocab_size, self.config.block_size, self.layout.groups,
+                       self.config.max_model_len)
         if self.layout.has_state:
             self.storage.zero_state([it.seq.state_slot for it in items if it.start == 0 and it.seq.state_slot >= 0])
         if self._graph_eligible(items):

@@ -135,11 +135,20 @@ def _check_step_index(positions, token_item, block_table, t):
     _want(block_table, "block_table", torch.int32, (None, None))
 
 
+def rope_table(inv_freq: torch.Tensor, num_positions: int) -> torch.Tensor:
+    """float32 [num_positions, 2, rotary_dim / 2]: cos and sin of ``position * inv_freq[j]``."""
+    _want(inv_freq, "inv_freq", torch.float32, (None,))
+    half = inv_freq.numel()
+    table = torch.empty((num_positions, 2, half), dtype=torch.float32, device=inv_freq.device)
+    check(lib().me_rope_table(_p(table), _p(inv_freq), _i(half), _i(num_positions), _stream()))
+    return table
+
+
 def qk_norm_rope_scatter(
     qkv: torch.Tensor,
     q_weight: torch.Tensor | None,
     k_weight: torch.Tensor | None,
-    inv_freq: torch.Tensor | None,
+    rope: torch.Tensor | None,
     positions: torch.Tensor,
     token_item: torch.Tensor,
     block_table: torch.Tensor,
@@ -152,8 +161,9 @@ def qk_norm_rope_scatter(
     write_kv: bool = True,
     q_out: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Per-head q/k RMSNorm (when weights are given), rotary encoding (when ``inv_freq`` float32
-    [rotary_dim/2] is given), and the write of keys and values into their pages.
+    """Per-head q/k RMSNorm (when weights are given), rotary encoding (when ``rope``, the table of
+    :func:`rope_table`, is given; it must cover every position of the step), and the write of keys
+    and values into their pages.
 
     qkv [T, (nh + 2 nkv) d] (or [T, nh d] with ``write_kv`` off: q only); k_cache [pages, nkv, bs, d]; v_cache [pages, nkv, d, bs];
     block_table int32 [items, width]. Returns q [T, nh, d]."""
@@ -167,14 +177,14 @@ def qk_norm_rope_scatter(
         if w is not None:
             _want(w, name, torch.float32, (d,))
     rd = 0
-    if inv_freq is not None:
-        _want(inv_freq, "inv_freq", torch.float32, (None,))
-        rd = 2 * inv_freq.numel()
+    if rope is not None:
+        _want(rope, "rope", torch.float32, (None, 2, None))
+        rd = 2 * rope.shape[2]
     if q_out is None:
         q_out = torch.empty((t, nh, d), dtype=dtype, device=qkv.device)
     _want(q_out, "q_out", dtype, (t, nh, d))
     check(lib().me_qk_norm_rope_scatter(
-        _p(qkv), _p(q_weight), _p(k_weight), _p(inv_freq), _p(positions), _p(token_item), _p(block_table),
+        _p(qkv), _p(q_weight), _p(k_weight), _p(rope), _p(positions), _p(token_item), _p(block_table),
         _i(block_table.shape[1]), _p(q_out), _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(nkv), _i(d), _i(rd),
         _i(bs), _f(eps), _i(1 if write_kv else 0), _i(_code(dtype)), _stream()))
     return q_out

@@ -85,10 +85,10 @@ class Attention(Mixer):
         owns = s.cache_from is None
         proj = K.linear(h, self.w_qkv)  # [T, (nh + 2 nkv) d] or [T, nh d]
         table = batch.block_table(b.group)
-        inv_freq = None if self.position is None else self.position.tables()
+        rope = None if self.position is None else self.position.tables(batch.max_ctx)
         eps = 0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps)
         q = K.qk_norm_rope_scatter(
-            proj, self.q_norm_w, self.k_norm_w if owns else None, inv_freq, batch.positions, batch.token_item,
+            proj, self.q_norm_w, self.k_norm_w if owns else None, rope, batch.positions, batch.token_item,
             table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns)
         out = self.attend(q, batch, table, b)
         return K.linear(out, self.w_o)

@@ -201,7 +201,8 @@ def test_qk_norm_rope_scatter(dtype, nh, nkv, d, bs, rd, norm):
     inv_freq = (1.0 / (theta ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd))) if rd else None
     kc, vc = dev(k_cache.clone()), dev(v_cache.clone())
     q_out = K().qk_norm_rope_scatter(dev(qkv), dev(qw) if norm else None, dev(kw) if norm else None,
-                                     dev(inv_freq) if rd else None, dev(positions), dev(token_item), dev(table_t),
+                                     K().rope_table(dev(inv_freq), int(positions.max()) + 1) if rd else None, dev(positions),
+                                     dev(token_item), dev(table_t),
                                      kc, vc, nh, nkv, d, eps)
     f = qkv.float()
     q, k, v = (f[:, : nh * d].view(t, nh, d), f[:, nh * d : (nh + nkv) * d].view(t, nkv, d),

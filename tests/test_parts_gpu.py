@@ -61,7 +61,12 @@ def test_rotary_part_tables():
 
     rot = POSITION_ENCODINGS.build(RotarySpec(rotary_dim=32, theta=1e6), torch.float32, torch.device("cuda"))
     want = 1.0 / (1e6 ** (torch.arange(0, 32, 2, dtype=torch.float32) / 32))
-    assert torch.equal(rot.tables().cpu(), want)  # model.py:75, bit for bit
+    assert torch.equal(rot.inv_freq.cpu(), want)  # model.py:75, bit for bit
+    table = rot.tables(300).cpu()
+    assert table.shape[0] >= 300 and table.shape[1:] == (2, 16)
+    pos = torch.arange(table.shape[0], dtype=torch.float32)[:, None]
+    torch.testing.assert_close(table[:, 0], torch.cos(pos * want), rtol=0, atol=2e-6)  # model.py:81-83
+    torch.testing.assert_close(table[:, 1], torch.sin(pos * want), rtol=0, atol=2e-6)
     with pytest.raises(ValueError):
         POSITION_ENCODINGS.build(RotarySpec(rotary_dim=7, theta=1e4), torch.float32, torch.device("cuda"))
 
