@@ -128,12 +128,32 @@ __device__ __forceinline__ void attend_tile(const bf16_t* __restrict__ kbase, co
 
 // ------------------------------------------------------------------------------------- decode
 // Partial results: part_o [items, nh, splits, D] (unnormalised), part_ml [items, nh, splits, 2].
-template <int D>
+//
+// FUSED: the kernel starts from the raw output of the q/k/v projection, qkv [items, (nh + 2 nkv) D],
+// and does the per-head RMSNorm and the rotary encoding itself (what me_qk_norm_rope_scatter does
+// for steps with longer items), in float32 with one rounding at the end:
+//   * every block norms and rotates the query heads it owns, straight into matrix-core operands
+//     (a lane's eight dims of a 32-wide chunk and their rotary partners, half a head away, sit in
+//     the same lane when D is a multiple of 64);
+//   * the block whose split holds the item's newest position also norms and rotates the new key,
+//     writes it and the new value into their page, and waits for those stores before it reads that
+//     page. No other block of the step reads that slot.
+struct DecodeFusedArgs {
+  const float* q_w;         // [D] or null: no q/k norm
+  const float* k_w;         // [D] or null
+  const float* rope_table;  // [positions, 2, D/2] or null: no rotary
+  float eps;
+  int write_kv;             // 0: a layer that reads another layer's cache
+  bf16_t* k_cache_w;
+  bf16_t* v_cache_w;
+};
+
+template <int D, bool FUSED>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
     float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int bs_shift, int window,
-    float scale_log2, int split_keys, int num_splits, int head_chunks) {
+    float scale_log2, int split_keys, int num_splits, int head_chunks, DecodeFusedArgs fa) {
   const int bs = 1 << bs_shift;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
@@ -153,15 +173,103 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   for (int dt = 0; dt < D / 16; ++dt) acc[0][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
   if (begin < end) {
+    const int* table = block_table + (size_t)item * table_width;
     Frag8 qf[1][D / 32];
+    if (FUSED) {
+      constexpr int HC = D / 64;  // chunks per half head
+      const int pos = ctx - 1;
+      const size_t row = (size_t)item * (fa.write_kv ? nh + 2 * nkv : nh) * D;
+      // ---- the new key and value of this kv head, by the block that will read them
+      if (fa.write_kv && end == ctx) {
+        const int page = table[pos >> bs_shift];
+        if (page >= 0) {
+          const int slot = pos & (bs - 1);
+          const bf16_t* ksrc = q + row + (size_t)(nh + kvh) * D;
+          const bf16_t* vsrc = q + row + (size_t)(nh + nkv + kvh) * D;
+          float k1[(D / 2 + 63) / 64], k2[(D / 2 + 63) / 64];
+          float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < D / 32; ++c) {
-      qf[0][c].u = make_uint4(0, 0, 0, 0);
-      if (r < heads_here)
-        qf[0][c].u = *reinterpret_cast<const uint4*>(q + ((size_t)item * nh + head0 + r) * D + c * 32 + g * 8);
+          for (int p = 0; p < (D / 2 + 63) / 64; ++p) {
+            const int j = lane + 64 * p;
+            k1[p] = j < D / 2 ? to_float(ksrc[j]) : 0.f;
+            k2[p] = j < D / 2 ? to_float(ksrc[j + D / 2]) : 0.f;
+            ss += k1[p] * k1[p] + k2[p] * k2[p];
+          }
+          const float inv = fa.k_w ? rsqrtf(wave_sum(ss) / (float)D + fa.eps) : 1.f;
+          bf16_t* kdst = fa.k_cache_w + (((size_t)page * nkv + kvh) * bs + slot) * D;
+          bf16_t* vdst = fa.v_cache_w + ((size_t)page * nkv + kvh) * D * bs + slot;
+#pragma unroll
+          for (int p = 0; p < (D / 2 + 63) / 64; ++p) {
+            const int j = lane + 64 * p;
+            if (j < D / 2) {
+              float a = k1[p], b = k2[p];
+              if (fa.k_w) {
+                a = a * inv * fa.k_w[j];
+                b = b * inv * fa.k_w[j + D / 2];
+              }
+              if (fa.rope_table) {
+                const float c = fa.rope_table[(size_t)pos * D + j], sn = fa.rope_table[(size_t)pos * D + D / 2 + j];
+                const float ra = a * c - b * sn, rb = b * c + a * sn;
+                a = ra;
+                b = rb;
+              }
+              kdst[j] = from_float<bf16_t>(a);
+              kdst[j + D / 2] = from_float<bf16_t>(b);
+              vdst[(size_t)j * bs] = vsrc[j];
+              vdst[(size_t)(j + D / 2) * bs] = vsrc[j + D / 2];
+            }
+          }
+          __threadfence_block();  // the stores have landed before this wave reads the page below
+        }
+      }
+      // ---- this block's query heads: norm, rotate, round once, as matrix-core operands
+      float qv[D / 32][8];
+      float ss = 0.f;
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c) {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (r < heads_here) raw = *reinterpret_cast<const uint4*>(q + row + (size_t)(head0 + r) * D + c * 32 + g * 8);
+        const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          qv[c][2 * i] = __uint_as_float(w4[i] << 16);
+          qv[c][2 * i + 1] = __uint_as_float(w4[i] & 0xffff0000u);
+          ss += qv[c][2 * i] * qv[c][2 * i] + qv[c][2 * i + 1] * qv[c][2 * i + 1];
+        }
+      }
+      if (fa.q_w) {
+        const float inv = rsqrtf(column_sum(ss) / (float)D + fa.eps);
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) qv[c][i] = qv[c][i] * inv * fa.q_w[c * 32 + g * 8 + i];
+      }
+      if (fa.rope_table) {
+#pragma unroll
+        for (int c = 0; c < HC; ++c)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const int j = c * 32 + g * 8 + i;
+            const float cs = fa.rope_table[(size_t)pos * D + j], sn = fa.rope_table[(size_t)pos * D + D / 2 + j];
+            const float a = qv[c][i], b = qv[c + HC][i];
+            qv[c][i] = a * cs - b * sn;
+            qv[c + HC][i] = b * cs + a * sn;
+          }
+      }
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c) {
+        qf[0][c].h[0] = pack_bf16x4(qv[c][0], qv[c][1], qv[c][2], qv[c][3]);
+        qf[0][c].h[1] = pack_bf16x4(qv[c][4], qv[c][5], qv[c][6], qv[c][7]);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c) {
+        qf[0][c].u = make_uint4(0, 0, 0, 0);
+        if (r < heads_here)
+          qf[0][c].u = *reinterpret_cast<const uint4*>(q + ((size_t)item * nh + head0 + r) * D + c * 32 + g * 8);
+      }
     }
     const int qpos[1] = {ctx - 1};
-    const int* table = block_table + (size_t)item * table_width;
     for (int key0 = begin; key0 < end; key0 += 16) {
       int page = table[key0 >> bs_shift];
       page = page < 0 ? 0 : page;
@@ -253,13 +361,23 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
 template <int D>
 static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* item_ctx, const int* table,
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
-                          float scale_log2, int split_keys, int num_splits, hipStream_t stream) {
+                          float scale_log2, int split_keys, int num_splits, const DecodeFusedArgs* fused,
+                          hipStream_t stream) {
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits);
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-  attention_decode_kernel<D><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, nkv,
-                                                      bs_shift, window, scale_log2, split_keys, num_splits, chunks);
+  if constexpr (D % 64 == 0) {
+    if (fused) {
+      attention_decode_kernel<D, true><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh,
+                                                                nkv, bs_shift, window, scale_log2, split_keys,
+                                                                num_splits, chunks, *fused);
+      return;
+    }
+  }
+  attention_decode_kernel<D, false><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, nkv,
+                                                             bs_shift, window, scale_log2, split_keys, num_splits,
+                                                             chunks, DecodeFusedArgs{});
 }
 
 // Head sizes that are multiples of 32 (instantiated: 32, 64, 96, 128, 192, 256) and pages of a power
@@ -272,11 +390,55 @@ extern "C" int me_attention_mfma_supported(int d, int bs) {
 // workspace: part_o float [items * nh * num_splits * d], part_ml float [items * nh * num_splits * 2].
 // Split s covers keys [s * split_keys, (s+1) * split_keys); num_splits * split_keys must cover every
 // context the step can hold (max_ctx).
+static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
+                         const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
+                         int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
+                         int max_ctx, const DecodeFusedArgs* fused, hipStream_t stream);
+
 extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                                         const int* block_table, int table_width, void* out, float* part_o,
                                         float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
                                         float scale, int split_keys, int num_splits, int max_ctx,
                                         hipStream_t stream) {
+  return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
+                       bs, window, scale, split_keys, num_splits, max_ctx, nullptr, stream);
+}
+
+// Head sizes and groupings for which the decode kernel can take the norm, the rotary encoding and
+// the page write as its prologue: a multiple of 64, full-width rotary or none, at most 16 heads per
+// kv head.
+extern "C" int me_attention_decode_fused_supported(int d, int bs, int rotary_dim, int group) {
+  return me_attention_mfma_supported(d, bs) && d % 64 == 0 && (rotary_dim == 0 || rotary_dim == d) && group <= 16;
+}
+
+// As me_attention_decode_bf16, from the raw projection qkv [items, (nh + 2 nkv) d] (or [items, nh d]
+// with write_kv == 0). rope_table must cover position max_ctx - 1.
+extern "C" int me_attention_decode_fused_bf16(const void* qkv, const float* q_w, const float* k_w,
+                                              const float* rope_table, int rotary_dim, float eps, int write_kv,
+                                              void* k_cache, void* v_cache, const int* item_ctx,
+                                              const int* block_table, int table_width, void* out, float* part_o,
+                                              float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
+                                              float scale, int split_keys, int num_splits, int max_ctx,
+                                              hipStream_t stream) {
+  if (nkv <= 0 || nh <= 0 || nh % nkv || !me_attention_decode_fused_supported(d, bs, rope_table ? rotary_dim : 0, nh / nkv))
+    return me_fail("me_attention_decode_fused_bf16: head_dim=%d block_size=%d rotary_dim=%d heads=%d/%d not supported", d,
+                   bs, rotary_dim, nh, nkv);
+  DecodeFusedArgs fa;
+  fa.q_w = q_w;
+  fa.k_w = k_w;
+  fa.rope_table = rope_table;
+  fa.eps = eps;
+  fa.write_kv = write_kv;
+  fa.k_cache_w = (bf16_t*)k_cache;
+  fa.v_cache_w = (bf16_t*)v_cache;
+  return decode_common(qkv, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
+                       bs, window, scale, split_keys, num_splits, max_ctx, &fa, stream);
+}
+
+static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
+                         const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
+                         int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
+                         int max_ctx, const DecodeFusedArgs* fused, hipStream_t stream) {
   if (items <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_decode_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
@@ -292,7 +454,7 @@ extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, cons
 #define ME_DECODE_CASE(DD)                                                                                      \
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
-                      split_keys, num_splits, stream);                                                          \
+                      split_keys, num_splits, fused, stream);                                                   \
     break;
   switch (d) {
     ME_DECODE_CASE(32)

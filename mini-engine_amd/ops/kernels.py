@@ -422,6 +422,50 @@ def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: flo
     return out
 
 
+def attention_decode_fused_supported(head_dim: int, block_size: int, rotary_dim: int, group: int) -> bool:
+    """Whether the decode kernel can take q/k norm, rotary encoding and the page write as its prologue."""
+    return bool(lib().me_attention_decode_fused_supported(_i(head_dim), _i(block_size), _i(rotary_dim), _i(group)))
+
+
+def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write_kv: bool, k_cache, v_cache, item_ctx,
+                                block_table, num_heads: int, scale: float, window: int, max_ctx: int,
+                                out: torch.Tensor | None = None) -> torch.Tensor:
+    """One new token per item, from the raw q/k/v projection: what :func:`qk_norm_rope_scatter` followed
+    by :func:`attention_decode_bf16` compute, in one launch. qkv [items, (nh + 2 nkv) d] bfloat16
+    (or [items, nh d] with ``write_kv`` off)."""
+    nkv, bs, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    nh = num_heads
+    _want(qkv, "qkv", torch.bfloat16, (None, ((nh + 2 * nkv) if write_kv else nh) * d))
+    items = qkv.shape[0]
+    _check_cache(k_cache, v_cache, torch.bfloat16, nkv, d, bs)
+    _want(item_ctx, "item_ctx", torch.int32, (items,))
+    _want(block_table, "block_table", torch.int32, (items, None))
+    if block_table.shape[1] * bs < max_ctx:
+        raise ValueError(f"block table of {block_table.shape[1]} pages cannot hold {max_ctx} keys")
+    for w, name in ((q_weight, "q_weight"), (k_weight, "k_weight")):
+        if w is not None:
+            _want(w, name, torch.float32, (d,))
+    rd = 0
+    if rope is not None:
+        _want(rope, "rope", torch.float32, (None, 2, None))
+        rd = 2 * rope.shape[2]
+        if rope.shape[0] < max_ctx:
+            raise ValueError(f"the rotary table covers {rope.shape[0]} positions, the step may reach {max_ctx}")
+    chunks = -(-(nh // nkv) // 16)
+    split_keys, num_splits = decode_splits(items, nkv * chunks, max_ctx)
+    part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=qkv.device)
+    part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=qkv.device)
+    if out is None:
+        out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=qkv.device)
+    _want(out, "out", torch.bfloat16, (items, nh * d))
+    check(lib().me_attention_decode_fused_bf16(
+        _p(qkv), _p(q_weight), _p(k_weight), _p(rope), _i(rd), _f(eps), _i(1 if write_kv else 0), _p(k_cache),
+        _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out), _p(part_o), _p(part_ml),
+        _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys), _i(num_splits), _i(max_ctx),
+        _stream()))
+    return out
+
+
 def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: list[int], block_table, scale: float,
                            window: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention of packed new tokens q [T, nh, d] bfloat16 over the paged cache (which already

@@ -87,6 +87,13 @@ class Attention(Mixer):
         table = batch.block_table(b.group)
         rope = None if self.position is None else self.position.tables(batch.max_ctx)
         eps = 0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps)
+        if (self.dtype is torch.bfloat16 and batch.decode_only and K.attention_decode_fused_supported(
+                self.d, b.block_size, 0 if rope is None else 2 * rope.shape[2], self.nh // self.nkv)):
+            # one new token per item: norm, rotary, page write and attention in one launch
+            out = K.attention_decode_fused_bf16(
+                proj, self.q_norm_w, self.k_norm_w if owns else None, rope, eps, owns, b.k_cache, b.v_cache,
+                batch.item_ctx, table, self.nh, float(s.scale), int(s.window), batch.max_ctx)
+            return K.linear(out, self.w_o)
         q = K.qk_norm_rope_scatter(
             proj, self.q_norm_w, self.k_norm_w if owns else None, rope, batch.positions, batch.token_item,
             table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns)

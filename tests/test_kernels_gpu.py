@@ -401,6 +401,35 @@ def test_attention_prefill_mfma(nh, nkv, d, bs, window):
     torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs", [(4, 2, 64, 16), (16, 8, 128, 16), (6, 1, 128, 32), (2, 2, 256, 16)])
+@pytest.mark.parametrize("norm,rotary,window", [(True, True, 0), (False, True, 37), (True, False, 0)])
+def test_attention_decode_fused_equals_the_two_kernels(nh, nkv, d, bs, norm, rotary, window):
+    """The decode kernel with the norm / rotary / page-write prologue against qk_norm_rope_scatter
+    followed by the plain decode kernel: same cache contents, same output."""
+    dtype = torch.bfloat16
+    ctxs = [1, 16, 17, 33, 100, 255, 64, 65, 700]
+    items = [(c - 1, 1) for c in ctxs]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=160)
+    assert K().attention_decode_fused_supported(d, bs, d if rotary else 0, nh // nkv)
+    g = torch.Generator().manual_seed(2)
+    qkv = torch.randn(len(items), (nh + 2 * nkv) * d, generator=g).to(dtype)
+    qw, kw = (dev(1 + 0.2 * torch.randn(d, generator=g)), dev(1 + 0.2 * torch.randn(d, generator=g))) if norm else (None, None)
+    inv_freq = 1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    rope = K().rope_table(dev(inv_freq), 4096) if rotary else None
+    item_ctx, scale = dev(torch.tensor(ctxs, dtype=torch.int32)), d**-0.5
+    wide = torch.zeros(len(items), 4096 // bs, dtype=torch.int32)
+    wide[:, : table_t.shape[1]] = table_t
+    kc1, vc1, kc2, vc2 = dev(k_cache.clone()), dev(v_cache.clone()), dev(k_cache.clone()), dev(v_cache.clone())
+    q = K().qk_norm_rope_scatter(dev(qkv), qw, kw, rope, dev(positions), dev(token_item), dev(wide), kc1, vc1, nh, nkv, d, 1e-5)
+    want = K().attention_decode_bf16(q, kc1, vc1, item_ctx, dev(wide), scale, window, 4096)
+    got = K().attention_decode_fused_bf16(dev(qkv), qw, kw, rope, 1e-5, True, kc2, vc2, item_ctx, dev(wide), nh, scale,
+                                          window, 4096)
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2)
+    assert not K().attention_decode_fused_supported(96, 16, 96, 1)
+    assert not K().attention_decode_fused_supported(128, 16, 64, 1)
+
+
 @pytest.mark.parametrize("kernel", ["decode", "prefill"])
 def test_mfma_attention_finds_one_far_key_and_respects_the_window_edge(kernel):
     dtype, nh, nkv, d, bs, ctx = torch.bfloat16, 4, 2, 64, 16, 600
