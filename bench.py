@@ -72,12 +72,20 @@ def main() -> int:
     max_batch = max([args.batch] + points)
     block = 16
     ctx, k, w = args.context, args.steps, args.warmup
-    prompt_len = ctx - (k + w) - 1
-    if prompt_len < 1:
-        raise SystemExit("context is too short for this many steps")
+    budget = 8192
+
+    def prompt_len_for(batch):
+        """Prompts are sized so that every sequence is still decoding, and within the context
+        length, when the timed steps end: the first sequences decode while the later ones are still
+        being prefilled under the token budget."""
+        prefill_steps = 0 if args.zero_context else -(-batch * ctx // budget) + 1
+        n = ctx - (k + w + prefill_steps) - 2
+        if n < 1:
+            raise SystemExit("context is too short for this many steps")
+        return n, prefill_steps
     blocks_per_seq = -(-ctx // block)
     econf = EngineConfig(block_size=block, num_blocks=max_batch * blocks_per_seq + 256, max_num_seqs=max_batch,
-                         max_num_batched_tokens=8192, max_model_len=ctx, enable_prefix_caching=False,
+                         max_num_batched_tokens=budget, max_model_len=ctx, enable_prefix_caching=False,
                          dtype=args.dtype, seed=0, cuda_graphs=True)
     engine = LLMEngine.from_random("Qwen3ForCausalLM", cfg, econf, seed=0)
     gen = torch.Generator().manual_seed(0)
@@ -110,7 +118,8 @@ def main() -> int:
     weight_bytes = engine.model.weight_bytes()
 
     def decode(batch):
-        params = SamplingParams(max_tokens=k + w + 1, temperature=0.0, ignore_eos=True)
+        prompt_len, prefill_steps = prompt_len_for(batch)
+        params = SamplingParams(max_tokens=k + w + prefill_steps + 2, temperature=0.0, ignore_eos=True)
         seqs = [engine.add_request(prompt(prompt_len), params) for _ in range(batch)]
         if args.zero_context:
             from mini_engine_amd.engine.sequence import SequenceStatus
@@ -125,18 +134,22 @@ def main() -> int:
         for _ in range(w - 1):
             engine.step()
         torch.cuda.synchronize()
-        ctx_before = sum(len(s) for s in seqs) / batch
+        tokens_before = sum(len(s) for s in seqs)
         t0 = time.perf_counter()
         for _ in range(k):
             engine.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        ctx_after = sum(len(s) for s in seqs) / batch
+        tokens_after = sum(len(s) for s in seqs)
+        live = sum(not s.is_finished for s in seqs)
+        if live != batch or tokens_after - tokens_before != batch * k:
+            raise SystemExit(f"batch {batch}: only {live} sequences were decoding through the timed steps "
+                             f"({tokens_after - tokens_before} tokens instead of {batch * k})")
         while engine.scheduler.has_unfinished():
             engine.step()
         ms = dt / k * 1e3
-        step_bytes = weight_bytes + batch * (ctx_before + ctx_after) / 2 * kv_per_token
-        return batch * k / dt, ms, step_bytes / (dt / k) / 1e9
+        step_bytes = weight_bytes + (tokens_before + tokens_after) / 2 * kv_per_token
+        return (tokens_after - tokens_before) / dt, ms, step_bytes / (dt / k) / 1e9
 
     tok_s, ms_per_step, gbs = decode(args.batch)
     pts = {f"decode_b{b}": round(decode(b)[0], 1) for b in points}

@@ -260,12 +260,13 @@ class NormedInput:
         return self._tensor
 
     def fusable(self, weight: torch.Tensor) -> bool:
-        return (self.dtype is torch.bfloat16 and self._tensor is None and self.x.shape[0] <= SMALL_MAX_ROWS
+        return (self.dtype is torch.bfloat16 and self._tensor is None and self.x.shape[0] <= SMALL_FAST_ROWS
                 and self.x.shape[1] % 8 == 0 and (self.delta is None or self.spare is not None)
                 and weight.dtype is torch.bfloat16)
 
 
-SMALL_MAX_ROWS = 64
+SMALL_MAX_ROWS = 64  # what the kernel accepts
+SMALL_FAST_ROWS = 16  # up to here it beats the GEMM library (one 16-row tile: the weights stream once, x is tiny)
 
 
 def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
@@ -316,8 +317,8 @@ def gemm_bf16_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
     return gemm_bf16_small(x, weight, out_dtype, False, out)
 
 
-def small_ok(x, weight: torch.Tensor) -> bool:
-    return (x.shape[0] <= SMALL_MAX_ROWS and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
+def small_ok(x, weight: torch.Tensor, max_rows: int = SMALL_FAST_ROWS) -> bool:
+    return (x.shape[0] <= max_rows and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
             and weight.data_ptr() % 16 == 0)
 
 
@@ -342,11 +343,8 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if gated:
         return swiglu(linear(x, weight, out_dtype))
-    if out_dtype is torch.float32 and x.shape[1] % 8 == 0:
-        out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
-        for lo in range(0, x.shape[0], SMALL_MAX_ROWS):
-            gemm_bf16_small(x[lo:lo + SMALL_MAX_ROWS], weight, torch.float32, False, out[lo:lo + SMALL_MAX_ROWS])
-        return out
+    if out_dtype is torch.float32 and small_ok(x, weight, SMALL_MAX_ROWS):
+        return gemm_bf16_small(x, weight, torch.float32, False)  # float32 logits of a few rows, unrounded
     y = torch.matmul(x, weight.t())
     return y if out_dtype is y.dtype else y.to(out_dtype)
 
