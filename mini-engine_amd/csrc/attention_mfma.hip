@@ -64,32 +64,42 @@ __device__ __forceinline__ float column_sum(float v) {
 
 #define LOG2E 1.4426950408889634f
 
-// One 16-key tile for NB blocks of 16 query columns. `kbase` points at K[page, kvh, off, 0], `vbase`
-// at V^T[page, kvh, 0, off]. key0 is the absolute position of the tile's first key. A key is
-// visible to column nb if lo <= key <= qpos[nb].
-template <int D, int NB>
-__device__ __forceinline__ void attend_tile(const bf16_t* __restrict__ kbase, const bf16_t* __restrict__ vbase,
-                                            int bs, int key0, int lo, const int (&qpos)[NB], bool need_mask,
-                                            const Frag8 (&qf)[NB][D / 32], float scale_log2,
-                                            float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16]) {
+// One 16-key tile for NB blocks of 16 query columns, in two halves so that a caller can have the
+// loads of the next tile in flight while it computes on this one. `kbase` points at
+// K[page, kvh, off, 0], `vbase` at V^T[page, kvh, 0, off]. key0 is the absolute position of the tile's
+// first key. A key is visible to column nb if lo <= key <= qpos[nb].
+template <int D>
+struct KvTile {
+  Frag8 kf[D / 32];
+  short4_t vf[D / 16];
+};
+
+template <int D>
+__device__ __forceinline__ void load_tile(KvTile<D>& t, const bf16_t* __restrict__ kbase,
+                                          const bf16_t* __restrict__ vbase, int bs) {
   const int lane = threadIdx.x & (ME_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  Frag8 kf[D / 32];
 #pragma unroll
-  for (int c = 0; c < D / 32; ++c) kf[c].u = *reinterpret_cast<const uint4*>(kbase + (size_t)r * D + c * 32 + g * 8);
-  short4_t vf[D / 16];
+  for (int c = 0; c < D / 32; ++c) t.kf[c].u = *reinterpret_cast<const uint4*>(kbase + (size_t)r * D + c * 32 + g * 8);
 #pragma unroll
   for (int dt = 0; dt < D / 16; ++dt)
-    vf[dt] = *reinterpret_cast<const short4_t*>(vbase + (size_t)(dt * 16 + r) * bs + g * 4);
+    t.vf[dt] = *reinterpret_cast<const short4_t*>(vbase + (size_t)(dt * 16 + r) * bs + g * 4);
+}
 
+template <int D, int NB>
+__device__ __forceinline__ void compute_tile(const KvTile<D>& t, int key0, int lo, const int (&qpos)[NB],
+                                             bool need_mask, const Frag8 (&qf)[NB][D / 32], float scale_log2,
+                                             float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16]) {
+  const int lane = threadIdx.x & (ME_WAVE - 1);
+  const int g = lane >> 4;
   short4_t pf[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     float4_t s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) {
-      s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[c].h[0], qf[nb][c].h[0], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[c].h[1], qf[nb][c].h[1], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.kf[c].h[0], qf[nb][c].h[0], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.kf[c].h[1], qf[nb][c].h[1], s, 0, 0, 0);
     }
     float sv[4];
 #pragma unroll
@@ -123,7 +133,7 @@ __device__ __forceinline__ void attend_tile(const bf16_t* __restrict__ kbase, co
   for (int dt = 0; dt < D / 16; ++dt)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
-      acc[nb][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[dt], pf[nb], acc[nb][dt], 0, 0, 0);
+      acc[nb][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.vf[dt], pf[nb], acc[nb][dt], 0, 0, 0);
 }
 
 // ------------------------------------------------------------------------------------- decode
@@ -174,6 +184,19 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 
   if (begin < end) {
     const int* table = block_table + (size_t)item * table_width;
+    // two tiles in flight: the loads of tile i+1 are issued before the products of tile i
+    auto fetch = [&](KvTile<D>& t, int key0) {
+      int page = table[min(key0 >> bs_shift, table_width - 1)];
+      page = page < 0 ? 0 : page;
+      const int off = key0 & (bs - 1);
+      load_tile<D>(t, k_cache + (((size_t)page * nkv + kvh) * bs + off) * D,
+                   v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
+    };
+    KvTile<D> ta, tb;
+    // the first tile is requested before the query is prepared, unless it holds the slot that this
+    // block is about to write
+    const bool early = !FUSED || begin + 16 < ctx;
+    if (early) fetch(ta, begin);
     Frag8 qf[1][D / 32];
     if (FUSED) {
       constexpr int HC = D / 64;  // chunks per half head
@@ -270,14 +293,13 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
       }
     }
     const int qpos[1] = {ctx - 1};
-    for (int key0 = begin; key0 < end; key0 += 16) {
-      int page = table[key0 >> bs_shift];
-      page = page < 0 ? 0 : page;
-      const int off = key0 & (bs - 1);
-      const bf16_t* kbase = k_cache + (((size_t)page * nkv + kvh) * bs + off) * D;
-      const bf16_t* vbase = v_cache + ((size_t)page * nkv + kvh) * D * bs + off;
-      const bool need_mask = key0 < lo || key0 + 16 > ctx;
-      attend_tile<D, 1>(kbase, vbase, bs, key0, lo, qpos, need_mask, qf, scale_log2, m, lsum, acc);
+    if (!early) fetch(ta, begin);
+    for (int key0 = begin; key0 < end; key0 += 32) {
+      fetch(tb, key0 + 16);  // may lie past `end`: a valid page, computed on only if it is in range
+      compute_tile<D, 1>(ta, key0, lo, qpos, key0 < lo || key0 + 16 > ctx, qf, scale_log2, m, lsum, acc);
+      fetch(ta, key0 + 32);
+      if (key0 + 16 < end)
+        compute_tile<D, 1>(tb, key0 + 16, lo, qpos, key0 + 16 < lo || key0 + 32 > ctx, qf, scale_log2, m, lsum, acc);
     }
   }
   if (r < heads_here) {

@@ -114,8 +114,8 @@ def test_gemm_bf16_small_with_norm_prologue_and_swiglu_epilogue(m, n, k, with_de
     w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
     xd, spare = dev(x.clone()), dev(torch.full((m, k), 7.0))
     h = K().NormedInput(xd, None if delta is None else dev(delta), dev(wn), 1e-5, torch.bfloat16, spare)
-    assert h.fusable(dev(w))
-    out = K().linear(h, dev(w), gated=gated).float().cpu()
+    assert h.fusable(dev(w)) == (m <= K().SMALL_FAST_ROWS)  # linear() fuses up to there; the kernel takes 64 rows
+    out = K().gemm_bf16_small(h, dev(w), torch.bfloat16, gated).float().cpu()
     s = x + (delta.float() if with_delta else 0)
     y = plain.rms_norm(s, wn, 1e-5) @ w.float().T
     want = plain.silu(y[:, :n]) * y[:, n:] if gated else y
