@@ -158,7 +158,7 @@ struct DecodeFusedArgs {
   bf16_t* v_cache_w;
 };
 
-template <int D, bool FUSED>
+template <int D, bool FUSED, bool PIPE>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
@@ -294,12 +294,21 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     }
     const int qpos[1] = {ctx - 1};
     if (!early) fetch(ta, begin);
-    for (int key0 = begin; key0 < end; key0 += 32) {
-      fetch(tb, key0 + 16);  // may lie past `end`: a valid page, computed on only if it is in range
-      compute_tile<D, 1>(ta, key0, lo, qpos, key0 < lo || key0 + 16 > ctx, qf, scale_log2, m, lsum, acc);
-      fetch(ta, key0 + 32);
-      if (key0 + 16 < end)
-        compute_tile<D, 1>(tb, key0 + 16, lo, qpos, key0 + 16 < lo || key0 + 32 > ctx, qf, scale_log2, m, lsum, acc);
+    if (PIPE) {
+      // short splits (few waves, each waiting on memory): keep two tiles in flight per wave
+      for (int key0 = begin; key0 < end; key0 += 32) {
+        fetch(tb, key0 + 16);  // may lie past `end`: a valid page, computed on only if it is in range
+        compute_tile<D, 1>(ta, key0, lo, qpos, key0 < lo || key0 + 16 > ctx, qf, scale_log2, m, lsum, acc);
+        fetch(ta, key0 + 32);
+        if (key0 + 16 < end)
+          compute_tile<D, 1>(tb, key0 + 16, lo, qpos, key0 + 16 < lo || key0 + 32 > ctx, qf, scale_log2, m, lsum, acc);
+      }
+    } else {
+      // long splits (the chip is full of waves): fewer registers, one more wave per SIMD
+      for (int key0 = begin; key0 < end; key0 += 16) {
+        if (key0 > begin) fetch(ta, key0);
+        compute_tile<D, 1>(ta, key0, lo, qpos, key0 < lo || key0 + 16 > ctx, qf, scale_log2, m, lsum, acc);
+      }
     }
   }
   if (r < heads_here) {
@@ -389,17 +398,25 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
   dim3 grid(items, nkv * chunks, num_splits);
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
+  const bool pipe = split_keys <= 256;
+#define ME_DECODE_LAUNCH(FUSED, PIPE, ARGS)                                                                          \
+  attention_decode_kernel<D, FUSED, PIPE><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
+                                                                   nkv, bs_shift, window, scale_log2, split_keys,     \
+                                                                   num_splits, chunks, ARGS)
   if constexpr (D % 64 == 0) {
     if (fused) {
-      attention_decode_kernel<D, true><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh,
-                                                                nkv, bs_shift, window, scale_log2, split_keys,
-                                                                num_splits, chunks, *fused);
+      if (pipe)
+        ME_DECODE_LAUNCH(true, true, *fused);
+      else
+        ME_DECODE_LAUNCH(true, false, *fused);
       return;
     }
   }
-  attention_decode_kernel<D, false><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, nkv,
-                                                             bs_shift, window, scale_log2, split_keys, num_splits,
-                                                             chunks, DecodeFusedArgs{});
+  if (pipe)
+    ME_DECODE_LAUNCH(false, true, DecodeFusedArgs{});
+  else
+    ME_DECODE_LAUNCH(false, false, DecodeFusedArgs{});
+#undef ME_DECODE_LAUNCH
 }
 
 // Head sizes that are multiples of 32 (instantiated: 32, 64, 96, 128, 192, 256) and pages of a power

@@ -343,8 +343,12 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if gated:
         return swiglu(linear(x, weight, out_dtype))
-    if out_dtype is torch.float32 and small_ok(x, weight, SMALL_MAX_ROWS):
-        return gemm_bf16_small(x, weight, torch.float32, False)  # float32 logits of a few rows, unrounded
+    if out_dtype is torch.float32:
+        try:
+            return torch.mm(x, weight.t(), out_dtype=torch.float32)  # float32 logits, not rounded to bfloat16
+        except (TypeError, RuntimeError):
+            if small_ok(x, weight, SMALL_MAX_ROWS):
+                return gemm_bf16_small(x, weight, torch.float32, False)
     y = torch.matmul(x, weight.t())
     return y if out_dtype is y.dtype else y.to(out_dtype)
 
