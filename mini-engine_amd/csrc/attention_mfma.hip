@@ -510,10 +510,13 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
 }
 
 // ------------------------------------------------------------------------------------ prefill
-// Block = 4 waves; a block owns the query columns of `tokens_per_block = 128 / group` consecutive
+// A block owns the query columns of `tokens_per_block = columns / group` consecutive
 // new tokens of one item for one kv head (column c -> token c / group, head c % group); wave w owns
-// columns 32w .. 32w+31 as two blocks of 16. Blocks are numbered over all items: item i has
-// ceil(qlen_i / tokens_per_block) of them, the later (longer) tiles of an item first.
+// NB blocks of 16 columns. Measured on 2,048-token prompts of the 0.6B shape: 8 waves x 1 block of
+// columns (128 columns a block) beats 4 x 2 (register pressure pushes the accumulators out of the
+// vector registers) and 4 x 1 (64 columns a block, twice the LDS traffic per product). Blocks are
+// numbered over all items: item i has ceil(qlen_i / tokens_per_block) of them, the later (longer)
+// tiles of an item first.
 //
 // Keys and values are staged through LDS in tiles of 64 keys, double-buffered: while the waves
 // multiply tile i out of one buffer, the global loads of tile i+1 are in flight and are written to
@@ -681,7 +684,6 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
     int window, float scale_log2, int tokens_per_block) {
   constexpr int THREADS = WAVES * 64;
-  static_assert(WAVES * NB * 16 == 128, "a block owns 128 query columns");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
   using L = PrefillLds<D>;
@@ -800,6 +802,9 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
 
 #define PF_NB 1
 #define PF_WAVES 8
+#define PF_COLUMNS (PF_NB * PF_WAVES * 16)  // query columns (token, head of the group) per block
+
+extern "C" int me_attention_prefill_columns() { return PF_COLUMNS; }
 
 template <int D>
 static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* positions,
@@ -819,7 +824,7 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
 }
 
 // q [T, nh, d]; item_start int [items + 1] (offsets of the items' tokens); positions int [T];
-// num_blocks = sum over items of ceil(qlen / (128 / group)), computed by the caller.
+// num_blocks = sum over items of ceil(qlen / (me_attention_prefill_columns() / group)), computed by the caller.
 extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, const int* positions,
                                          const int* item_start, int num_items, const int* block_table, int table_width,
                                          void* out, int num_blocks, int nh, int nkv, int d, int bs, int window,
@@ -832,7 +837,7 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   if (group > 16) return me_fail("me_attention_prefill_bf16: group size %d exceeds 16", group);
   if (nkv > 65535) return me_fail("me_attention_prefill_bf16: %d kv heads exceed the grid", nkv);
   if (table_width <= 0) return me_fail("me_attention_prefill_bf16: empty block table");
-  const int tpb = 128 / group;
+  const int tpb = PF_COLUMNS / group;
   const float sl = scale * LOG2E;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;

@@ -347,8 +347,11 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         try:
             return torch.mm(x, weight.t(), out_dtype=torch.float32)  # float32 logits, not rounded to bfloat16
         except (TypeError, RuntimeError):
-            if small_ok(x, weight, SMALL_MAX_ROWS):
-                return gemm_bf16_small(x, weight, torch.float32, False)
+            if x.shape[1] % 8 == 0:  # slices of 64 rows through the matrix-core kernel
+                out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
+                for lo in range(0, x.shape[0], SMALL_MAX_ROWS):
+                    gemm_bf16_small(x[lo:lo + SMALL_MAX_ROWS], weight, torch.float32, False, out[lo:lo + SMALL_MAX_ROWS])
+                return out
     y = torch.matmul(x, weight.t())
     return y if out_dtype is y.dtype else y.to(out_dtype)
 
@@ -486,7 +489,7 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
     group = nh // nkv
     if group > 16:
         raise ValueError(f"group size {group} exceeds what the matrix-core prefill kernel takes (16)")
-    tpb = 128 // group
+    tpb = lib().me_attention_prefill_columns() // group
     num_blocks = sum(-(-n // tpb) for n in qlens)
     if out is None:
         out = torch.empty((t, nh * d), dtype=torch.bfloat16, device=q.device)
