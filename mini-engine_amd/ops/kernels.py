@@ -389,7 +389,7 @@ def attention_mfma_supported(head_dim: int, block_size: int, group: int = 1) -> 
     return bool(lib().me_attention_mfma_supported(_i(head_dim), _i(block_size))) and group <= 16
 
 
-def decode_splits(items: int, kv_units: int, max_ctx: int, target_waves: int = 2048) -> tuple[int, int]:
+def decode_splits(items: int, kv_units: int, max_ctx: int, target_waves: int = 1024) -> tuple[int, int]:
     """(keys per split, number of splits) for the decode kernel: enough waves to fill the chip,
     splits of at least 64 keys, boundaries at multiples of 64."""
     want = max(1, target_waves // max(1, items * kv_units))
