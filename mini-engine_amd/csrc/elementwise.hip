@@ -190,12 +190,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
     const float* __restrict__ rope_table, const int* __restrict__ positions, const int* __restrict__ token_item,
     const int* __restrict__ block_table, int table_width, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, int nh, int nkv, int d, int rd, int bs, float eps, int write_kv, int heads_per_block) {
+    T* __restrict__ v_cache, int nh, int nkv, int d, int rd, int bs, float eps, int write_kv, int heads_per_block,
+    int skip_v) {
   __shared__ float stage[4][ME_MAX_HEAD_DIM];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int t = blockIdx.x;
-  const int heads_total = write_kv ? nh + 2 * nkv : nh;
-  const int width = heads_total * d;  // q-only rows when nothing is written
+  const int heads_row = write_kv ? nh + 2 * nkv : nh;
+  const int heads_total = skip_v ? nh + nkv : heads_row;  // value heads are written by the page-tile kernel
+  const int width = heads_row * d;  // q-only rows when nothing is written
   const int pos = positions[t];
   const int half = rd / 2;
   const float* cs = rope_table ? rope_table + (size_t)pos * rd : nullptr;  // [2, half] of this position
@@ -274,31 +276,196 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
   }
 }
 
+// The same work for the common geometry (head size a power of two from 16 to 256, rotary over the
+// whole head or none): a lane owns the four dims (2p, 2p+1, 2p+d/2, 2p+1+d/2), i.e. two rotary pairs,
+// so no value has to cross lanes for the rotation, loads and stores are 4 bytes wide, and a wave
+// handles 64 / (d/4) heads at a time. Unit u of the grid is (token, head) = (u / heads, u % heads).
+template <typename T>
+struct Pair2 {
+  T a, b;
+};
+
+template <typename T, int LPH>  // LPH = d / 4 lanes per head
+__global__ __launch_bounds__(256) void qk_norm_rope_scatter_quad_kernel(
+    const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    const float* __restrict__ rope_table, const int* __restrict__ positions, const int* __restrict__ token_item,
+    const int* __restrict__ block_table, int table_width, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, int num_tokens, int nh, int nkv, int bs, float eps, int write_kv, int skip_v) {
+  constexpr int D = LPH * 4, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
+  const int lane = threadIdx.x & (ME_WAVE - 1);
+  const int sub = lane / LPH, p = lane % LPH;
+  const int heads_row = write_kv ? nh + 2 * nkv : nh;
+  const int heads = skip_v ? nh + nkv : heads_row;
+  const long long unit = ((long long)blockIdx.x * (blockDim.x / ME_WAVE) + threadIdx.x / ME_WAVE) * HPW + sub;
+  if (unit >= (long long)num_tokens * heads) return;
+  const int t = (int)(unit / heads), hd = (int)(unit % heads);
+  const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
+  const T* src = qkv + ((size_t)t * heads_row + hd) * D;
+  const Pair2<T> lo = *reinterpret_cast<const Pair2<T>*>(src + 2 * p);
+  const Pair2<T> hi = *reinterpret_cast<const Pair2<T>*>(src + 2 * p + HALF);
+  float v[4] = {to_float(lo.a), to_float(lo.b), to_float(hi.a), to_float(hi.b)};
+  const int pos = positions[t];
+  const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
+  if (w) {
+    float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, ME_WAVE);  // within the head's lanes
+    const float inv = rsqrtf(ss / (float)D + eps);
+    v[0] *= inv * w[2 * p];
+    v[1] *= inv * w[2 * p + 1];
+    v[2] *= inv * w[2 * p + HALF];
+    v[3] *= inv * w[2 * p + 1 + HALF];
+  }
+  if (kind != 2 && rope_table) {
+    const float* cs = rope_table + (size_t)pos * D;  // [2, HALF]: cosines then sines
+    const float c0 = cs[2 * p], c1 = cs[2 * p + 1], s0 = cs[HALF + 2 * p], s1 = cs[HALF + 2 * p + 1];
+    const float a0 = v[0] * c0 - v[2] * s0, b0 = v[2] * c0 + v[0] * s0;
+    const float a1 = v[1] * c1 - v[3] * s1, b1 = v[3] * c1 + v[1] * s1;
+    v[0] = a0;
+    v[1] = a1;
+    v[2] = b0;
+    v[3] = b1;
+  }
+  const Pair2<T> out_lo = {from_float<T>(v[0]), from_float<T>(v[1])}, out_hi = {from_float<T>(v[2]), from_float<T>(v[3])};
+  if (kind == 0) {
+    T* dst = q_out + ((size_t)t * nh + hd) * D;
+    *reinterpret_cast<Pair2<T>*>(dst + 2 * p) = out_lo;
+    *reinterpret_cast<Pair2<T>*>(dst + 2 * p + HALF) = out_hi;
+    return;
+  }
+  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs];
+  if (page < 0) return;
+  const int slot = pos % bs;
+  if (kind == 1) {
+    T* dst = k_cache + (((size_t)page * nkv + (hd - nh)) * bs + slot) * D;
+    *reinterpret_cast<Pair2<T>*>(dst + 2 * p) = out_lo;
+    *reinterpret_cast<Pair2<T>*>(dst + 2 * p + HALF) = out_hi;
+  } else {
+    T* dst = v_cache + ((size_t)page * nkv + (hd - nh - nkv)) * D * bs + slot;
+    dst[(size_t)(2 * p) * bs] = out_lo.a;
+    dst[(size_t)(2 * p + 1) * bs] = out_lo.b;
+    dst[(size_t)(2 * p + HALF) * bs] = out_hi.a;
+    dst[(size_t)(2 * p + 1 + HALF) * bs] = out_hi.b;
+  }
+}
+
+template <typename T>
+static bool launch_quad(const T* qkv, const float* q_w, const float* k_w, const float* rope_table, const int* positions,
+                        const int* token_item, const int* block_table, int table_width, T* q_out, T* k_cache,
+                        T* v_cache, int num_tokens, int nh, int nkv, int d, int bs, float eps, int write_kv, int skip_v,
+                        hipStream_t stream) {
+  const int heads = write_kv ? (skip_v ? nh + nkv : nh + 2 * nkv) : nh;
+  const long long units = (long long)num_tokens * heads;
+#define ME_QUAD(LPH)                                                                                                  \
+  {                                                                                                                   \
+    const long long per_block = 4 * (64 / LPH);                                                                       \
+    qk_norm_rope_scatter_quad_kernel<T, LPH><<<(unsigned)((units + per_block - 1) / per_block), 256, 0, stream>>>(    \
+        qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, q_out, k_cache, v_cache,          \
+        num_tokens, nh, nkv, bs, eps, write_kv, skip_v);                                                              \
+    return true;                                                                                                      \
+  }
+  switch (d) {
+    case 16: ME_QUAD(4)
+    case 32: ME_QUAD(8)
+    case 64: ME_QUAD(16)
+    case 128: ME_QUAD(32)
+    case 256: ME_QUAD(64)
+  }
+#undef ME_QUAD
+  return false;
+}
+
+// Values of many consecutive tokens: one block per (16-slot segment of a page that the step's tokens
+// touch, kv head). The segment's tokens are read row by row into LDS and written transposed, 16 slots
+// (32 bytes) per head dimension, instead of one 2-byte store per (token, dimension). Segments are
+// numbered over all items; item i touches segments pos0/16 .. (pos0 + qlen - 1)/16 of its positions.
+template <typename T>
+__global__ __launch_bounds__(256) void v_scatter_tiles_kernel(const T* __restrict__ qkv, const int* __restrict__ positions,
+                                                              const int* __restrict__ item_start, int num_items,
+                                                              const int* __restrict__ block_table, int table_width,
+                                                              T* __restrict__ v_cache, int nh, int nkv, int d, int bs) {
+  __shared__ T tile[16][ME_MAX_HEAD_DIM + 2];
+  __shared__ int s_item, s_seg;
+  if (threadIdx.x == 0) {
+    int left = blockIdx.x, it = 0;
+    for (; it < num_items; ++it) {
+      const int p0 = positions[item_start[it]], n = item_start[it + 1] - item_start[it];
+      const int segs = (p0 + n - 1) / 16 - p0 / 16 + 1;
+      if (left < segs) break;
+      left -= segs;
+    }
+    s_item = it;
+    s_seg = left;
+  }
+  __syncthreads();
+  const int item = s_item;
+  if (item >= num_items) return;
+  const int kvh = blockIdx.y;
+  const int t0 = item_start[item], n = item_start[item + 1] - t0;
+  const int p0 = positions[t0];
+  const int seg_pos = (p0 / 16 + s_seg) * 16;           // first position of the segment
+  const int first = max(seg_pos, p0), last = min(seg_pos + 15, p0 + n - 1);  // positions present
+  const int width = (nh + 2 * nkv) * d;
+  const T* src = qkv + (size_t)(nh + nkv + kvh) * d;
+  for (int idx = threadIdx.x; idx < (last - first + 1) * d; idx += blockDim.x) {
+    const int row = idx / d, col = idx % d;
+    tile[first - seg_pos + row][col] = src[(size_t)(t0 + first - p0 + row) * width + col];
+  }
+  __syncthreads();
+  const int page = block_table[(size_t)item * table_width + seg_pos / bs];
+  if (page < 0) return;
+  T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + seg_pos % bs;
+  const int lo = first - seg_pos, hi = last - seg_pos;
+  for (int idx = threadIdx.x; idx < d * 16; idx += blockDim.x) {
+    const int dim = idx / 16, slot = idx % 16;
+    if (slot >= lo && slot <= hi) dst[(size_t)dim * bs + slot] = tile[slot][dim];
+  }
+}
+
 // rope_table: float32 [num_positions, 2, rd / 2] or null; every position of the step must be below
 // num_positions (checked by the caller against the engine's length limit).
+// item_start / num_items / num_segments: when given (num_segments > 0), the values are written by the
+// page-tile kernel; num_segments is the sum over items of (pos0 + qlen - 1)/16 - pos0/16 + 1.
 extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table,
                                        const int* positions, const int* token_item, const int* block_table,
                                        int table_width, void* q_out, void* k_cache, void* v_cache, int num_tokens,
                                        int nh, int nkv, int d, int rd, int bs, float eps, int write_kv, int dtype,
-                                       hipStream_t stream) {
+                                       const int* item_start, int num_items, int num_segments, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || d > ME_MAX_HEAD_DIM || d % 2)
     return me_fail("me_qk_norm_rope_scatter: head_dim=%d must be even and at most %d", d, ME_MAX_HEAD_DIM);
   if (rd < 0 || rd > d || rd % 2) return me_fail("me_qk_norm_rope_scatter: rotary_dim=%d with head_dim=%d", rd, d);
   if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
     return me_fail("me_qk_norm_rope_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
-  const int heads_total = write_kv ? nh + 2 * nkv : nh;
+  const bool tiles = write_kv && num_segments > 0 && item_start != nullptr && bs % 16 == 0;
+  if (tiles && (num_items <= 0 || nkv > 65535)) return me_fail("me_qk_norm_rope_scatter: %d items, %d kv heads", num_items, nkv);
+  const int heads_total = write_kv ? (tiles ? nh + nkv : nh + 2 * nkv) : nh;
   // few tokens: spread the heads over many blocks; many tokens: a block per token keeps its table rows hot
   const int hpb = num_tokens >= 512 ? heads_total : 4;
   dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
   if (grid.y > 65535) return me_fail("me_qk_norm_rope_scatter: too many heads");
-  if (dtype == ME_F32)
-    qk_norm_rope_scatter_kernel<float><<<grid, 256, 0, stream>>>(
-        (const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (float*)q_out,
-        (float*)k_cache, (float*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb);
-  else
-    qk_norm_rope_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
-        (const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (bf16_t*)q_out,
-        (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb);
+  const bool quad = (rd == d || rope_table == nullptr) && (d & (d - 1)) == 0 && d >= 16 && d <= 256;
+  if (dtype == ME_F32) {
+    if (!(quad && launch_quad<float>((const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
+                                     table_width, (float*)q_out, (float*)k_cache, (float*)v_cache, num_tokens, nh, nkv,
+                                     d, bs, eps, write_kv, tiles ? 1 : 0, stream)))
+      qk_norm_rope_scatter_kernel<float><<<grid, 256, 0, stream>>>(
+          (const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (float*)q_out,
+          (float*)k_cache, (float*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb, tiles ? 1 : 0);
+    if (tiles)
+      v_scatter_tiles_kernel<float><<<dim3(num_segments, nkv), 256, 0, stream>>>(
+          (const float*)qkv, positions, item_start, num_items, block_table, table_width, (float*)v_cache, nh, nkv, d, bs);
+  } else {
+    if (!(quad && launch_quad<bf16_t>((const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
+                                      table_width, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, num_tokens, nh,
+                                      nkv, d, bs, eps, write_kv, tiles ? 1 : 0, stream)))
+      qk_norm_rope_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+          (const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (bf16_t*)q_out,
+          (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb, tiles ? 1 : 0);
+    if (tiles)
+      v_scatter_tiles_kernel<bf16_t><<<dim3(num_segments, nkv), 256, 0, stream>>>(
+          (const bf16_t*)qkv, positions, item_start, num_items, block_table, table_width, (bf16_t*)v_cache, nh, nkv, d,
+          bs);
+  }
   return me_check_launch("me_qk_norm_rope_scatter");
 }

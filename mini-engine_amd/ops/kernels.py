@@ -160,13 +160,20 @@ def qk_norm_rope_scatter(
     eps: float,
     write_kv: bool = True,
     q_out: torch.Tensor | None = None,
+    item_start: torch.Tensor | None = None,
+    starts: list[int] | None = None,
+    qlens: list[int] | None = None,
 ) -> torch.Tensor:
     """Per-head q/k RMSNorm (when weights are given), rotary encoding (when ``rope``, the table of
     :func:`rope_table`, is given; it must cover every position of the step), and the write of keys
     and values into their pages.
 
     qkv [T, (nh + 2 nkv) d] (or [T, nh d] with ``write_kv`` off: q only); k_cache [pages, nkv, bs, d]; v_cache [pages, nkv, d, bs];
-    block_table int32 [items, width]. Returns q [T, nh, d]."""
+    block_table int32 [items, width]. Returns q [T, nh, d].
+
+    With ``item_start`` (int32 [items + 1] on the device) and the items' first positions and lengths
+    on the host, steps with many tokens write the values a page segment at a time (a transposed
+    tile) instead of element by element."""
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     _want(qkv, "qkv", None, (None, ((nh + 2 * nkv) if write_kv else nh) * d))
     t, dtype = qkv.shape[0], qkv.dtype
@@ -183,10 +190,18 @@ def qk_norm_rope_scatter(
     if q_out is None:
         q_out = torch.empty((t, nh, d), dtype=dtype, device=qkv.device)
     _want(q_out, "q_out", dtype, (t, nh, d))
+    segments, items = 0, 0
+    if write_kv and item_start is not None and starts is not None and qlens is not None and t >= 64:
+        items = len(qlens)
+        if sum(qlens) != t or len(starts) != items:
+            raise ValueError("item lengths do not add up to the number of tokens")
+        _want(item_start, "item_start", torch.int32, (items + 1,))
+        segments = sum((p0 + n - 1) // 16 - p0 // 16 + 1 for p0, n in zip(starts, qlens))
     check(lib().me_qk_norm_rope_scatter(
         _p(qkv), _p(q_weight), _p(k_weight), _p(rope), _p(positions), _p(token_item), _p(block_table),
         _i(block_table.shape[1]), _p(q_out), _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(nkv), _i(d), _i(rd),
-        _i(bs), _f(eps), _i(1 if write_kv else 0), _i(_code(dtype)), _stream()))
+        _i(bs), _f(eps), _i(1 if write_kv else 0), _i(_code(dtype)), _p(item_start if segments else None), _i(items),
+        _i(segments), _stream()))
     return q_out
 
 

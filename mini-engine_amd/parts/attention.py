@@ -96,7 +96,8 @@ class Attention(Mixer):
             return K.linear(out, self.w_o)
         q = K.qk_norm_rope_scatter(
             proj, self.q_norm_w, self.k_norm_w if owns else None, rope, batch.positions, batch.token_item,
-            table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns)
+            table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns,
+            item_start=batch.item_start, starts=batch.starts, qlens=batch.qlens)
         out = self.attend(q, batch, table, b)
         return K.linear(out, self.w_o)
 

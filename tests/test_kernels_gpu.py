@@ -228,6 +228,36 @@ def test_qk_norm_rope_scatter(dtype, nh, nkv, d, bs, rd, norm):
     assert torch.equal(vc.permute(0, 3, 1, 2)[keep], v_cache.float().permute(0, 3, 1, 2)[keep])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,bs", [(4, 2, 32, 16), (16, 8, 128, 16), (3, 1, 64, 32), (2, 2, 48, 8)])
+def test_qk_norm_rope_scatter_writes_values_by_page_tiles(dtype, nh, nkv, d, bs):
+    """Many tokens: the values go through the page-tile kernel (pages of a multiple of 16 slots). Items
+    start inside a page, end inside a page, span many pages, and one has a single token; slots that
+    the step does not touch keep what they held. Same cache as the element-wise path."""
+    items = [(5, 70), (0, 33), (31, 1), (16, 16), (47, 100)]
+    k_cache, v_cache, tables, table_t, positions, token_item, _, _ = make_paged(items, nkv, d, bs, dtype, num_pages=96)
+    t = positions.numel()
+    qkv = torch.randn(t, (nh + 2 * nkv) * d).to(dtype)
+    qw, kw = 1 + 0.2 * torch.randn(d), 1 + 0.2 * torch.randn(d)
+    rope = K().rope_table(dev(1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))), 256)
+    qlens = [n for _, n in items]
+    item_start = torch.tensor([0] + torch.tensor(qlens).cumsum(0).tolist(), dtype=torch.int32)
+    out = {}
+    for tiled in (False, True):
+        kc, vc = dev(k_cache.clone()), dev(v_cache.clone())
+        extra = dict(item_start=dev(item_start), starts=[c for c, _ in items], qlens=qlens) if tiled else {}
+        q = K().qk_norm_rope_scatter(dev(qkv), dev(qw), dev(kw), rope, dev(positions), dev(token_item), dev(table_t),
+                                     kc, vc, nh, nkv, d, 1e-6, **extra)
+        out[tiled] = (q.cpu(), kc.cpu(), vc.cpu())
+    for a, b in zip(out[False], out[True]):
+        assert torch.equal(a, b)
+    v = qkv[:, (nh + nkv) * d :].view(t, nkv, d)
+    vc = out[True][2]
+    for i in range(t):
+        table, pos = tables[token_item[i]], int(positions[i])
+        assert torch.equal(vc[table[pos // bs], :, :, pos % bs], v[i])
+
+
 def dense_reference(qs, ks, vs, items, scale, window):
     outs = []
     for q, k, v, (cached, new) in zip(qs, ks, vs, items):
@@ -424,7 +454,10 @@ def test_attention_decode_fused_equals_the_two_kernels(nh, nkv, d, bs, norm, rot
     want = K().attention_decode_bf16(q, kc1, vc1, item_ctx, dev(wide), scale, window, 4096)
     got = K().attention_decode_fused_bf16(dev(qkv), qw, kw, rope, 1e-5, True, kc2, vc2, item_ctx, dev(wide), nh, scale,
                                           window, 4096)
-    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    # values are copied bit for bit; keys go through a float32 norm whose sum the two kernels take in
+    # different orders, so a key may differ in its last bfloat16 bit
+    assert torch.equal(vc1, vc2)
+    torch.testing.assert_close(kc1.float(), kc2.float(), rtol=2**-7, atol=1e-6)
     torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2)
     assert not K().attention_decode_fused_supported(96, 16, 96, 1)
     assert not K().attention_decode_fused_supported(128, 16, 64, 1)
