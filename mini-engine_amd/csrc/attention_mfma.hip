@@ -556,25 +556,33 @@ __device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)
                                              int tid, const int* __restrict__ table, int table_width, int bs_shift,
                                              int nkv, int kvh, const bf16_t* __restrict__ k_cache,
                                              const bf16_t* __restrict__ v_cache) {
+  // The 64 lanes of a wave fetch pieces of one 16-key sub-tile (8D/64 consecutive pieces never
+  // straddle one), so the page of a piece is the same for the whole wave: it is read into a scalar
+  // register and the base address of the page is scalar arithmetic; a lane only adds its own offset.
   const int bs_mask = (1 << bs_shift) - 1;
+  const int lane = tid & (ME_WAVE - 1), wave_c0 = tid - lane;
 #pragma unroll
   for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
-    const int c = tid + i * THREADS;
-    if ((8 * D) % THREADS != 0 && c >= 8 * D) break;  // only the last round can be partial
+    const int c_first = wave_c0 + i * THREADS;  // the wave's first piece of this round
+    if ((8 * D) % THREADS != 0 && c_first >= 8 * D) break;  // only the last round can be partial
+    const int c = c_first + lane;
     {
-      const int row = c / (D / 8), col = c % (D / 8);
-      const int key = key0 + row;
-      int page = table[min(key >> bs_shift, table_width - 1)];
+      const int key_w = key0 + ((c_first / (D / 8)) & ~15);  // first key of the wave's sub-tile
+      int page = __builtin_amdgcn_readfirstlane(table[min(key_w >> bs_shift, table_width - 1)]);
       page = page < 0 ? 0 : page;
-      kreg[i] = *reinterpret_cast<const uint4*>(k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + (key & bs_mask)) * D + col * 8);
+      const bf16_t* base = k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + (key_w & bs_mask)) * D;
+      const int row = c / (D / 8) - (c_first / (D / 8) & ~15), col = c % (D / 8);
+      kreg[i] = *reinterpret_cast<const uint4*>(base + row * D + col * 8);
     }
     {
-      const int sub = c / (2 * D), rem = c % (2 * D);
-      const int d = rem >> 1, half = rem & 1;
-      const int key = key0 + sub * 16 + half * 8;
-      int page = table[min(key >> bs_shift, table_width - 1)];
+      const int sub = c_first / (2 * D);
+      const int key_w = key0 + sub * 16;
+      int page = __builtin_amdgcn_readfirstlane(table[min(key_w >> bs_shift, table_width - 1)]);
       page = page < 0 ? 0 : page;
-      vreg[i] = *reinterpret_cast<const uint4*>(v_cache + ((((size_t)page * nkv + kvh) * D + d) << bs_shift) + (key & bs_mask));
+      const bf16_t* base = v_cache + ((((size_t)page * nkv + kvh) * D) << bs_shift) + (key_w & bs_mask);
+      const int rem = c - sub * (2 * D);
+      const int d = rem >> 1, half = rem & 1;
+      vreg[i] = *reinterpret_cast<const uint4*>(base + ((size_t)d << bs_shift) + half * 8);
     }
   }
 }
