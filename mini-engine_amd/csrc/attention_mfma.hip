@@ -525,11 +525,14 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
 //   S^T (16 keys x 16 columns) += K[16 keys, 32 d] . Q^T[32 d, 16 columns]
 //   O^T (16 d x 16 columns)   += V^T[16 d, 32 keys] . P^T[32 keys, 16 columns]
 // For the second product the 32 keys of a lane's B operand are the four keys it holds of each of two
-// 16-key score tiles (keys 4g..4g+3 and 16+4g..16+4g+3 of the 32); the A operand reads V^T in the
-// same order, so the contraction pairs up.
+// 16-key score tiles (keys 4g..4g+3 and 16+4g..16+4g+3 of the 32); the value tile is stored in LDS in
+// that order, so the A operand is one 16-byte read and the contraction pairs up.
 //
-// LDS rows are padded (keys: +8 elements, values: +4) so that the 16-byte key reads and the 8-byte
-// value reads of a wave spread over all banks.
+// LDS rows are padded (keys and values: +16 elements) so that the 16-byte reads of a wave spread over
+// all banks. A 16-byte read is served in four groups of lanes
+// (0-3 with 12-15 and 20-27, 4-11 with 16-19 and 28-31, and the same in the upper half): with 16 rows
+// read by lane % 16 the groups are free of conflicts when the row stride is 32 bytes off a multiple
+// of 64 (measured: 5.3 cycles per wave instruction against 8 with a stride 16 bytes off).
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
@@ -539,8 +542,8 @@ typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 
 template <int D>
 struct PrefillLds {
-  static constexpr int KROW = D + 8;        // elements per key row
-  static constexpr int VROW = PF_KT + 4;    // elements per value row (one d, 64 keys)
+  static constexpr int KROW = D + 16;       // elements per key row
+  static constexpr int VROW = PF_KT + 16;   // elements per value row (one d, 64 keys)
   static constexpr int K_ELEMS = PF_KT * KROW;
   static constexpr int V_ELEMS = D * VROW;
   static constexpr int BUF_ELEMS = K_ELEMS + V_ELEMS;
@@ -552,12 +555,33 @@ struct PrefillLds {
 // (c % (D/8)) * 8. Values: piece c -> 16-key sub-tile c / (2D), then d = (c % 2D) / 2, half = c % 2,
 // which walks a transposed value page front to back. The page size is a power of two.
 template <int D, int THREADS>
+struct PfPages {
+  int k[PF_PIECES(D, THREADS)], v[PF_PIECES(D, THREADS)];  // block-table entries, still per lane
+};
+
+// Block-table entries of the pages that the wave's pieces of tile `key0` lie in. The loads are only
+// issued here; pf_load_tile waits for them, an iteration later, so their latency hides behind a
+// whole tile of work instead of standing at the head of every iteration.
+template <int D, int THREADS>
+__device__ __forceinline__ void pf_fetch_pages(PfPages<D, THREADS>& pages, int key0, int tid, const int* __restrict__ table,
+                                               int table_width, int bs_shift) {
+  const int wave_c0 = tid & ~(ME_WAVE - 1);
+#pragma unroll
+  for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
+    const int c_first = wave_c0 + i * THREADS;
+    const int key_k = key0 + ((c_first / (D / 8)) & ~15);
+    const int key_v = key0 + (c_first / (2 * D)) * 16;
+    pages.k[i] = table[min(key_k >> bs_shift, table_width - 1)];
+    pages.v[i] = table[min(key_v >> bs_shift, table_width - 1)];
+  }
+}
+
+template <int D, int THREADS>
 __device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)], uint4 (&vreg)[PF_PIECES(D, THREADS)], int key0,
-                                             int tid, const int* __restrict__ table, int table_width, int bs_shift,
-                                             int nkv, int kvh, const bf16_t* __restrict__ k_cache,
-                                             const bf16_t* __restrict__ v_cache) {
+                                             int tid, const PfPages<D, THREADS>& pages, int bs_shift, int nkv, int kvh,
+                                             const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache) {
   // The 64 lanes of a wave fetch pieces of one 16-key sub-tile (8D/64 consecutive pieces never
-  // straddle one), so the page of a piece is the same for the whole wave: it is read into a scalar
+  // straddle one), so the page of a piece is the same for the whole wave: it goes into a scalar
   // register and the base address of the page is scalar arithmetic; a lane only adds its own offset.
   const int bs_mask = (1 << bs_shift) - 1;
   const int lane = tid & (ME_WAVE - 1), wave_c0 = tid - lane;
@@ -568,7 +592,7 @@ __device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)
     const int c = c_first + lane;
     {
       const int key_w = key0 + ((c_first / (D / 8)) & ~15);  // first key of the wave's sub-tile
-      int page = __builtin_amdgcn_readfirstlane(table[min(key_w >> bs_shift, table_width - 1)]);
+      int page = __builtin_amdgcn_readfirstlane(pages.k[i]);
       page = page < 0 ? 0 : page;
       const bf16_t* base = k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + (key_w & bs_mask)) * D;
       const int row = c / (D / 8) - (c_first / (D / 8) & ~15), col = c % (D / 8);
@@ -577,7 +601,7 @@ __device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)
     {
       const int sub = c_first / (2 * D);
       const int key_w = key0 + sub * 16;
-      int page = __builtin_amdgcn_readfirstlane(table[min(key_w >> bs_shift, table_width - 1)]);
+      int page = __builtin_amdgcn_readfirstlane(pages.v[i]);
       page = page < 0 ? 0 : page;
       const bf16_t* base = v_cache + ((((size_t)page * nkv + kvh) * D) << bs_shift) + (key_w & bs_mask);
       const int rem = c - sub * (2 * D);
@@ -600,87 +624,116 @@ __device__ __forceinline__ void pf_store_tile(const uint4 (&kreg)[PF_PIECES(D, T
     *reinterpret_cast<uint4*>(ks + row * L::KROW + col * 8) = kreg[i];
     const int sub = c / (2 * D), rem = c % (2 * D);
     const int d = rem >> 1, half = rem & 1;
-    uint2* dst = reinterpret_cast<uint2*>(vs + d * L::VROW + sub * 16 + half * 8);
+    // Within a group of 32 keys the row holds, for g = 0..3, keys 4g..4g+3 and then keys 16+4g..16+4g+3:
+    // the eight keys a lane multiplies with its eight probabilities, as one 16-byte read.
+    uint2* dst = reinterpret_cast<uint2*>(vs + d * L::VROW + (sub >> 1) * 32 + half * 16 + (sub & 1) * 4);
     dst[0] = make_uint2(vreg[i].x, vreg[i].y);
-    dst[1] = make_uint2(vreg[i].z, vreg[i].w);
+    dst[2] = make_uint2(vreg[i].z, vreg[i].w);
   }
 }
 
 typedef unsigned uint4v_t __attribute__((ext_vector_type(4)));
 
-// 32 keys (two 16-key score tiles) against NB blocks of 16 query columns, out of one LDS buffer.
-// MASK is a compile-time switch: tiles that every column of the wave sees whole skip the compares.
+// Maximum without the quieting of signalling NaNs that fmaxf brings along (an extra instruction per
+// operand): scores are finite or -inf here.
+__device__ __forceinline__ float max_raw(float a, float b) {
+  float d;
+  asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+__device__ __forceinline__ float column_max_raw(float v) {
+  unsigned u = __float_as_uint(v);
+  uint2v_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  u = __float_as_uint(max_raw(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return max_raw(__uint_as_float(a[0]), __uint_as_float(a[1]));
+}
+
+// One 64-key tile (four 16-key score tiles) against NB blocks of 16 query columns, out of one LDS
+// buffer, with one pass of the running softmax for all 64 keys. MASK is a compile-time switch:
+// tiles that every column of the wave sees whole skip the compares.
 template <int D, int NB, bool MASK>
-__device__ __forceinline__ void pf_attend32(const bf16_t* __restrict__ ks, const bf16_t* __restrict__ vs, int kbase_row,
-                                            int key_base, int r, int g, const bf16x8_t (&qf)[NB][D / 32],
-                                            const int (&qpos)[NB], const int (&lo_col)[NB], float scale_log2,
-                                            float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16]) {
+__device__ __forceinline__ void pf_attend64(const bf16_t* __restrict__ ks, const bf16_t* __restrict__ vs, int key_base, int r,
+                                            int g, const bf16x8_t (&qf)[NB][D / 32], const int (&qpos)[NB],
+                                            const int (&lo_col)[NB], float scale_log2, float (&m)[NB], float (&lsum)[NB],
+                                            float4_t (&acc)[NB][D / 16]) {
   using L = PrefillLds<D>;
-  float4_t s0[NB], s1[NB];
+  float4_t s[NB][4];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) s0[nb] = s1[nb] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) s[nb][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int c = 0; c < D / 32; ++c) {
-    const bf16x8_t k0 = *reinterpret_cast<const bf16x8_t*>(ks + (kbase_row + r) * L::KROW + c * 32 + g * 8);
-    const bf16x8_t k1 = *reinterpret_cast<const bf16x8_t*>(ks + (kbase_row + 16 + r) * L::KROW + c * 32 + g * 8);
+    bf16x8_t kf[4];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      s0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[nb][c], s0[nb], 0, 0, 0);
-      s1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[nb][c], s1[nb], 0, 0, 0);
-    }
+    for (int t = 0; t < 4; ++t) kf[t] = *reinterpret_cast<const bf16x8_t*>(ks + (t * 16 + r) * L::KROW + c * 32 + g * 8);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t], qf[nb][c], s[nb][t], 0, 0, 0);
   }
-  bf16x8_t pf[NB];
+  bf16x8_t pf[NB][2];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    float sv[8];
+    float sv[16];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      sv[i] = s0[nb][i];
-      sv[4 + i] = s1[nb][i];
-    }
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sv[t * 4 + i] = s[nb][t][i];
     if (MASK) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < 16; ++i) {
         const int key = key_base + (i >> 2) * 16 + g * 4 + (i & 3);
         if (key < lo_col[nb] || key > qpos[nb]) sv[i] = -INFINITY;
       }
     }
     // statistics are kept in units of the raw score times scale*log2(e): one fused multiply-add per
     // score feeds the exponential
-    float tmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-    tmax = column_max(tmax) * scale_log2;
-    const float m_new = fmaxf(m[nb], tmax);
+    float tmax = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), max3_raw(sv[6], sv[7], sv[8]));
+    tmax = max3_raw(tmax, max3_raw(sv[9], sv[10], sv[11]), max3_raw(sv[12], sv[13], sv[14]));
+    tmax = column_max_raw(max_raw(tmax, sv[15])) * scale_log2;
+    const float m_new = max_raw(m[nb], tmax);
     const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // a column with no visible key so far
     const float alpha = fast_exp2(m[nb] - m_ref);
-    float p[8];
+    float p[16];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(sv[i], scale_log2, -m_ref));
-    lsum[nb] = fmaf(lsum[nb], alpha, column_sum(((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))));
+    for (int i = 0; i < 16; ++i) p[i] = fast_exp2(fmaf(sv[i], scale_log2, -m_ref));
+    const float psum = (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))) +
+                       (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
+    lsum[nb] = fmaf(lsum[nb], alpha, column_sum(psum));
     m[nb] = m_new;
-    // the running maximum rarely moves after the first tiles: skip the rescale of the accumulator
-    // when no column of the wave needs it
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+    // (a branch that skips the rescale when no column's maximum moved costs more than it saves: the
+    // accumulator then lives in two sets of registers and is copied where it is not multiplied)
 #pragma unroll
-      for (int dt = 0; dt < D / 16; ++dt) {
-        acc[nb][dt][0] *= alpha;
-        acc[nb][dt][1] *= alpha;
-        acc[nb][dt][2] *= alpha;
-        acc[nb][dt][3] *= alpha;
-      }
+    for (int dt = 0; dt < D / 16; ++dt) {
+      acc[nb][dt][0] *= alpha;
+      acc[nb][dt][1] *= alpha;
+      acc[nb][dt][2] *= alpha;
+      acc[nb][dt][3] *= alpha;
     }
+    // the B operand of the second product: for each half of 32 keys, the lane's four keys of the first
+    // score tile and then those of the second
 #pragma unroll
-    for (int i = 0; i < 8; ++i) pf[nb][i] = (__bf16)p[i];  // round to nearest even in hardware
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pf[nb][h][i] = (__bf16)p[h * 8 + i];  // round to nearest even in hardware
   }
+  // halves outermost: the two products into one accumulator are D/16 instructions apart
 #pragma unroll
-  for (int dt = 0; dt < D / 16; ++dt) {
-    const bf16_t* vrow = vs + (dt * 16 + r) * L::VROW + kbase_row + g * 4;
-    const uint2 v0 = *reinterpret_cast<const uint2*>(vrow);
-    const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + 16);
-    const uint4v_t packed = {v0.x, v0.y, v1.x, v1.y};
-    const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, packed);
+  for (int h = 0; h < 2; ++h) {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-      acc[nb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[nb], acc[nb][dt], 0, 0, 0);
+    for (int dt = 0; dt < D / 16; ++dt) {
+      const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r) * L::VROW + h * 32 + g * 8);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        acc[nb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[nb][h], acc[nb][dt], 0, 0, 0);
+    }
   }
 }
 
@@ -697,7 +750,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   using L = PrefillLds<D>;
   __shared__ int s_item, s_tile, s_lo, s_hi;
   if (threadIdx.x == 0) {
-    int left = blockIdx.x, it = 0, tiles = 0;
+    int left = blockIdx.x / nkv, it = 0, tiles = 0;
     for (; it < num_items; ++it) {
       tiles = (item_start[it + 1] - item_start[it] + tokens_per_block - 1) / tokens_per_block;
       if (left < tiles) break;
@@ -716,7 +769,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   __syncthreads();
   const int item = s_item;
   if (item >= num_items) return;
-  const int kvh = blockIdx.y;
+  const int kvh = blockIdx.x % nkv;
   const int group = nh / nkv;
   const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
@@ -768,28 +821,26 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   uint4 kreg[PF_PIECES(D, THREADS)], vreg[PF_PIECES(D, THREADS)];
   const int first_tile = (s_lo / PF_KT) * PF_KT;
   const int last_key = s_hi;
-  pf_load_tile<D, THREADS>(kreg, vreg, first_tile, tid, table, table_width, bs_shift, nkv, kvh, k_cache, v_cache);
+  PfPages<D, THREADS> pages;
+  pf_fetch_pages<D, THREADS>(pages, first_tile, tid, table, table_width, bs_shift);
+  pf_load_tile<D, THREADS>(kreg, vreg, first_tile, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
+  pf_fetch_pages<D, THREADS>(pages, first_tile + PF_KT, tid, table, table_width, bs_shift);
   pf_store_tile<D, THREADS>(kreg, vreg, lds, tid);
   __syncthreads();
   int buf = 0;
   for (int key0 = first_tile; key0 <= last_key; key0 += PF_KT, buf ^= 1) {
     // the next tile is fetched unconditionally (the page index is clamped to the table, so a tile
     // past the last key reads valid memory that nobody uses): no control flow around the registers
-    pf_load_tile<D, THREADS>(kreg, vreg, key0 + PF_KT, tid, table, table_width, bs_shift, nkv, kvh, k_cache, v_cache);
+    pf_load_tile<D, THREADS>(kreg, vreg, key0 + PF_KT, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
+    pf_fetch_pages<D, THREADS>(pages, key0 + 2 * PF_KT, tid, table, table_width, bs_shift);  // for the next iteration
     if (key0 <= wave_max_pos) {
       const bf16_t* ks = lds + (size_t)buf * L::BUF_ELEMS;
       const bf16_t* vs = ks + L::K_ELEMS;
       const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || window > 0;
-      if (need_mask) {
-#pragma unroll
-        for (int kg = 0; kg < PF_KT / 32; ++kg)
-          if (key0 + kg * 32 <= wave_max_pos)
-            pf_attend32<D, NB, true>(ks, vs, kg * 32, key0 + kg * 32, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
-      } else {
-#pragma unroll
-        for (int kg = 0; kg < PF_KT / 32; ++kg)
-          pf_attend32<D, NB, false>(ks, vs, kg * 32, key0 + kg * 32, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
-      }
+      if (need_mask)
+        pf_attend64<D, NB, true>(ks, vs, key0, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
+      else
+        pf_attend64<D, NB, false>(ks, vs, key0, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
     }
     pf_store_tile<D, THREADS>(kreg, vreg, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, tid);
     __syncthreads();
@@ -849,7 +900,7 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   const float sl = scale * LOG2E;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-  dim3 grid(num_blocks, nkv);
+  dim3 grid((unsigned)num_blocks * nkv);
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
   int rc = 0;
 #define ME_PREFILL_CASE(DD)                                                                                        \
