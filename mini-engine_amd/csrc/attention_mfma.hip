@@ -47,6 +47,7 @@ __device__ __forceinline__ short4_t pack_bf16x4(float a, float b, float c, float
 // speed: after a swap of a register with a copy of itself, the two results hold, in every lane, the
 // lane's own value and that of lane ^ 16 (resp. lane ^ 32), in one order or the other.
 typedef unsigned uint2v_t __attribute__((ext_vector_type(2)));
+typedef unsigned uint4v_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float column_max(float v) {
   unsigned u = __float_as_uint(v);
   uint2v_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
@@ -577,7 +578,7 @@ __device__ __forceinline__ void pf_fetch_pages(PfPages<D, THREADS>& pages, int k
 }
 
 template <int D, int THREADS>
-__device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)], uint4 (&vreg)[PF_PIECES(D, THREADS)], int key0,
+__device__ __forceinline__ void pf_load_tile(uint4v_t (&kreg)[PF_PIECES(D, THREADS)], uint4v_t (&vreg)[PF_PIECES(D, THREADS)], int key0,
                                              int tid, const PfPages<D, THREADS>& pages, int bs_shift, int nkv, int kvh,
                                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache) {
   // The 64 lanes of a wave fetch pieces of one 16-key sub-tile (8D/64 consecutive pieces never
@@ -596,7 +597,7 @@ __device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)
       page = page < 0 ? 0 : page;
       const bf16_t* base = k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + (key_w & bs_mask)) * D;
       const int row = c / (D / 8) - (c_first / (D / 8) & ~15), col = c % (D / 8);
-      kreg[i] = *reinterpret_cast<const uint4*>(base + row * D + col * 8);
+      kreg[i] = *reinterpret_cast<const uint4v_t*>(base + row * D + col * 8);
     }
     {
       const int sub = c_first / (2 * D);
@@ -606,13 +607,13 @@ __device__ __forceinline__ void pf_load_tile(uint4 (&kreg)[PF_PIECES(D, THREADS)
       const bf16_t* base = v_cache + ((((size_t)page * nkv + kvh) * D) << bs_shift) + (key_w & bs_mask);
       const int rem = c - sub * (2 * D);
       const int d = rem >> 1, half = rem & 1;
-      vreg[i] = *reinterpret_cast<const uint4*>(base + ((size_t)d << bs_shift) + half * 8);
+      vreg[i] = *reinterpret_cast<const uint4v_t*>(base + ((size_t)d << bs_shift) + half * 8);
     }
   }
 }
 
 template <int D, int THREADS>
-__device__ __forceinline__ void pf_store_tile(const uint4 (&kreg)[PF_PIECES(D, THREADS)], const uint4 (&vreg)[PF_PIECES(D, THREADS)],
+__device__ __forceinline__ void pf_store_tile(const uint4v_t (&kreg)[PF_PIECES(D, THREADS)], const uint4v_t (&vreg)[PF_PIECES(D, THREADS)],
                                               bf16_t* ks, int tid) {
   using L = PrefillLds<D>;
   bf16_t* vs = ks + L::K_ELEMS;
@@ -621,18 +622,17 @@ __device__ __forceinline__ void pf_store_tile(const uint4 (&kreg)[PF_PIECES(D, T
     const int c = tid + i * THREADS;
     if ((8 * D) % THREADS != 0 && c >= 8 * D) break;
     const int row = c / (D / 8), col = c % (D / 8);
-    *reinterpret_cast<uint4*>(ks + row * L::KROW + col * 8) = kreg[i];
+    *reinterpret_cast<uint4v_t*>(ks + row * L::KROW + col * 8) = kreg[i];
     const int sub = c / (2 * D), rem = c % (2 * D);
     const int d = rem >> 1, half = rem & 1;
     // Within a group of 32 keys the row holds, for g = 0..3, keys 4g..4g+3 and then keys 16+4g..16+4g+3:
     // the eight keys a lane multiplies with its eight probabilities, as one 16-byte read.
-    uint2* dst = reinterpret_cast<uint2*>(vs + d * L::VROW + (sub >> 1) * 32 + half * 16 + (sub & 1) * 4);
-    dst[0] = make_uint2(vreg[i].x, vreg[i].y);
-    dst[2] = make_uint2(vreg[i].z, vreg[i].w);
+    uint2v_t* dst = reinterpret_cast<uint2v_t*>(vs + d * L::VROW + (sub >> 1) * 32 + half * 16 + (sub & 1) * 4);
+    dst[0] = (uint2v_t){vreg[i][0], vreg[i][1]};
+    dst[2] = (uint2v_t){vreg[i][2], vreg[i][3]};
   }
 }
 
-typedef unsigned uint4v_t __attribute__((ext_vector_type(4)));
 
 // Maximum without the quieting of signalling NaNs that fmaxf brings along (an extra instruction per
 // operand): scores are finite or -inf here.
@@ -654,16 +654,12 @@ __device__ __forceinline__ float column_max_raw(float v) {
   return max_raw(__uint_as_float(a[0]), __uint_as_float(a[1]));
 }
 
-// One 64-key tile (four 16-key score tiles) against NB blocks of 16 query columns, out of one LDS
-// buffer, with one pass of the running softmax for all 64 keys. MASK is a compile-time switch:
-// tiles that every column of the wave sees whole skip the compares.
-template <int D, int NB, bool MASK>
-__device__ __forceinline__ void pf_attend64(const bf16_t* __restrict__ ks, const bf16_t* __restrict__ vs, int key_base, int r,
-                                            int g, const bf16x8_t (&qf)[NB][D / 32], const int (&qpos)[NB],
-                                            const int (&lo_col)[NB], float scale_log2, float (&m)[NB], float (&lsum)[NB],
-                                            float4_t (&acc)[NB][D / 16]) {
+// First product of one 64-key tile: four 16-key score tiles against NB blocks of 16 query columns,
+// out of the key half of one LDS buffer.
+template <int D, int NB>
+__device__ __forceinline__ void pf_scores64(const bf16_t* __restrict__ ks, int r, int g, const bf16x8_t (&qf)[NB][D / 32],
+                                            float4_t (&s)[NB][4]) {
   using L = PrefillLds<D>;
-  float4_t s[NB][4];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -678,6 +674,17 @@ __device__ __forceinline__ void pf_attend64(const bf16_t* __restrict__ ks, const
 #pragma unroll
       for (int t = 0; t < 4; ++t) s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t], qf[nb][c], s[nb][t], 0, 0, 0);
   }
+}
+
+// One pass of the running softmax over the 64 scores of each column, then the second product out of the
+// value half of the LDS buffer. MASK is a compile-time switch: tiles that every column of the wave
+// sees whole skip the compares.
+template <int D, int NB, bool MASK>
+__device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, int key_base, int r, int g,
+                                                const float4_t (&s)[NB][4], const int (&qpos)[NB], const int (&lo_col)[NB],
+                                                float scale_log2, float (&m)[NB], float (&lsum)[NB],
+                                                float4_t (&acc)[NB][D / 16]) {
+  using L = PrefillLds<D>;
   bf16x8_t pf[NB][2];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
@@ -817,8 +824,12 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     for (int dt = 0; dt < D / 16; ++dt) acc[nb][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- global -> register -> LDS staging of one 64-key tile (pf_load_tile / pf_store_tile)
-  uint4 kreg[PF_PIECES(D, THREADS)], vreg[PF_PIECES(D, THREADS)];
+  // ---- global -> register -> LDS staging of 64-key tiles (pf_load_tile / pf_store_tile). While tile i
+  // is multiplied out of LDS buffer i % 2, tile i+1 waits in registers: it is written to the other buffer
+  // in the middle of the iteration, behind the first product, where the LDS writes and the global loads
+  // of tile i+2 that follow them overlap with the softmax arithmetic instead of standing between two
+  // barriers. The other buffer is free then: it was last read before the barrier that ended iteration i-1.
+  uint4v_t kreg[PF_PIECES(D, THREADS)], vreg[PF_PIECES(D, THREADS)];
   const int first_tile = (s_lo / PF_KT) * PF_KT;
   const int last_key = s_hi;
   PfPages<D, THREADS> pages;
@@ -826,23 +837,28 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   pf_load_tile<D, THREADS>(kreg, vreg, first_tile, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
   pf_fetch_pages<D, THREADS>(pages, first_tile + PF_KT, tid, table, table_width, bs_shift);
   pf_store_tile<D, THREADS>(kreg, vreg, lds, tid);
+  pf_load_tile<D, THREADS>(kreg, vreg, first_tile + PF_KT, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
+  pf_fetch_pages<D, THREADS>(pages, first_tile + 2 * PF_KT, tid, table, table_width, bs_shift);
   __syncthreads();
   int buf = 0;
   for (int key0 = first_tile; key0 <= last_key; key0 += PF_KT, buf ^= 1) {
-    // the next tile is fetched unconditionally (the page index is clamped to the table, so a tile
-    // past the last key reads valid memory that nobody uses): no control flow around the registers
-    pf_load_tile<D, THREADS>(kreg, vreg, key0 + PF_KT, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
-    pf_fetch_pages<D, THREADS>(pages, key0 + 2 * PF_KT, tid, table, table_width, bs_shift);  // for the next iteration
-    if (key0 <= wave_max_pos) {
-      const bf16_t* ks = lds + (size_t)buf * L::BUF_ELEMS;
-      const bf16_t* vs = ks + L::K_ELEMS;
+    const bf16_t* ks = lds + (size_t)buf * L::BUF_ELEMS;
+    const bf16_t* vs = ks + L::K_ELEMS;
+    const bool active = key0 <= wave_max_pos;  // else every column of the wave lies before this tile
+    float4_t s[NB][4];
+    pf_scores64<D, NB>(ks, r, g, qf, s);  // also by a wave that will not use them: no control flow around s
+    // Tiles are fetched unconditionally (the page index is clamped to the table, so a tile past the last
+    // key reads valid memory that nobody uses): no control flow around the registers.
+    pf_store_tile<D, THREADS>(kreg, vreg, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, tid);
+    pf_load_tile<D, THREADS>(kreg, vreg, key0 + 2 * PF_KT, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
+    pf_fetch_pages<D, THREADS>(pages, key0 + 3 * PF_KT, tid, table, table_width, bs_shift);  // for the next iteration
+    if (active) {
       const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || window > 0;
       if (need_mask)
-        pf_attend64<D, NB, true>(ks, vs, key0, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
+        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc);
       else
-        pf_attend64<D, NB, false>(ks, vs, key0, r, g, qf, qpos, lo_col, scale_log2, m, lsum, acc);
+        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc);
     }
-    pf_store_tile<D, THREADS>(kreg, vreg, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, tid);
     __syncthreads();
   }
 #pragma unroll
