@@ -159,7 +159,7 @@ struct DecodeFusedArgs {
   bf16_t* v_cache_w;
 };
 
-template <int D, bool FUSED, bool PIPE>
+template <int D, bool FUSED, int DEPTH>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
@@ -173,6 +173,21 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
   const int heads_here = min(16, group - chunk * 16);
   const int head0 = kvh * group + chunk * 16;
+  const int* table = block_table + (size_t)item * table_width;
+  auto fetch = [&](KvTile<D>& t, int key0) {
+    int page = table[min(key0 >> bs_shift, table_width - 1)];
+    page = page < 0 ? 0 : page;
+    const int off = key0 & (bs - 1);
+    load_tile<D>(t, k_cache + (((size_t)page * nkv + kvh) * bs + off) * D,
+                 v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
+  };
+  KvTile<D> t[DEPTH];
+  // Without a window the first key of a split does not depend on the item's length: its tile is
+  // requested at once, beside the load of the length instead of behind it (one memory round trip less
+  // at the head of every block). A split that turns out to lie past the item's end has read a valid page
+  // (an entry of the table, or page 0) that it does not use.
+  const bool speculative = window <= 0;
+  if (speculative) fetch(t[0], split * split_keys);
   const int ctx = item_ctx[item];
   const int lo = window > 0 ? max(ctx - window, 0) : 0;
   const int begin = max(split * split_keys, (lo / 16) * 16);
@@ -184,20 +199,10 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   for (int dt = 0; dt < D / 16; ++dt) acc[0][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
   if (begin < end) {
-    const int* table = block_table + (size_t)item * table_width;
-    // two tiles in flight: the loads of tile i+1 are issued before the products of tile i
-    auto fetch = [&](KvTile<D>& t, int key0) {
-      int page = table[min(key0 >> bs_shift, table_width - 1)];
-      page = page < 0 ? 0 : page;
-      const int off = key0 & (bs - 1);
-      load_tile<D>(t, k_cache + (((size_t)page * nkv + kvh) * bs + off) * D,
-                   v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
-    };
-    KvTile<D> ta, tb;
-    // the first tile is requested before the query is prepared, unless it holds the slot that this
-    // block is about to write
+    // otherwise the first tile is requested before the query is prepared, unless it holds the slot that
+    // this block is about to write: then it is requested (again) after that write
     const bool early = !FUSED || begin + 16 < ctx;
-    if (early) fetch(ta, begin);
+    if (early && !speculative) fetch(t[0], begin);
     Frag8 qf[1][D / 32];
     if (FUSED) {
       constexpr int HC = D / 64;  // chunks per half head
@@ -294,21 +299,21 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
       }
     }
     const int qpos[1] = {ctx - 1};
-    if (!early) fetch(ta, begin);
-    if (PIPE) {
-      // short splits (few waves, each waiting on memory): keep two tiles in flight per wave
-      for (int key0 = begin; key0 < end; key0 += 32) {
-        fetch(tb, key0 + 16);  // may lie past `end`: a valid page, computed on only if it is in range
-        compute_tile<D, 1>(ta, key0, lo, qpos, key0 < lo || key0 + 16 > ctx, qf, scale_log2, m, lsum, acc);
-        fetch(ta, key0 + 32);
-        if (key0 + 16 < end)
-          compute_tile<D, 1>(tb, key0 + 16, lo, qpos, key0 + 16 < lo || key0 + 32 > ctx, qf, scale_log2, m, lsum, acc);
-      }
-    } else {
-      // long splits (the chip is full of waves): fewer registers, one more wave per SIMD
-      for (int key0 = begin; key0 < end; key0 += 16) {
-        if (key0 > begin) fetch(ta, key0);
-        compute_tile<D, 1>(ta, key0, lo, qpos, key0 < lo || key0 + 16 > ctx, qf, scale_log2, m, lsum, acc);
+    if (!early) fetch(t[0], begin);
+    // DEPTH tiles in flight per wave: tile i + DEPTH - 1 is requested before the products of tile i. Short
+    // splits (few waves, each waiting on memory) want two (four measured no better); with long splits the
+    // chip is full of waves and fewer registers, one more wave per SIMD, serve better. A tile past `end` is a valid page that
+    // nobody computes on.
+#pragma unroll
+    for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], begin + 16 * j);
+    for (int key0 = begin; key0 < end; key0 += 16 * DEPTH) {
+#pragma unroll
+      for (int j = 0; j < DEPTH; ++j) {
+        const int k = key0 + 16 * j;
+        if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], k + 16 * (DEPTH - 1));
+        else if (k > begin) fetch(t[0], k);
+        if (j == 0 || k < end)
+          compute_tile<D, 1>(t[j], k, lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc);
       }
     }
   }
@@ -399,24 +404,24 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
   dim3 grid(items, nkv * chunks, num_splits);
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-  const bool pipe = split_keys <= 256;
-#define ME_DECODE_LAUNCH(FUSED, PIPE, ARGS)                                                                          \
-  attention_decode_kernel<D, FUSED, PIPE><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
-                                                                   nkv, bs_shift, window, scale_log2, split_keys,     \
-                                                                   num_splits, chunks, ARGS)
+  const int depth = split_keys <= 256 ? 2 : 1;
+#define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                                                                         \
+  attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
+                                                                    nkv, bs_shift, window, scale_log2, split_keys,    \
+                                                                    num_splits, chunks, ARGS)
   if constexpr (D % 64 == 0) {
     if (fused) {
-      if (pipe)
-        ME_DECODE_LAUNCH(true, true, *fused);
+      if (depth == 2)
+        ME_DECODE_LAUNCH(true, 2, *fused);
       else
-        ME_DECODE_LAUNCH(true, false, *fused);
+        ME_DECODE_LAUNCH(true, 1, *fused);
       return;
     }
   }
-  if (pipe)
-    ME_DECODE_LAUNCH(false, true, DecodeFusedArgs{});
+  if (depth == 2)
+    ME_DECODE_LAUNCH(false, 2, DecodeFusedArgs{});
   else
-    ME_DECODE_LAUNCH(false, false, DecodeFusedArgs{});
+    ME_DECODE_LAUNCH(false, 1, DecodeFusedArgs{});
 #undef ME_DECODE_LAUNCH
 }
 

@@ -413,6 +413,31 @@ def test_attention_decode_mfma(nh, nkv, d, bs, window):
         torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
 
 
+def test_attention_decode_many_splits():
+    """A long context of one item is cut into more splits than a wave has lanes; a far key is made to
+    dominate so that a split that is dropped or weighted wrongly shows."""
+    dtype = torch.bfloat16
+    nh, nkv, d, bs = 4, 1, 64, 16
+    ctx = 9000
+    items = [(ctx - 1, 1), (4999, 1)]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=900)
+    g = torch.Generator().manual_seed(3)
+    qs = [torch.randn(1, nh, d, generator=g).to(dtype) for _ in items]
+    ks[0][1234] = (qs[0][0, 1:2].float() * 2.0).to(dtype)  # head 1 of item 0 looks at key 1234 almost alone
+    k_cache[tables[0][1234 // bs], :, 1234 % bs, :] = ks[0][1234]
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    scale = d**-0.5
+    want = dense_reference(qs, ks, vs, items, scale, 0)
+    item_ctx = torch.tensor([ctx, 5000], dtype=torch.int32)
+    max_ctx = 16384
+    wide = torch.zeros(len(items), max_ctx // bs, dtype=torch.int32)
+    wide[:, : table_t.shape[1]] = table_t
+    assert K().decode_splits(len(items), nkv, max_ctx)[1] > 64
+    out = K().attention_decode_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide), scale, 0,
+                                    max_ctx)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("nh,nkv,d,bs", [s for s in MFMA_SHAPES if s[0] // s[1] <= 16])
 @pytest.mark.parametrize("window", [0, 37])
 def test_attention_prefill_mfma(nh, nkv, d, bs, window):
