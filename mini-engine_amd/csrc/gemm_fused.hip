@@ -169,7 +169,14 @@ static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x
                          const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
                          hipStream_t stream) {
   const int mt = (M + 15) / 16;
-  if (mt == 1)
+  // up to 16 rows: as many chunks of 32 k per wave and round as it takes to have all of k in flight at
+  // once (a second round of loads costs a memory round trip, which is most of such a kernel's time)
+  const int chunks = (K + 31) / 32;
+  if (mt == 1 && chunks > 8 * 8)
+    launch_variant<1, 8, 12, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else if (mt == 1 && chunks > 8 * 4)
+    launch_variant<1, 8, 8, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else if (mt == 1)
     launch_variant<1, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
   else if (mt == 2)
     launch_variant<2, 8, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
