@@ -520,9 +520,14 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
 // new tokens of one item for one kv head (column c -> token c / group, head c % group); wave w owns
 // NB blocks of 16 columns. Measured on 2,048-token prompts of the 0.6B shape: 8 waves x 1 block of
 // columns (128 columns a block) beats 4 x 2 (register pressure pushes the accumulators out of the
-// vector registers) and 4 x 1 (64 columns a block, twice the LDS traffic per product). Blocks are
-// numbered over all items: item i has ceil(qlen_i / tokens_per_block) of them, the later (longer)
-// tiles of an item first.
+// vector registers) and 4 x 1 (64 columns a block, twice the LDS traffic per product, also when a long and
+// a short tile share a compute unit). What a block does is an entry of a work list that the host lays
+// out once per step, longest first: which tokens, which range of keys. Causal prompts give tiles of
+// very different lengths; a block costs about 3 us plus 1.5 us per 64 keys, so at 2,048 tokens (one block
+// per compute unit) the last tile's 32 key tiles set the time. Cutting long tiles into ranges, whose
+// partial results a second kernel adds up, evens that out but pays the fixed cost and the partial
+// results again: measured worth it only where the step has fewer blocks than the chip has compute
+// units (a short portion of a prompt over a long context), which is where the host does it.
 //
 // Keys and values are staged through LDS in tiles of 64 keys, double-buffered: while the waves
 // multiply tile i out of one buffer, the global loads of tile i+1 are in flight and are written to
@@ -749,44 +754,38 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
   }
 }
 
+// One entry of the work list that the host lays out for a step (heaviest first): a tile of consecutive
+// query tokens of one item and a range of keys. The positions of an item's tokens are consecutive, so the
+// first one's stands for all. A tile whose keys are cut into several ranges gives partial results that
+// attention_prefill_combine_kernel adds up; `chunk` is -1 for a tile in one piece.
+struct PrefillWork {
+  int item;
+  int token_begin, token_count;  // the tile's tokens among the packed tokens of the step
+  int pos_first;                 // position of the first of them
+  int key_begin;                 // first key, a multiple of 64
+  int key_last;                  // last key, inclusive
+  int chunk;
+  int pad;
+};
+
 // WAVES waves per block, NB blocks of 16 query columns per wave: WAVES * NB * 16 = 128 columns.
 template <int D, int NB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-    const int* __restrict__ positions, const int* __restrict__ item_start, int num_items,
-    const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
-    int window, float scale_log2, int tokens_per_block) {
+    const PrefillWork* __restrict__ work, const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window, float scale_log2,
+    int tokens_per_block) {
   constexpr int THREADS = WAVES * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
   using L = PrefillLds<D>;
-  __shared__ int s_item, s_tile, s_lo, s_hi;
-  if (threadIdx.x == 0) {
-    int left = blockIdx.x / nkv, it = 0, tiles = 0;
-    for (; it < num_items; ++it) {
-      tiles = (item_start[it + 1] - item_start[it] + tokens_per_block - 1) / tokens_per_block;
-      if (left < tiles) break;
-      left -= tiles;
-    }
-    s_item = it;
-    s_tile = tiles - 1 - left;  // long tiles first
-    if (it < num_items) {
-      const int tb = item_start[it] + s_tile * tokens_per_block;
-      const int te = min(item_start[it + 1], tb + tokens_per_block);
-      const int p_first = positions[tb], p_last = positions[te - 1];
-      s_lo = window > 0 ? max(p_first - window + 1, 0) : 0;
-      s_hi = p_last;
-    }
-  }
-  __syncthreads();
-  const int item = s_item;
-  if (item >= num_items) return;
+  const PrefillWork w = work[blockIdx.x / nkv];  // the same for every lane: scalar loads
+  const int item = w.item;
   const int kvh = blockIdx.x % nkv;
   const int group = nh / nkv;
   const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  const int t_begin = item_start[item] + s_tile * tokens_per_block;
-  const int t_end = min(item_start[item + 1], t_begin + tokens_per_block);
+  const int t_begin = w.token_begin, t_end = w.token_begin + w.token_count;
   const int* table = block_table + (size_t)item * table_width;
 
   // this lane's query column in each of the wave's blocks
@@ -799,7 +798,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     tok[nb] = t_begin + c / group;
     head[nb] = kvh * group + c % group;
     col_ok[nb] = c < tokens_per_block * group && tok[nb] < t_end;
-    qpos[nb] = col_ok[nb] ? positions[tok[nb]] : -1;
+    qpos[nb] = col_ok[nb] ? w.pos_first + c / group : -1;
     lo_col[nb] = window > 0 ? max(qpos[nb] - window + 1, 0) : 0;
     wave_max_pos = max(wave_max_pos, qpos[nb]);
     if (col_ok[nb]) wave_min_pos = min(wave_min_pos, qpos[nb]);
@@ -835,8 +834,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   // of tile i+2 that follow them overlap with the softmax arithmetic instead of standing between two
   // barriers. The other buffer is free then: it was last read before the barrier that ended iteration i-1.
   uint4v_t kreg[PF_PIECES(D, THREADS)], vreg[PF_PIECES(D, THREADS)];
-  const int first_tile = (s_lo / PF_KT) * PF_KT;
-  const int last_key = s_hi;
+  const int first_tile = w.key_begin;
+  const int last_key = w.key_last;
   PfPages<D, THREADS> pages;
   pf_fetch_pages<D, THREADS>(pages, first_tile, tid, table, table_width, bs_shift);
   pf_load_tile<D, THREADS>(kreg, vreg, first_tile, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
@@ -866,6 +865,21 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     }
     __syncthreads();
   }
+  if (w.chunk >= 0) {
+    // one range of several: the unnormalised sums and the statistics of every column
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      if (!col_ok[nb]) continue;
+      const size_t slot = ((size_t)tok[nb] * nh + head[nb]) * max_chunks + w.chunk;
+      if (g == 0) {
+        part_ml[slot * 2] = m[nb];
+        part_ml[slot * 2 + 1] = lsum[nb];
+      }
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) *reinterpret_cast<float4_t*>(part_o + slot * D + dt * 16 + g * 4) = acc[nb][dt];
+    }
+    return;
+  }
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     if (!col_ok[nb]) continue;
@@ -880,6 +894,47 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   }
 }
 
+// Adds up the ranges of the tokens whose keys were cut: out[token, head, :] = sum_c 2^(m_c - M) o_c /
+// sum_c 2^(m_c - M) l_c over the token's chunks (token_chunks[token]; tokens with one chunk were written
+// by the attention kernel itself). One block per token; a thread owns four consecutive outputs of a head
+// at a time, so that all loads of a block are independent of each other.
+__global__ __launch_bounds__(256) void attention_prefill_combine_kernel(const float* __restrict__ part_o,
+                                                                        const float* __restrict__ part_ml,
+                                                                        const int* __restrict__ token_chunks,
+                                                                        bf16_t* __restrict__ out, int nh, int d,
+                                                                        int max_chunks) {
+  const int tok = blockIdx.x;
+  const int nc = token_chunks[tok];
+  if (nc <= 1) return;
+  const int quads = nh * d / 4;  // d is a multiple of 32
+  for (int v = threadIdx.x; v < quads; v += 256) {
+    const int head = v * 4 / d, e = v * 4 % d;
+    const size_t unit = (size_t)tok * nh + head;
+    const float* ml = part_ml + unit * max_chunks * 2;
+    const float* po = part_o + unit * max_chunks * d + e;
+    float big = -INFINITY;
+    for (int c = 0; c < nc; ++c)
+      if (ml[c * 2 + 1] > 0.f) big = fmaxf(big, ml[c * 2]);
+    float denom = 0.f;
+    float4_t total = {0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < nc; ++c) {
+      const float l = ml[c * 2 + 1];
+      if (l > 0.f) {  // a range with no visible key has no weight
+        const float wgt = fast_exp2(ml[c * 2] - big);
+        const float4_t o = *reinterpret_cast<const float4_t*>(po + (size_t)c * d);
+        denom += wgt * l;
+        total[0] = fmaf(wgt, o[0], total[0]);
+        total[1] = fmaf(wgt, o[1], total[1]);
+        total[2] = fmaf(wgt, o[2], total[2]);
+        total[3] = fmaf(wgt, o[3], total[3]);
+      }
+    }
+    const float inv = 1.f / denom;
+    *reinterpret_cast<short4_t*>(out + unit * d + e) =
+        pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
+  }
+}
+
 #define PF_NB 1
 #define PF_WAVES 8
 #define PF_COLUMNS (PF_NB * PF_WAVES * 16)  // query columns (token, head of the group) per block
@@ -887,9 +942,10 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
 extern "C" int me_attention_prefill_columns() { return PF_COLUMNS; }
 
 template <int D>
-static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* positions,
-                          const int* item_start, int num_items, const int* table, int width, bf16_t* out, int nh,
-                          int nkv, int bs_shift, int window, float sl, int tpb, hipStream_t stream) {
+static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const PrefillWork* work,
+                          const int* table, int width, bf16_t* out,
+                          float* part_o, float* part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window,
+                          float sl, int tpb, hipStream_t stream) {
   static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, PF_NB, PF_WAVES>),
@@ -899,35 +955,43 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
     configured = true;
   }
   attention_prefill_kernel<D, PF_NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
-      q, kc, vc, positions, item_start, num_items, table, width, out, nh, nkv, bs_shift, window, sl, tpb);
+      q, kc, vc, work, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb);
   return 0;
 }
 
-// q [T, nh, d]; item_start int [items + 1] (offsets of the items' tokens); positions int [T];
-// num_blocks = sum over items of ceil(qlen / (me_attention_prefill_columns() / group)), computed by the caller.
-extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, const int* positions,
-                                         const int* item_start, int num_items, const int* block_table, int table_width,
-                                         void* out, int num_blocks, int nh, int nkv, int d, int bs, int window,
+// q [T, nh, d], packed new tokens. work: num_work entries of eight ints laid out by the caller (item, first
+// token and number of tokens of the tile (at most me_attention_prefill_columns() / group), position of the
+// first token, first key (a multiple of 64), last key, chunk or -1, one unused); every entry is run for
+// every kv head. When a tile's keys are cut into chunks (max_chunks > 1), part_o float
+// [T, nh, max_chunks, d] and part_ml float [T, nh, max_chunks, 2] take the partial results and
+// token_chunks int [T] says how many chunks each token's tile has (1: in one piece).
+extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                                         const int* block_table, int table_width, void* out, const int* work,
+                                         int num_work, float* part_o, float* part_ml, const int* token_chunks,
+                                         int max_chunks, int num_tokens, int nh, int nkv, int d, int bs, int window,
                                          float scale, hipStream_t stream) {
-  if (num_items <= 0 || num_blocks <= 0) return 0;
+  if (num_items <= 0 || num_work <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_prefill_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
   if (nh <= 0 || nkv <= 0 || nh % nkv) return me_fail("me_attention_prefill_bf16: nh=%d nkv=%d", nh, nkv);
   const int group = nh / nkv;
   if (group > 16) return me_fail("me_attention_prefill_bf16: group size %d exceeds 16", group);
-  if (nkv > 65535) return me_fail("me_attention_prefill_bf16: %d kv heads exceed the grid", nkv);
+  if ((long long)num_work * nkv > 0x7fffffffLL) return me_fail("me_attention_prefill_bf16: %d x %d blocks exceed the grid", num_work, nkv);
   if (table_width <= 0) return me_fail("me_attention_prefill_bf16: empty block table");
+  if (!work) return me_fail("me_attention_prefill_bf16: no work list");
+  if (max_chunks < 1 || (max_chunks > 1 && (!part_o || !part_ml || !token_chunks || num_tokens <= 0)))
+    return me_fail("me_attention_prefill_bf16: %d chunks need the partial buffers and the chunk counts", max_chunks);
   const int tpb = PF_COLUMNS / group;
   const float sl = scale * LOG2E;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-  dim3 grid((unsigned)num_blocks * nkv);
+  dim3 grid((unsigned)num_work * nkv);
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
   int rc = 0;
 #define ME_PREFILL_CASE(DD)                                                                                        \
   case DD:                                                                                                         \
-    rc = launch_prefill<DD>(grid, qq, kc, vc, positions, item_start, num_items, block_table, table_width,          \
-                            (bf16_t*)out, nh, nkv, bs_shift, window, sl, tpb, stream);                             \
+    rc = launch_prefill<DD>(grid, qq, kc, vc, (const PrefillWork*)work, block_table, table_width, (bf16_t*)out,   \
+                            part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb, stream);              \
     break;
   switch (d) {
     ME_PREFILL_CASE(32)
@@ -939,5 +1003,11 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   }
 #undef ME_PREFILL_CASE
   if (rc) return rc;
-  return me_check_launch("me_attention_prefill_bf16");
+  if (me_check_launch("me_attention_prefill_bf16")) return 1;
+  if (max_chunks > 1) {
+    attention_prefill_combine_kernel<<<num_tokens, 256, 0, stream>>>(part_o, part_ml, token_chunks, (bf16_t*)out, nh, d,
+                                                                     max_chunks);
+    return me_check_launch("me_attention_prefill_combine");
+  }
+  return 0;
 }

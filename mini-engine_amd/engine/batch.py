@@ -67,6 +67,8 @@ class StepBatch:
         self.max_qlen = 1
         self.max_ctx = 1
         self.decode_only = True
+        # what parts derive from this step's items for all of their layers (work lists and the like)
+        self.derived: dict = {}
 
     def block_table(self, group: int) -> torch.Tensor:
         return self._tables[group]

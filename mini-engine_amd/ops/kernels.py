@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import ctypes
 
+import numpy as np
 import torch
 
 from .library import check, lib
@@ -486,11 +487,86 @@ def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write
     return out
 
 
+_PARTIAL_BYTES_MAX = 256 << 20  # most memory the partial results of cut tiles may take
+
+
+class PrefillPlan:
+    """The work list of one step's prefill attention, on the device: which tile of query tokens meets
+    which range of keys, heaviest first. It depends on the step's items and on the attention's window,
+    not on the layer, so a step builds it once."""
+
+    def __init__(self, work: torch.Tensor, token_chunks: torch.Tensor | None, num_work: int, max_chunks: int):
+        self.work, self.token_chunks, self.num_work, self.max_chunks = work, token_chunks, num_work, max_chunks
+
+
+def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int,
+                      partial_row_bytes: int = 0):
+    """Host side of :class:`PrefillPlan`: (entries int32 [n, 8], chunks per token int32 [T], max chunks).
+
+    A tile of ``tpb`` query tokens of an item meets the keys from its window's first (rounded down to a
+    multiple of 64) to its last token's position: ``n`` key tiles of 64. Every entry runs once per kv
+    head. When that gives fewer blocks than the chip has compute units (``slots``), a short portion of
+    a prompt over a long context for instance, tiles longer than ``cap`` key tiles, ``cap`` being the
+    work per compute unit if it were spread evenly, are cut into ranges of at most ``cap``, whose
+    partial results a second kernel adds up. Entries are sorted by length, longest first: the hardware
+    starts blocks in that order. An entry is (item, first token, tokens, first position, first key,
+    last key, chunk or -1, 0)."""
+    rows = []  # item, first token, tokens, first position, first key, last key, key tiles
+    offset = 0
+    for i, (s0, n) in enumerate(zip(starts, qlens)):
+        tiles = np.arange(-(-n // tpb), dtype=np.int64)
+        count = np.minimum(tpb, n - tiles * tpb)
+        p_first = s0 + tiles * tpb
+        p_last = p_first + count - 1
+        lo = np.maximum(p_first - window + 1, 0) if window > 0 else np.zeros_like(p_first)
+        k0 = (lo // 64) * 64
+        nt = (p_last - k0) // 64 + 1
+        rows.append(np.stack([np.full_like(tiles, i), offset + tiles * tpb, count, p_first, k0, p_last, nt], axis=1))
+        offset += n
+    rows = np.concatenate(rows, axis=0)
+    nc = np.ones(rows.shape[0], dtype=np.int64)
+    if rows.shape[0] * nkv < slots:
+        cap = max(4, -(-int(rows[:, 6].sum()) * nkv // slots))
+        while True:
+            nc = -(-rows[:, 6] // cap)
+            if int(nc.max()) == 1 or partial_row_bytes * int(nc.max()) * offset <= _PARTIAL_BYTES_MAX:
+                break
+            cap *= 2
+    max_chunks = int(nc.max())
+    token_chunks = np.ones(offset, dtype=np.int32)
+    entries = []
+    for (item, tb, count, p_first, k0, p_last, nt), c in zip(rows.tolist(), nc.tolist()):
+        if c == 1:
+            entries.append((nt, item, tb, count, p_first, k0, p_last, -1))
+            continue
+        token_chunks[tb:tb + count] = c
+        for j in range(c):
+            t0, t1 = j * nt // c, (j + 1) * nt // c
+            entries.append((t1 - t0, item, tb, count, p_first, k0 + 64 * t0, min(p_last, k0 + 64 * t1 - 1), j))
+    entries.sort(key=lambda e: -e[0])
+    work = np.zeros((len(entries), 8), dtype=np.int32)
+    work[:, :7] = np.array([e[1:] for e in entries], dtype=np.int64)
+    return work, token_chunks, max_chunks
+
+
+def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device) -> PrefillPlan:
+    tpb = lib().me_attention_prefill_columns() // (nh // nkv)
+    slots = torch.cuda.get_device_properties(device).multi_processor_count
+    work, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4)
+    if max_chunks == 1:
+        return PrefillPlan(torch.from_numpy(work.reshape(-1)).to(device), None, work.shape[0], 1)
+    both = torch.from_numpy(np.concatenate([work.reshape(-1), token_chunks])).to(device)  # one upload
+    return PrefillPlan(both[: work.size], both[work.size:], work.shape[0], max_chunks)
+
+
 def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: list[int], block_table, scale: float,
-                           window: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
+                           window: int = 0, out: torch.Tensor | None = None, starts: list[int] | None = None,
+                           plan: PrefillPlan | None = None) -> torch.Tensor:
     """Causal attention of packed new tokens q [T, nh, d] bfloat16 over the paged cache (which already
     holds the new tokens' keys and values). item_start int32 [items + 1] are the items' offsets into
-    the packed tokens, ``qlens`` the same lengths on the host (they size the grid)."""
+    the packed tokens, ``qlens`` the same lengths on the host and ``starts`` the position of each item's
+    first token (read back from ``positions`` when not given); ``plan`` is what :func:`prefill_plan`
+    makes of them, for callers that run several layers on one step."""
     _want(q, "q", torch.bfloat16, (None, None, None))
     t, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -504,13 +580,21 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
     group = nh // nkv
     if group > 16:
         raise ValueError(f"group size {group} exceeds what the matrix-core prefill kernel takes (16)")
-    tpb = lib().me_attention_prefill_columns() // group
-    num_blocks = sum(-(-n // tpb) for n in qlens)
+    if plan is None:
+        if starts is None:
+            firsts = np.concatenate([[0], np.cumsum(qlens)[:-1]])
+            starts = positions[torch.from_numpy(firsts).to(positions.device)].tolist()
+        plan = prefill_plan(starts, qlens, nh, nkv, d, window, q.device)
     if out is None:
         out = torch.empty((t, nh * d), dtype=torch.bfloat16, device=q.device)
     _want(out, "out", torch.bfloat16, (t, nh * d))
+    part_o = part_ml = None
+    if plan.max_chunks > 1:
+        part_o = torch.empty((t * nh * plan.max_chunks * d,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((t * nh * plan.max_chunks * 2,), dtype=torch.float32, device=q.device)
     check(lib().me_attention_prefill_bf16(
-        _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(item_start), _i(items), _p(block_table),
-        _i(block_table.shape[1]), _p(out), _i(num_blocks), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
+        _p(q), _p(k_cache), _p(v_cache), _i(items), _p(block_table),
+        _i(block_table.shape[1]), _p(out), _p(plan.work), _i(plan.num_work), _p(part_o), _p(part_ml),
+        _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
         _stream()))
     return out

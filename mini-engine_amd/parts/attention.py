@@ -111,8 +111,13 @@ class Attention(Mixer):
             if batch.decode_only:
                 return K.attention_decode_bf16(q, b.k_cache, b.v_cache, batch.item_ctx, table, scale, window,
                                                batch.max_ctx)
+            key = ("prefill_plan", self.nh, self.nkv, self.d, window)
+            plan = batch.derived.get(key)
+            if plan is None:  # the same for every layer of this shape: made once per step
+                plan = K.prefill_plan(batch.starts, batch.qlens, self.nh, self.nkv, self.d, window, q.device)
+                batch.derived[key] = plan
             return K.attention_prefill_bf16(q, b.k_cache, b.v_cache, batch.positions, batch.item_start, batch.qlens,
-                                            table, scale, window)
+                                            table, scale, window, plan=plan)
         return K.attention_general(q, b.k_cache, b.v_cache, batch.positions, batch.token_item, table, scale, window)
 
 

@@ -456,6 +456,36 @@ def test_attention_prefill_mfma(nh, nkv, d, bs, window):
     torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs,window", [(4, 2, 64, 16, 0), (16, 8, 128, 16, 0), (3, 1, 96, 64, 900)])
+def test_attention_prefill_cuts_long_tiles_when_the_step_is_small(nh, nkv, d, bs, window):
+    """A short portion over a long context: too few tiles to fill the chip, so their keys are cut into
+    ranges and added up by the second kernel. One far key dominates a head, so that a range that is
+    dropped or weighted wrongly shows; a second, short item stays in one piece beside it."""
+    dtype = torch.bfloat16
+    items = [(3000, 70), (0, 5)]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=256)
+    g = torch.Generator().manual_seed(11)
+    qs = [torch.randn(n, nh, d, generator=g).to(dtype) for _, n in items]
+    far = 2500
+    ks[0][far, 0] = (qs[0][3, 0].float() * 1.5).to(dtype)  # token 3, head 0 of item 0 looks at key 2500
+    k_cache[tables[0][far // bs], :, far % bs, :] = ks[0][far]
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    scale = d**-0.5
+    qlens = [n for _, n in items]
+    starts = [c for c, _ in items]
+    item_start = torch.tensor([0] + torch.tensor(qlens).cumsum(0).tolist(), dtype=torch.int32)
+    plan = K().prefill_plan(starts, qlens, nh, nkv, d, window, torch.device("cuda:0"))
+    assert plan.max_chunks > 1
+    out = K().attention_prefill_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(positions), dev(item_start),
+                                     qlens, dev(table_t), scale, window, plan=plan)
+    want = dense_reference(qs, ks, vs, items, scale, window)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    # and without a plan from the caller: the item starts are read back from the positions
+    out2 = K().attention_prefill_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(positions), dev(item_start),
+                                      qlens, dev(table_t), scale, window)
+    assert torch.equal(out, out2)
+
+
 @pytest.mark.parametrize("nh,nkv,d,bs", [(4, 2, 64, 16), (16, 8, 128, 16), (6, 1, 128, 32), (2, 2, 256, 16)])
 @pytest.mark.parametrize("norm,rotary,window", [(True, True, 0), (False, True, 37), (True, False, 0)])
 def test_attention_decode_fused_equals_the_two_kernels(nh, nkv, d, bs, norm, rotary, window):

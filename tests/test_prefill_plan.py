@@ -1,0 +1,61 @@
+"""The host-side work list of the prefill attention kernel: every tile of query tokens meets exactly
+the keys it may see, in one piece or in ranges that tile its keys without gap or overlap."""
+
+import random
+
+import numpy as np
+
+from mini_engine_amd.ops.kernels import prefill_work_list
+
+
+def check_plan(starts, qlens, tpb, window, nkv, slots):
+    work, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, partial_row_bytes=4096)
+    offsets = np.concatenate([[0], np.cumsum(qlens)])
+    assert token_chunks.shape == (offsets[-1],)
+    by_tile = {}
+    for item, tb, count, p_first, k0, k_last, chunk, pad in work.tolist():
+        assert pad == 0 and k0 % 64 == 0 and k0 <= k_last
+        by_tile.setdefault((item, tb, count, p_first), []).append((chunk, k0, k_last))
+    # every tile of every item is there, with the right tokens and positions
+    want_tiles = set()
+    for i, (s0, n) in enumerate(zip(starts, qlens)):
+        for t in range(-(-n // tpb)):
+            want_tiles.add((i, int(offsets[i]) + t * tpb, min(tpb, n - t * tpb), s0 + t * tpb))
+    assert set(by_tile) == want_tiles
+    for (item, tb, count, p_first), pieces in by_tile.items():
+        p_last = p_first + count - 1
+        lo = max(p_first - window + 1, 0) if window > 0 else 0
+        pieces.sort(key=lambda p: p[1])
+        if len(pieces) == 1:
+            assert pieces[0][0] == -1
+            assert (token_chunks[tb:tb + count] == 1).all()
+        else:
+            assert [p[0] for p in pieces] == list(range(len(pieces))) and len(pieces) <= max_chunks
+            assert (token_chunks[tb:tb + count] == len(pieces)).all()
+        assert pieces[0][1] == (lo // 64) * 64 and pieces[-1][2] == p_last
+        for (_, _, last), (_, nxt, _) in zip(pieces, pieces[1:]):
+            assert nxt == last + 1  # no gap, no overlap
+    lengths = [(e[5] - e[4]) // 64 + 1 for e in work.tolist()]
+    assert lengths == sorted(lengths, reverse=True)  # longest first
+    return work, max_chunks
+
+
+def test_whole_prompt_on_a_full_chip_is_not_cut():
+    work, max_chunks = check_plan([0], [2048], 64, 0, 8, 256)
+    assert max_chunks == 1 and work.shape[0] == 32
+
+
+def test_short_portion_over_long_context_is_cut_to_fill_the_chip():
+    work, max_chunks = check_plan([30000, 5], [64, 3], 64, 0, 8, 256)
+    assert max_chunks > 8
+    assert 128 <= work.shape[0] * 8 <= 512
+
+
+def test_random_steps():
+    rng = random.Random(0)
+    for _ in range(200):
+        n_items = rng.randint(1, 5)
+        starts = [rng.choice([0, 0, 3, 64, 1000, 5000]) for _ in range(n_items)]
+        qlens = [rng.choice([1, 2, 7, 64, 65, 200, 700]) for _ in range(n_items)]
+        check_plan(starts, qlens, rng.choice([8, 32, 64, 128]), rng.choice([0, 0, 37, 500]), rng.choice([1, 2, 8]),
+                   rng.choice([16, 256]))
