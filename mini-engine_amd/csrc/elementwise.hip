@@ -61,10 +61,90 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
   }
 }
 
+// The same for many bfloat16 rows (256 or more): a wave per row, the row in registers (CHUNKS x 8 elements per lane), 16-byte
+// loads and stores, no LDS and no barrier. dim is a multiple of 8 and at most 512 * CHUNKS.
+template <typename T, int CHUNKS>
+__global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                                                const float* __restrict__ w, T* __restrict__ h,
+                                                                const int* __restrict__ rows, int num_rows, int dim,
+                                                                float eps, int write_x) {
+  const int lane = threadIdx.x & (ME_WAVE - 1);
+  const int r = blockIdx.x * 4 + threadIdx.x / ME_WAVE;
+  if (r >= num_rows) return;
+  const int src = rows ? rows[r] : r;
+  float* xr = x + (size_t)src * dim;
+  const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+  float s[CHUNKS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int e = (c * ME_WAVE + lane) * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[c][j] = 0.f;
+    if (e < dim) {
+      const float4 a = *reinterpret_cast<const float4*>(xr + e), b = *reinterpret_cast<const float4*>(xr + e + 4);
+      s[c][0] = a.x, s[c][1] = a.y, s[c][2] = a.z, s[c][3] = a.w, s[c][4] = b.x, s[c][5] = b.y, s[c][6] = b.z, s[c][7] = b.w;
+      if (dr) {
+        struct alignas(sizeof(T) * 8) Pack {
+          T v[8];
+        };
+        const Pack d = *reinterpret_cast<const Pack*>(dr + e);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[c][j] += to_float(d.v[j]);
+        if (write_x) {
+          *reinterpret_cast<float4*>(xr + e) = make_float4(s[c][0], s[c][1], s[c][2], s[c][3]);
+          *reinterpret_cast<float4*>(xr + e + 4) = make_float4(s[c][4], s[c][5], s[c][6], s[c][7]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = fmaf(s[c][j], s[c][j], ss);
+    }
+  }
+  const float inv = rsqrtf(wave_sum(ss) / (float)dim + eps);
+  T* hr = h + (size_t)r * dim;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int e = (c * ME_WAVE + lane) * 8;
+    if (e < dim) {
+      const float4 a = *reinterpret_cast<const float4*>(w + e), b = *reinterpret_cast<const float4*>(w + e + 4);
+      const float wv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      struct alignas(sizeof(T) * 8) Pack {
+        T v[8];
+      } o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o.v[j] = from_float<T>(s[c][j] * inv * wv[j]);
+      *reinterpret_cast<Pack*>(hr + e) = o;
+    }
+  }
+}
+
+template <typename T>
+static bool launch_add_rmsnorm_rows(float* x, const T* delta, const float* w, T* h, const int* rows, int num_rows, int dim,
+                                    float eps, int write_x, hipStream_t stream) {
+  if (num_rows < 256 || dim % 8 || dim > 4096) return false;
+  if (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)h) & 15) return false;
+  const unsigned blocks = (num_rows + 3) / 4;
+#define ME_ROWS_CASE(C) add_rmsnorm_rows_kernel<T, C><<<blocks, 256, 0, stream>>>(x, delta, w, h, rows, num_rows, dim, eps, write_x)
+  if (dim <= 512)
+    ME_ROWS_CASE(1);
+  else if (dim <= 1024)
+    ME_ROWS_CASE(2);
+  else if (dim <= 2048)
+    ME_ROWS_CASE(4);
+  else
+    ME_ROWS_CASE(8);
+#undef ME_ROWS_CASE
+  return true;
+}
+
 extern "C" int me_add_rmsnorm(void* x, const void* delta, const float* w, void* h, const int* rows,
                               int num_rows, int dim, float eps, int write_x, int dtype, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   if (dim <= 0) return me_fail("me_add_rmsnorm: dim=%d", dim);
+  // bfloat16 only: in float32 the order of a row's sum stays the same for every number of rows
+  if (dtype == ME_BF16 && launch_add_rmsnorm_rows<bf16_t>((float*)x, (const bf16_t*)delta, w, (bf16_t*)h, rows, num_rows,
+                                                          dim, eps, write_x, stream))
+    return me_check_launch("me_add_rmsnorm");
   const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
   if (dtype == ME_F32)
     add_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((float*)x, (const float*)delta, w, (float*)h, rows,
