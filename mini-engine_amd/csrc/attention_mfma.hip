@@ -754,10 +754,12 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
   }
 }
 
-// One entry of the work list that the host lays out for a step (heaviest first): a tile of consecutive
-// query tokens of one item and a range of keys. The positions of an item's tokens are consecutive, so the
-// first one's stands for all. A tile whose keys are cut into several ranges gives partial results that
-// attention_prefill_combine_kernel adds up; `chunk` is -1 for a tile in one piece.
+// One entry of the work list that the host lays out for a step: a tile of consecutive query tokens of one
+// item and a range of keys. The positions of an item's tokens are consecutive, so the first one's stands
+// for all. A tile whose keys are cut into several ranges gives partial results that
+// attention_prefill_combine_kernel adds up; `chunk` is -1 for a tile in one piece. A block runs the
+// entries from its first one (bundle_first[block]) up to and including the next one marked `last`: the
+// host packs entries into bundles of about equal work when a step has too few tiles to go round.
 struct PrefillWork {
   int item;
   int token_begin, token_count;  // the tile's tokens among the packed tokens of the step
@@ -765,26 +767,27 @@ struct PrefillWork {
   int key_begin;                 // first key, a multiple of 64
   int key_last;                  // last key, inclusive
   int chunk;
-  int pad;
+  int last;
 };
 
 // WAVES waves per block, NB blocks of 16 query columns per wave: WAVES * NB * 16 = 128 columns.
 template <int D, int NB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-    const PrefillWork* __restrict__ work, const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window, float scale_log2,
-    int tokens_per_block) {
+    const PrefillWork* __restrict__ work, const int* __restrict__ bundle_first, const int* __restrict__ block_table,
+    int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
+    int nh, int nkv, int bs_shift, int window, float scale_log2, int tokens_per_block) {
   constexpr int THREADS = WAVES * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
   using L = PrefillLds<D>;
-  const PrefillWork w = work[blockIdx.x / nkv];  // the same for every lane: scalar loads
-  const int item = w.item;
   const int kvh = blockIdx.x % nkv;
   const int group = nh / nkv;
   const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
+  for (int wi = bundle_first[blockIdx.x / nkv];; ++wi) {
+  const PrefillWork w = work[wi];  // the same for every lane: scalar loads
+  const int item = w.item;
   const int t_begin = w.token_begin, t_end = w.token_begin + w.token_count;
   const int* table = block_table + (size_t)item * table_width;
 
@@ -878,19 +881,21 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) *reinterpret_cast<float4_t*>(part_o + slot * D + dt * 16 + g * 4) = acc[nb][dt];
     }
-    return;
-  }
+  } else {
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    if (!col_ok[nb]) continue;
-    const float inv = 1.f / lsum[nb];
-    bf16_t* orow = out + ((size_t)tok[nb] * nh + head[nb]) * D;
+    for (int nb = 0; nb < NB; ++nb) {
+      if (!col_ok[nb]) continue;
+      const float inv = 1.f / lsum[nb];
+      bf16_t* orow = out + ((size_t)tok[nb] * nh + head[nb]) * D;
 #pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt) {
-      const short4_t o = pack_bf16x4(acc[nb][dt][0] * inv, acc[nb][dt][1] * inv, acc[nb][dt][2] * inv,
-                                     acc[nb][dt][3] * inv);
-      *reinterpret_cast<short4_t*>(orow + dt * 16 + g * 4) = o;
+      for (int dt = 0; dt < D / 16; ++dt) {
+        const short4_t o = pack_bf16x4(acc[nb][dt][0] * inv, acc[nb][dt][1] * inv, acc[nb][dt][2] * inv,
+                                       acc[nb][dt][3] * inv);
+        *reinterpret_cast<short4_t*>(orow + dt * 16 + g * 4) = o;
+      }
     }
+  }
+  if (w.last) break;  // (the loop over keys ended with a barrier: LDS is free for the next entry)
   }
 }
 
@@ -943,7 +948,7 @@ extern "C" int me_attention_prefill_columns() { return PF_COLUMNS; }
 
 template <int D>
 static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const PrefillWork* work,
-                          const int* table, int width, bf16_t* out,
+                          const int* bundle_first, const int* table, int width, bf16_t* out,
                           float* part_o, float* part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window,
                           float sl, int tpb, hipStream_t stream) {
   static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
@@ -955,21 +960,23 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
     configured = true;
   }
   attention_prefill_kernel<D, PF_NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
-      q, kc, vc, work, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb);
+      q, kc, vc, work, bundle_first, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb);
   return 0;
 }
 
-// q [T, nh, d], packed new tokens. work: num_work entries of eight ints laid out by the caller (item, first
-// token and number of tokens of the tile (at most me_attention_prefill_columns() / group), position of the
-// first token, first key (a multiple of 64), last key, chunk or -1, one unused); every entry is run for
-// every kv head. When a tile's keys are cut into chunks (max_chunks > 1), part_o float
-// [T, nh, max_chunks, d] and part_ml float [T, nh, max_chunks, 2] take the partial results and
-// token_chunks int [T] says how many chunks each token's tile has (1: in one piece).
+// q [T, nh, d], packed new tokens. work: entries of eight ints laid out by the caller (item, first token and
+// number of tokens of the tile (at most me_attention_prefill_columns() / group), position of the first
+// token, first key (a multiple of 64), last key, chunk or -1, 1 on the last entry of a bundle);
+// bundle_first int [num_bundles]: the first entry of each bundle. Every bundle is run by one block per kv
+// head. When a tile's keys are cut into chunks (max_chunks > 1), part_o float [T, nh, max_chunks, d] and
+// part_ml float [T, nh, max_chunks, 2] take the partial results and token_chunks int [T] says how many
+// chunks each token's tile has (1: in one piece).
 extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items,
                                          const int* block_table, int table_width, void* out, const int* work,
-                                         int num_work, float* part_o, float* part_ml, const int* token_chunks,
-                                         int max_chunks, int num_tokens, int nh, int nkv, int d, int bs, int window,
-                                         float scale, hipStream_t stream) {
+                                         const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
+                                         const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
+                                         int d, int bs, int window, float scale, hipStream_t stream) {
+  const int num_work = num_bundles;
   if (num_items <= 0 || num_work <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_prefill_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
@@ -978,7 +985,7 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   if (group > 16) return me_fail("me_attention_prefill_bf16: group size %d exceeds 16", group);
   if ((long long)num_work * nkv > 0x7fffffffLL) return me_fail("me_attention_prefill_bf16: %d x %d blocks exceed the grid", num_work, nkv);
   if (table_width <= 0) return me_fail("me_attention_prefill_bf16: empty block table");
-  if (!work) return me_fail("me_attention_prefill_bf16: no work list");
+  if (!work || !bundle_first) return me_fail("me_attention_prefill_bf16: no work list");
   if (max_chunks < 1 || (max_chunks > 1 && (!part_o || !part_ml || !token_chunks || num_tokens <= 0)))
     return me_fail("me_attention_prefill_bf16: %d chunks need the partial buffers and the chunk counts", max_chunks);
   const int tpb = PF_COLUMNS / group;
@@ -990,7 +997,8 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   int rc = 0;
 #define ME_PREFILL_CASE(DD)                                                                                        \
   case DD:                                                                                                         \
-    rc = launch_prefill<DD>(grid, qq, kc, vc, (const PrefillWork*)work, block_table, table_width, (bf16_t*)out,   \
+    rc = launch_prefill<DD>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table, table_width,    \
+                            (bf16_t*)out,                                                                          \
                             part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb, stream);              \
     break;
   switch (d) {

@@ -492,25 +492,59 @@ _PARTIAL_BYTES_MAX = 256 << 20  # most memory the partial results of cut tiles m
 
 class PrefillPlan:
     """The work list of one step's prefill attention, on the device: which tile of query tokens meets
-    which range of keys, heaviest first. It depends on the step's items and on the attention's window,
-    not on the layer, so a step builds it once."""
+    which range of keys, and which block runs which entries. It depends on the step's items and on the
+    attention's window, not on the layer, so a step builds it once."""
 
-    def __init__(self, work: torch.Tensor, token_chunks: torch.Tensor | None, num_work: int, max_chunks: int):
-        self.work, self.token_chunks, self.num_work, self.max_chunks = work, token_chunks, num_work, max_chunks
+    def __init__(self, work: torch.Tensor, bundle_first: torch.Tensor, token_chunks: torch.Tensor | None,
+                 num_bundles: int, max_chunks: int):
+        self.work, self.bundle_first, self.token_chunks = work, bundle_first, token_chunks
+        self.num_bundles, self.max_chunks = num_bundles, max_chunks
+
+
+PIECE_OVERHEAD = 2  # what starting another piece of work costs a block, in key tiles (3 us against 1.5 us)
+
+
+def _cut(lengths: list[int], cap: int) -> list[tuple[int, int, int, int]]:
+    """Pieces (length, entry, chunk or -1, first key tile) of entries cut into ranges of at most ``cap``
+    key tiles: full ranges first, the remainder last (small remainders fill the gaps beside long pieces)."""
+    pieces = []
+    for i, n in enumerate(lengths):
+        if n <= cap:
+            pieces.append((n, i, -1, 0))
+            continue
+        for j, t0 in enumerate(range(0, n, cap)):
+            pieces.append((min(cap, n - t0), i, j, t0))
+    return pieces
+
+
+def _pack(pieces, bins: int):
+    """Longest piece first into the least loaded bin: (makespan, the bins' pieces)."""
+    import heapq
+
+    heap = [(0, b) for b in range(bins)]
+    loads: list[list] = [[] for _ in range(bins)]
+    for piece in sorted(pieces, key=lambda q: -q[0]):
+        load, b = heapq.heappop(heap)
+        loads[b].append(piece)
+        heapq.heappush(heap, (load + piece[0] + PIECE_OVERHEAD, b))
+    return max(load for load, _ in heap), loads
 
 
 def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int,
                       partial_row_bytes: int = 0):
-    """Host side of :class:`PrefillPlan`: (entries int32 [n, 8], chunks per token int32 [T], max chunks).
+    """Host side of :class:`PrefillPlan`: (entries int32 [n, 8], first entry of each bundle int32 [b],
+    chunks per token int32 [T], max chunks).
 
     A tile of ``tpb`` query tokens of an item meets the keys from its window's first (rounded down to a
-    multiple of 64) to its last token's position: ``n`` key tiles of 64. Every entry runs once per kv
-    head. When that gives fewer blocks than the chip has compute units (``slots``), a short portion of
-    a prompt over a long context for instance, tiles longer than ``cap`` key tiles, ``cap`` being the
-    work per compute unit if it were spread evenly, are cut into ranges of at most ``cap``, whose
-    partial results a second kernel adds up. Entries are sorted by length, longest first: the hardware
-    starts blocks in that order. An entry is (item, first token, tokens, first position, first key,
-    last key, chunk or -1, 0)."""
+    multiple of 64) to its last token's position: ``n`` key tiles of 64. A bundle of entries is run by one
+    block per kv head. With at least two tiles per compute unit and kv head the bundles are the tiles,
+    longest first (the hardware starts blocks in that order and evens them out). With fewer (a prompt
+    of a few thousand tokens, whose causal tiles differ in length by a factor of their number; a short
+    portion over a long context) the tiles are cut into ranges of at most ``cap`` key tiles, whose
+    partial results a second kernel adds up, and the pieces are packed into one bundle per compute
+    unit, longest piece first into the emptiest bundle; ``cap`` is the candidate with the shortest
+    longest bundle. An entry is (item, first token, tokens, first position, first key, last key, chunk
+    or -1, 1 if its bundle ends with it)."""
     rows = []  # item, first token, tokens, first position, first key, last key, key tiles
     offset = 0
     for i, (s0, n) in enumerate(zip(starts, qlens)):
@@ -523,40 +557,65 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
         nt = (p_last - k0) // 64 + 1
         rows.append(np.stack([np.full_like(tiles, i), offset + tiles * tpb, count, p_first, k0, p_last, nt], axis=1))
         offset += n
-    rows = np.concatenate(rows, axis=0)
-    nc = np.ones(rows.shape[0], dtype=np.int64)
-    if rows.shape[0] * nkv < slots:
-        cap = max(4, -(-int(rows[:, 6].sum()) * nkv // slots))
-        while True:
-            nc = -(-rows[:, 6] // cap)
-            if int(nc.max()) == 1 or partial_row_bytes * int(nc.max()) * offset <= _PARTIAL_BYTES_MAX:
-                break
-            cap *= 2
-    max_chunks = int(nc.max())
+    rows = np.concatenate(rows, axis=0).tolist()
+    lengths = [r[6] for r in rows]
+    bins = max(1, slots // max(1, nkv))
+    longest, total = max(lengths), sum(lengths)
+    if len(rows) >= 2 * bins:
+        bundles = [[piece] for piece in sorted(_cut(lengths, longest), key=lambda q: -q[0])]
+    else:
+        chunk_limit = 1 << 30
+        if partial_row_bytes:
+            chunk_limit = max(1, _PARTIAL_BYTES_MAX // (partial_row_bytes * offset))
+        caps = {longest, -(-total // bins), -(-total // (2 * bins)), -(-longest // 2), -(-longest // 3)}
+        best = None
+        for cap in sorted(c for c in caps if c >= 1 and -(-longest // c) <= chunk_limit):
+            pieces = _cut(lengths, cap)
+            span, loads = _pack(pieces, bins)
+            score = (span + 0.01 * len(pieces), cap)
+            if best is None or score < best[0]:
+                best = (score, loads)
+        bundles = sorted((b for b in best[1] if b), key=lambda b: -sum(q[0] for q in b))
     token_chunks = np.ones(offset, dtype=np.int32)
-    entries = []
-    for (item, tb, count, p_first, k0, p_last, nt), c in zip(rows.tolist(), nc.tolist()):
-        if c == 1:
-            entries.append((nt, item, tb, count, p_first, k0, p_last, -1))
-            continue
-        token_chunks[tb:tb + count] = c
-        for j in range(c):
-            t0, t1 = j * nt // c, (j + 1) * nt // c
-            entries.append((t1 - t0, item, tb, count, p_first, k0 + 64 * t0, min(p_last, k0 + 64 * t1 - 1), j))
-    entries.sort(key=lambda e: -e[0])
-    work = np.zeros((len(entries), 8), dtype=np.int32)
-    work[:, :7] = np.array([e[1:] for e in entries], dtype=np.int64)
-    return work, token_chunks, max_chunks
+    chunks_of = {}
+    for bundle in bundles:
+        for _, i, chunk, _ in bundle:
+            chunks_of[i] = max(chunks_of.get(i, 1), chunk + 1)
+    work, bundle_first = [], []
+    for bundle in bundles:
+        bundle_first.append(len(work))
+        for n, i, chunk, t0 in bundle:
+            item, tb, count, p_first, k0, p_last, _ = rows[i]
+            work.append((item, tb, count, p_first, k0 + 64 * t0, min(p_last, k0 + 64 * (t0 + n) - 1), chunk, 0))
+        work[-1] = work[-1][:7] + (1,)
+    for i, c in chunks_of.items():
+        if c > 1:
+            token_chunks[rows[i][1]:rows[i][1] + rows[i][2]] = c
+    return (np.array(work, dtype=np.int32), np.array(bundle_first, dtype=np.int32), token_chunks,
+            max(chunks_of.values()))
+
+
+_PLANS: dict = {}  # the last plans made, by what they were made from: steps of a serving loop repeat
 
 
 def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device) -> PrefillPlan:
+    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device))
+    plan = _PLANS.get(key)
+    if plan is None:
+        if len(_PLANS) >= 64:
+            _PLANS.pop(next(iter(_PLANS)))
+        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device)
+    return plan
+
+
+def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device) -> PrefillPlan:
     tpb = lib().me_attention_prefill_columns() // (nh // nkv)
     slots = torch.cuda.get_device_properties(device).multi_processor_count
-    work, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4)
-    if max_chunks == 1:
-        return PrefillPlan(torch.from_numpy(work.reshape(-1)).to(device), None, work.shape[0], 1)
-    both = torch.from_numpy(np.concatenate([work.reshape(-1), token_chunks])).to(device)  # one upload
-    return PrefillPlan(both[: work.size], both[work.size:], work.shape[0], max_chunks)
+    work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4)
+    parts = [work.reshape(-1), first] + ([token_chunks] if max_chunks > 1 else [])
+    both = torch.from_numpy(np.concatenate(parts)).to(device)  # one upload
+    a, b = work.size, work.size + first.size
+    return PrefillPlan(both[:a], both[a:b], both[b:] if max_chunks > 1 else None, first.size, max_chunks)
 
 
 def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: list[int], block_table, scale: float,
@@ -594,7 +653,7 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
         part_ml = torch.empty((t * nh * plan.max_chunks * 2,), dtype=torch.float32, device=q.device)
     check(lib().me_attention_prefill_bf16(
         _p(q), _p(k_cache), _p(v_cache), _i(items), _p(block_table),
-        _i(block_table.shape[1]), _p(out), _p(plan.work), _i(plan.num_work), _p(part_o), _p(part_ml),
+        _i(block_table.shape[1]), _p(out), _p(plan.work), _p(plan.bundle_first), _i(plan.num_bundles), _p(part_o), _p(part_ml),
         _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
         _stream()))
     return out

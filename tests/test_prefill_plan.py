@@ -9,12 +9,18 @@ from mini_engine_amd.ops.kernels import prefill_work_list
 
 
 def check_plan(starts, qlens, tpb, window, nkv, slots):
-    work, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, partial_row_bytes=4096)
+    work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots,
+                                                              partial_row_bytes=4096)
     offsets = np.concatenate([[0], np.cumsum(qlens)])
     assert token_chunks.shape == (offsets[-1],)
+    # bundles: every entry belongs to exactly one, each ends with its only `last` mark
+    assert first[0] == 0 and (np.diff(first) > 0).all() and first[-1] < work.shape[0]
+    ends = set((first[1:] - 1).tolist()) | {work.shape[0] - 1}
+    assert {i for i, e in enumerate(work.tolist()) if e[7] == 1} == ends
+    assert len(first) <= max(slots // nkv, 1) or len(first) == work.shape[0]
     by_tile = {}
-    for item, tb, count, p_first, k0, k_last, chunk, pad in work.tolist():
-        assert pad == 0 and k0 % 64 == 0 and k0 <= k_last
+    for item, tb, count, p_first, k0, k_last, chunk, last in work.tolist():
+        assert last in (0, 1) and k0 % 64 == 0 and k0 <= k_last
         by_tile.setdefault((item, tb, count, p_first), []).append((chunk, k0, k_last))
     # every tile of every item is there, with the right tokens and positions
     want_tiles = set()
@@ -35,20 +41,32 @@ def check_plan(starts, qlens, tpb, window, nkv, slots):
         assert pieces[0][1] == (lo // 64) * 64 and pieces[-1][2] == p_last
         for (_, _, last), (_, nxt, _) in zip(pieces, pieces[1:]):
             assert nxt == last + 1  # no gap, no overlap
-    lengths = [(e[5] - e[4]) // 64 + 1 for e in work.tolist()]
-    assert lengths == sorted(lengths, reverse=True)  # longest first
-    return work, max_chunks
+    return work, first, max_chunks
 
 
-def test_whole_prompt_on_a_full_chip_is_not_cut():
-    work, max_chunks = check_plan([0], [2048], 64, 0, 8, 256)
-    assert max_chunks == 1 and work.shape[0] == 32
+def bundle_loads(work, first):
+    bounds = first.tolist() + [work.shape[0]]
+    return [sum((e[5] - e[4]) // 64 + 1 for e in work[a:b].tolist()) for a, b in zip(bounds, bounds[1:])]
+
+
+def test_many_tiles_are_left_whole_longest_first():
+    work, first, max_chunks = check_plan([0], [4096], 64, 0, 8, 256)
+    assert max_chunks == 1 and work.shape[0] == 64 and len(first) == 64
+    loads = bundle_loads(work, first)
+    assert loads == sorted(loads, reverse=True)
+
+
+def test_causal_prompt_with_one_tile_per_compute_unit_is_evened_out():
+    work, first, max_chunks = check_plan([0], [2048], 64, 0, 8, 256)
+    loads = bundle_loads(work, first)
+    assert len(first) == 32 and max_chunks == 2
+    assert max(loads) <= 20 < 32  # whole tiles would give 32 key tiles to the last block
 
 
 def test_short_portion_over_long_context_is_cut_to_fill_the_chip():
-    work, max_chunks = check_plan([30000, 5], [64, 3], 64, 0, 8, 256)
-    assert max_chunks > 8
-    assert 128 <= work.shape[0] * 8 <= 512
+    work, first, max_chunks = check_plan([30000, 5], [64, 3], 64, 0, 8, 256)
+    assert max_chunks > 8 and len(first) == 32
+    assert max(bundle_loads(work, first)) <= 20
 
 
 def test_random_steps():
