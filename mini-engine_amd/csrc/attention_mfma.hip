@@ -725,14 +725,18 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
                        (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
     lsum[nb] = fmaf(lsum[nb], alpha, column_sum(psum));
     m[nb] = m_new;
-    // (a branch that skips the rescale when no column's maximum moved costs more than it saves: the
-    // accumulator then lives in two sets of registers and is copied where it is not multiplied)
+    // The running maximum rarely moves after the first tiles: the rescale of the accumulator is skipped
+    // when no column of the wave needs it. The multiplication is written as instructions that work in
+    // place: as plain C++ under a branch the accumulator ends up in two sets of registers and is copied
+    // on the path that does not multiply, which costs more than multiplying always.
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt) {
-      acc[nb][dt][0] *= alpha;
-      acc[nb][dt][1] *= alpha;
-      acc[nb][dt][2] *= alpha;
-      acc[nb][dt][3] *= alpha;
+      for (int dt = 0; dt < D / 16; ++dt) {
+        float a0 = acc[nb][dt][0], a1 = acc[nb][dt][1], a2 = acc[nb][dt][2], a3 = acc[nb][dt][3];
+        asm volatile("v_mul_f32 %0, %0, %4\n v_mul_f32 %1, %1, %4\n v_mul_f32 %2, %2, %4\n v_mul_f32 %3, %3, %4"
+                     : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3) : "v"(alpha));
+        acc[nb][dt] = (float4_t){a0, a1, a2, a3};
+      }
     }
     // the B operand of the second product: for each half of 32 keys, the lane's four keys of the first
     // score tile and then those of the second
