@@ -537,31 +537,29 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
 
     A tile of ``tpb`` query tokens of an item meets the keys from its window's first (rounded down to a
     multiple of 64) to its last token's position: ``n`` key tiles of 64. A bundle of entries is run by one
-    block per kv head. With at least two tiles per compute unit and kv head the bundles are the tiles,
-    longest first (the hardware starts blocks in that order and evens them out). With fewer (a prompt
-    of a few thousand tokens, whose causal tiles differ in length by a factor of their number; a short
-    portion over a long context) the tiles are cut into ranges of at most ``cap`` key tiles, whose
-    partial results a second kernel adds up, and the pieces are packed into one bundle per compute
-    unit, longest piece first into the emptiest bundle; ``cap`` is the candidate with the shortest
-    longest bundle. An entry is (item, first token, tokens, first position, first key, last key, chunk
+    block per kv head. With more tiles than compute units per kv head the bundles are the tiles,
+    longest first (the hardware starts blocks in that order and evens them out). With at most that many
+    (a prompt of up to a few thousand tokens, whose causal tiles differ in length by a factor of their
+    number; a short portion over a long context) the tiles are cut into ranges of at most ``cap`` key
+    tiles, whose partial results a second kernel adds up, and the pieces are packed into one bundle per
+    compute unit, longest piece first into the emptiest bundle; ``cap`` is the candidate with the
+    shortest longest bundle. (Packing costs a few tenths of a millisecond on the host; steps that mix
+    decoded tokens with a portion have more tiles than that and skip it.) An entry is (item, first token, tokens, first position, first key, last key, chunk
     or -1, 1 if its bundle ends with it)."""
     rows = []  # item, first token, tokens, first position, first key, last key, key tiles
     offset = 0
     for i, (s0, n) in enumerate(zip(starts, qlens)):
-        tiles = np.arange(-(-n // tpb), dtype=np.int64)
-        count = np.minimum(tpb, n - tiles * tpb)
-        p_first = s0 + tiles * tpb
-        p_last = p_first + count - 1
-        lo = np.maximum(p_first - window + 1, 0) if window > 0 else np.zeros_like(p_first)
-        k0 = (lo // 64) * 64
-        nt = (p_last - k0) // 64 + 1
-        rows.append(np.stack([np.full_like(tiles, i), offset + tiles * tpb, count, p_first, k0, p_last, nt], axis=1))
+        for t0 in range(0, n, tpb):
+            count = min(tpb, n - t0)
+            p_first = s0 + t0
+            p_last = p_first + count - 1
+            k0 = (max(p_first - window + 1, 0) // 64) * 64 if window > 0 else 0
+            rows.append((i, offset + t0, count, p_first, k0, p_last, (p_last - k0) // 64 + 1))
         offset += n
-    rows = np.concatenate(rows, axis=0).tolist()
     lengths = [r[6] for r in rows]
     bins = max(1, slots // max(1, nkv))
     longest, total = max(lengths), sum(lengths)
-    if len(rows) >= 2 * bins:
+    if len(rows) > bins:
         bundles = [[piece] for piece in sorted(_cut(lengths, longest), key=lambda q: -q[0])]
     else:
         chunk_limit = 1 << 30

@@ -17,7 +17,7 @@ def check_plan(starts, qlens, tpb, window, nkv, slots):
     assert first[0] == 0 and (np.diff(first) > 0).all() and first[-1] < work.shape[0]
     ends = set((first[1:] - 1).tolist()) | {work.shape[0] - 1}
     assert {i for i, e in enumerate(work.tolist()) if e[7] == 1} == ends
-    assert len(first) <= max(slots // nkv, 1) or len(first) == work.shape[0]
+    assert len(first) <= max(slots // nkv, 1) or len(first) == work.shape[0]  # packed, or one tile per bundle
     by_tile = {}
     for item, tb, count, p_first, k0, k_last, chunk, last in work.tolist():
         assert last in (0, 1) and k0 % 64 == 0 and k0 <= k_last
