@@ -357,21 +357,22 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
 }
 
 // The same work for the common geometry (head size a power of two from 16 to 256, rotary over the
-// whole head or none): a lane owns the four dims (2p, 2p+1, 2p+d/2, 2p+1+d/2), i.e. two rotary pairs,
-// so no value has to cross lanes for the rotation, loads and stores are 4 bytes wide, and a wave
-// handles 64 / (d/4) heads at a time. Unit u of the grid is (token, head) = (u / heads, u % heads).
+// whole head or none): a lane owns eight consecutive dims of the lower half of a head and their rotary
+// partners half a head away, so no value has to cross lanes for the rotation, loads and stores are
+// 8 elements wide (16 bytes in bfloat16), and a wave handles 64 / (d/16) heads at a time. Unit u of the
+// grid is (token, head) = (u / heads, u % heads).
 template <typename T>
-struct Pair2 {
-  T a, b;
+struct alignas(sizeof(T) * 8) Pack8 {
+  T v[8];
 };
 
-template <typename T, int LPH>  // LPH = d / 4 lanes per head
-__global__ __launch_bounds__(256) void qk_norm_rope_scatter_quad_kernel(
+template <typename T, int LPH>  // LPH = d / 16 lanes per head
+__global__ __launch_bounds__(256) void qk_norm_rope_scatter_wide_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
     const float* __restrict__ rope_table, const int* __restrict__ positions, const int* __restrict__ token_item,
     const int* __restrict__ block_table, int table_width, T* __restrict__ q_out, T* __restrict__ k_cache,
     T* __restrict__ v_cache, int num_tokens, int nh, int nkv, int bs, float eps, int write_kv, int skip_v) {
-  constexpr int D = LPH * 4, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
+  constexpr int D = LPH * 16, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
   const int lane = threadIdx.x & (ME_WAVE - 1);
   const int sub = lane / LPH, p = lane % LPH;
   const int heads_row = write_kv ? nh + 2 * nkv : nh;
@@ -381,36 +382,57 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_quad_kernel(
   const int t = (int)(unit / heads), hd = (int)(unit % heads);
   const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
   const T* src = qkv + ((size_t)t * heads_row + hd) * D;
-  const Pair2<T> lo = *reinterpret_cast<const Pair2<T>*>(src + 2 * p);
-  const Pair2<T> hi = *reinterpret_cast<const Pair2<T>*>(src + 2 * p + HALF);
-  float v[4] = {to_float(lo.a), to_float(lo.b), to_float(hi.a), to_float(hi.b)};
+  const Pack8<T> lo = *reinterpret_cast<const Pack8<T>*>(src + 8 * p);
+  const Pack8<T> hi = *reinterpret_cast<const Pack8<T>*>(src + 8 * p + HALF);
+  float a[8], b[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    a[j] = to_float(lo.v[j]);
+    b[j] = to_float(hi.v[j]);
+  }
   const int pos = positions[t];
   const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
   if (w) {
-    float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss = fmaf(a[j], a[j], fmaf(b[j], b[j], ss));
 #pragma unroll
     for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, ME_WAVE);  // within the head's lanes
     const float inv = rsqrtf(ss / (float)D + eps);
-    v[0] *= inv * w[2 * p];
-    v[1] *= inv * w[2 * p + 1];
-    v[2] *= inv * w[2 * p + HALF];
-    v[3] *= inv * w[2 * p + 1 + HALF];
+    const float4 wa0 = *reinterpret_cast<const float4*>(w + 8 * p), wa1 = *reinterpret_cast<const float4*>(w + 8 * p + 4);
+    const float4 wb0 = *reinterpret_cast<const float4*>(w + 8 * p + HALF),
+                 wb1 = *reinterpret_cast<const float4*>(w + 8 * p + HALF + 4);
+    const float wa[8] = {wa0.x, wa0.y, wa0.z, wa0.w, wa1.x, wa1.y, wa1.z, wa1.w};
+    const float wb[8] = {wb0.x, wb0.y, wb0.z, wb0.w, wb1.x, wb1.y, wb1.z, wb1.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      a[j] *= inv * wa[j];
+      b[j] *= inv * wb[j];
+    }
   }
   if (kind != 2 && rope_table) {
-    const float* cs = rope_table + (size_t)pos * D;  // [2, HALF]: cosines then sines
-    const float c0 = cs[2 * p], c1 = cs[2 * p + 1], s0 = cs[HALF + 2 * p], s1 = cs[HALF + 2 * p + 1];
-    const float a0 = v[0] * c0 - v[2] * s0, b0 = v[2] * c0 + v[0] * s0;
-    const float a1 = v[1] * c1 - v[3] * s1, b1 = v[3] * c1 + v[1] * s1;
-    v[0] = a0;
-    v[1] = a1;
-    v[2] = b0;
-    v[3] = b1;
+    const float* cs = rope_table + (size_t)pos * D + 8 * p;  // [2, HALF]: cosines then sines
+    const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(cs + HALF), s1 = *reinterpret_cast<const float4*>(cs + HALF + 4);
+    const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float ra = a[j] * c[j] - b[j] * sn[j], rb = b[j] * c[j] + a[j] * sn[j];
+      a[j] = ra;
+      b[j] = rb;
+    }
   }
-  const Pair2<T> out_lo = {from_float<T>(v[0]), from_float<T>(v[1])}, out_hi = {from_float<T>(v[2]), from_float<T>(v[3])};
+  Pack8<T> out_lo, out_hi;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    out_lo.v[j] = from_float<T>(a[j]);
+    out_hi.v[j] = from_float<T>(b[j]);
+  }
   if (kind == 0) {
     T* dst = q_out + ((size_t)t * nh + hd) * D;
-    *reinterpret_cast<Pair2<T>*>(dst + 2 * p) = out_lo;
-    *reinterpret_cast<Pair2<T>*>(dst + 2 * p + HALF) = out_hi;
+    *reinterpret_cast<Pack8<T>*>(dst + 8 * p) = out_lo;
+    *reinterpret_cast<Pack8<T>*>(dst + 8 * p + HALF) = out_hi;
     return;
   }
   const int page = block_table[(size_t)token_item[t] * table_width + pos / bs];
@@ -418,40 +440,45 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_quad_kernel(
   const int slot = pos % bs;
   if (kind == 1) {
     T* dst = k_cache + (((size_t)page * nkv + (hd - nh)) * bs + slot) * D;
-    *reinterpret_cast<Pair2<T>*>(dst + 2 * p) = out_lo;
-    *reinterpret_cast<Pair2<T>*>(dst + 2 * p + HALF) = out_hi;
+    *reinterpret_cast<Pack8<T>*>(dst + 8 * p) = out_lo;
+    *reinterpret_cast<Pack8<T>*>(dst + 8 * p + HALF) = out_hi;
   } else {
     T* dst = v_cache + ((size_t)page * nkv + (hd - nh - nkv)) * D * bs + slot;
-    dst[(size_t)(2 * p) * bs] = out_lo.a;
-    dst[(size_t)(2 * p + 1) * bs] = out_lo.b;
-    dst[(size_t)(2 * p + HALF) * bs] = out_hi.a;
-    dst[(size_t)(2 * p + 1 + HALF) * bs] = out_hi.b;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      dst[(size_t)(8 * p + j) * bs] = out_lo.v[j];
+      dst[(size_t)(8 * p + j + HALF) * bs] = out_hi.v[j];
+    }
   }
 }
 
 template <typename T>
-static bool launch_quad(const T* qkv, const float* q_w, const float* k_w, const float* rope_table, const int* positions,
+static bool launch_wide(const T* qkv, const float* q_w, const float* k_w, const float* rope_table, const int* positions,
                         const int* token_item, const int* block_table, int table_width, T* q_out, T* k_cache,
                         T* v_cache, int num_tokens, int nh, int nkv, int d, int bs, float eps, int write_kv, int skip_v,
                         hipStream_t stream) {
+  // 8-element accesses need aligned bases (row lengths are multiples of the head size, itself one of 16)
+  const uintptr_t align = sizeof(T) * 8 - 1;
+  if (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache) & align) return false;
+  if (((uintptr_t)q_w | (uintptr_t)k_w | (uintptr_t)rope_table) & 15) return false;
   const int heads = write_kv ? (skip_v ? nh + nkv : nh + 2 * nkv) : nh;
   const long long units = (long long)num_tokens * heads;
-#define ME_QUAD(LPH)                                                                                                  \
+#define ME_WIDE(LPH)                                                                                                  \
   {                                                                                                                   \
     const long long per_block = 4 * (64 / LPH);                                                                       \
-    qk_norm_rope_scatter_quad_kernel<T, LPH><<<(unsigned)((units + per_block - 1) / per_block), 256, 0, stream>>>(    \
+    qk_norm_rope_scatter_wide_kernel<T, LPH><<<(unsigned)((units + per_block - 1) / per_block), 256, 0, stream>>>(    \
         qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, q_out, k_cache, v_cache,          \
         num_tokens, nh, nkv, bs, eps, write_kv, skip_v);                                                              \
     return true;                                                                                                      \
   }
   switch (d) {
-    case 16: ME_QUAD(4)
-    case 32: ME_QUAD(8)
-    case 64: ME_QUAD(16)
-    case 128: ME_QUAD(32)
-    case 256: ME_QUAD(64)
+    case 16: ME_WIDE(1)
+    case 32: ME_WIDE(2)
+    case 64: ME_WIDE(4)
+    case 128: ME_WIDE(8)
+    case 256: ME_WIDE(16)
   }
-#undef ME_QUAD
+#undef ME_WIDE
   return false;
 }
 
@@ -487,15 +514,35 @@ __global__ __launch_bounds__(256) void v_scatter_tiles_kernel(const T* __restric
   const int first = max(seg_pos, p0), last = min(seg_pos + 15, p0 + n - 1);  // positions present
   const int width = (nh + 2 * nkv) * d;
   const T* src = qkv + (size_t)(nh + nkv + kvh) * d;
-  for (int idx = threadIdx.x; idx < (last - first + 1) * d; idx += blockDim.x) {
-    const int row = idx / d, col = idx % d;
-    tile[first - seg_pos + row][col] = src[(size_t)(t0 + first - p0 + row) * width + col];
+  const bool wide = d % 8 == 0 && (((uintptr_t)qkv | (uintptr_t)v_cache) & (sizeof(T) * 8 - 1)) == 0;
+  if (wide) {  // rows in pieces of eight elements
+    for (int idx = threadIdx.x; idx < (last - first + 1) * (d / 8); idx += blockDim.x) {
+      const int row = idx / (d / 8), col = idx % (d / 8) * 8;
+      const Pack8<T> v = *reinterpret_cast<const Pack8<T>*>(src + (size_t)(t0 + first - p0 + row) * width + col);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) tile[first - seg_pos + row][col + j] = v.v[j];
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < (last - first + 1) * d; idx += blockDim.x) {
+      const int row = idx / d, col = idx % d;
+      tile[first - seg_pos + row][col] = src[(size_t)(t0 + first - p0 + row) * width + col];
+    }
   }
   __syncthreads();
   const int page = block_table[(size_t)item * table_width + seg_pos / bs];
   if (page < 0) return;
   T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + seg_pos % bs;
   const int lo = first - seg_pos, hi = last - seg_pos;
+  if (wide && lo == 0 && hi == 15) {  // a whole segment: eight slots of one dimension per store
+    for (int idx = threadIdx.x; idx < d * 2; idx += blockDim.x) {
+      const int dim = idx >> 1, half = idx & 1;
+      Pack8<T> v;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v.v[j] = tile[half * 8 + j][dim];
+      *reinterpret_cast<Pack8<T>*>(dst + (size_t)dim * bs + half * 8) = v;
+    }
+    return;
+  }
   for (int idx = threadIdx.x; idx < d * 16; idx += blockDim.x) {
     const int dim = idx / 16, slot = idx % 16;
     if (slot >= lo && slot <= hi) dst[(size_t)dim * bs + slot] = tile[slot][dim];
@@ -524,9 +571,9 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
   const int hpb = num_tokens >= 512 ? heads_total : 4;
   dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
   if (grid.y > 65535) return me_fail("me_qk_norm_rope_scatter: too many heads");
-  const bool quad = (rd == d || rope_table == nullptr) && (d & (d - 1)) == 0 && d >= 16 && d <= 256;
+  const bool wide = (rd == d || rope_table == nullptr) && (d & (d - 1)) == 0 && d >= 16 && d <= 256;
   if (dtype == ME_F32) {
-    if (!(quad && launch_quad<float>((const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
+    if (!(wide && launch_wide<float>((const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
                                      table_width, (float*)q_out, (float*)k_cache, (float*)v_cache, num_tokens, nh, nkv,
                                      d, bs, eps, write_kv, tiles ? 1 : 0, stream)))
       qk_norm_rope_scatter_kernel<float><<<grid, 256, 0, stream>>>(
@@ -536,7 +583,7 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
       v_scatter_tiles_kernel<float><<<dim3(num_segments, nkv), 256, 0, stream>>>(
           (const float*)qkv, positions, item_start, num_items, block_table, table_width, (float*)v_cache, nh, nkv, d, bs);
   } else {
-    if (!(quad && launch_quad<bf16_t>((const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
+    if (!(wide && launch_wide<bf16_t>((const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
                                       table_width, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, num_tokens, nh,
                                       nkv, d, bs, eps, write_kv, tiles ? 1 : 0, stream)))
       qk_norm_rope_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
