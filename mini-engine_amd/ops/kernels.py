@@ -333,6 +333,36 @@ def gemm_bf16_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
     return gemm_bf16_small(x, weight, out_dtype, False, out)
 
 
+TILED_MIN_ROWS = 256
+
+
+def gemm_bf16_tiled(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
+                    out: torch.Tensor | None = None, shape: int = 0) -> torch.Tensor:
+    """bfloat16 ``x @ weight.T`` for any number of rows with LDS-tiled matrix-core blocks, float32
+    accumulation; K must be a multiple of 64. With ``swiglu`` the weight holds gate rows then up rows,
+    [2N, K], and the result is ``silu(gate) * up`` [M, N] in bfloat16, without the [M, 2N] product ever
+    going to memory. ``shape`` names a block tile (0: the default)."""
+    _want(x, "x", torch.bfloat16, (None, None))
+    m, k = x.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0]
+    if swiglu:
+        if n % 2:
+            raise ValueError(f"a gate/up weight needs an even number of rows, got {n}")
+        n //= 2
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=weight.device)
+    _want(out, "out", out_dtype, (m, n))
+    check(lib().me_gemm_bf16_tiled(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(1 if swiglu else 0),
+                                   _i(_code(out_dtype)), _i(shape), _stream()))
+    return out
+
+
+def tiled_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (x.shape[0] >= TILED_MIN_ROWS and x.shape[1] % 64 == 0 and x.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0)
+
+
 def small_ok(x, weight: torch.Tensor, max_rows: int = SMALL_FAST_ROWS) -> bool:
     return (x.shape[0] <= max_rows and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0
             and weight.data_ptr() % 16 == 0)
@@ -343,8 +373,10 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     then up rows) and the result is ``silu(gate) * up``. ``x`` may be a :class:`NormedInput`.
 
     float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16: the
-    fused matrix-core kernel for up to 64 rows, else the GEMM library; rows are processed in slices
-    of 64 when a float32 result is wanted from bfloat16 inputs (logits)."""
+    fused matrix-core kernel for up to 16 rows; the tiled matrix-core kernel with the SwiGLU as its
+    epilogue for gated products of 256 rows or more; else the GEMM library (for the plain projections
+    of a prompt it is as fast as the tiled kernel or faster, measured). Rows are processed in slices of
+    64 when a float32 result is wanted from bfloat16 inputs (logits) and the library cannot give one."""
     if isinstance(x, NormedInput):
         if x.fusable(weight):
             return gemm_bf16_small(x, weight, out_dtype or x.dtype, gated)
@@ -358,6 +390,8 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     if small_ok(x, weight):
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if gated:
+        if tiled_ok(x, weight) and out_dtype is torch.bfloat16:
+            return gemm_bf16_tiled(x, weight, out_dtype, True)  # measured ahead of the library product + SwiGLU kernel
         return swiglu(linear(x, weight, out_dtype))
     if out_dtype is torch.float32:
         try:
@@ -655,3 +689,4 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
         _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
         _stream()))
     return out
+

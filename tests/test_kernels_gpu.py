@@ -84,6 +84,30 @@ def test_gemm_f32(m, n, k):
     torch.testing.assert_close(out.cpu(), (x.double() @ w.double().T).float(), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("m,n,k,gated", [(130, 200, 128, False), (257, 96, 192, True), (2048, 1024, 1024, False),
+                                         (77, 50, 64, True), (300, 333, 256, False), (513, 1000, 320, True)])
+@pytest.mark.parametrize("shape", [0, 1, 2, 6, 8])
+def test_gemm_bf16_tiled(m, n, k, gated, shape):
+    """The LDS-tiled matrix-core product at sizes that are no multiple of its tiles, against a float32
+    product of the same bfloat16 inputs; every block tile shape, plain and with the SwiGLU epilogue."""
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n * (2 if gated else 1), k, generator=g) * 0.1).bfloat16()
+    want = x.float() @ w.float().T
+    if gated:
+        want = plain.silu(want[:, :n]) * want[:, n:]
+    out_types = (torch.bfloat16,) if gated else (torch.bfloat16, torch.float32)
+    for out_dtype in out_types:
+        got = K().gemm_bf16_tiled(dev(x), dev(w), out_dtype, gated, shape=shape).float().cpu()
+        scale = max(1.0, want.abs().max().item())
+        tol_abs = (2**-7 if out_dtype is torch.bfloat16 else 1e-4) * scale
+        assert (got - want).abs().max().item() <= tol_abs, (out_dtype, (got - want).abs().max().item(), scale)
+    from mini_engine_amd.ops.library import KernelError
+
+    with pytest.raises(KernelError, match="multiple of 64"):
+        K().gemm_bf16_tiled(dev(x[:, : k - 8].contiguous()), dev(w[:, : k - 8].contiguous()), torch.bfloat16, gated)
+
+
 def test_gemm_f32_rows_do_not_depend_on_the_batch():
     """The value of a row is bit-identical whatever other rows are in the product."""
     x, w = torch.randn(90, 200), torch.randn(77, 200)
