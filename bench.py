@@ -5,7 +5,8 @@
 Prints ONE JSON line. ``value`` is decoded tokens a second at batch 8 with every sequence at the
 benchmark context length; a step is one decode step of the whole engine (schedule, step function
 from the cache, greedy sampling, postprocess). The same line carries the 2,048-token prefill, the
-HBM roofline of the decode step, and decode at batch 1 and 64.
+HBM roofline of the decode step, and under ``points`` decode at batch 1 and 64 and the reference's own
+throughput workload (64 requests of 256 prompt and 128 output tokens through ``generate``).
 """
 
 from __future__ import annotations
@@ -151,8 +152,23 @@ def main() -> int:
         step_bytes = weight_bytes + (tokens_before + tokens_after) / 2 * kv_per_token
         return (tokens_after - tokens_before) / dt, ms, step_bytes / (dt / k) / 1e9
 
+    def reference_workload():
+        """The reference's own throughput workload (benchmarks/bench.py:52-62, :113-123): 64 requests of
+        256 random prompt ids and 128 greedy output tokens, all submitted at once; output tokens over
+        the wall time of the whole run, prefill and scheduling included."""
+        params = SamplingParams(max_tokens=128, temperature=0.0, ignore_eos=True)
+        prompts = [prompt(256) for _ in range(64)]
+        engine.generate([prompt(256) for _ in range(2)], params)  # graphs of the smaller buckets, code objects
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = engine.generate(prompts, params)
+        torch.cuda.synchronize()
+        return sum(len(o) for o in outs) / (time.perf_counter() - t0)
+
     tok_s, ms_per_step, gbs = decode(args.batch)
     pts = {f"decode_b{b}": round(decode(b)[0], 1) for b in points}
+    if max_batch >= 64 and not args.zero_context:
+        pts["throughput_64x256in_128out"] = round(reference_workload(), 1)
     line = {
         "metric": "decode tok/s at batch 8 (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
