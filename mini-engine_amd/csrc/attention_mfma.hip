@@ -164,7 +164,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
     float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int bs_shift, int window,
-    float scale_log2, int split_keys, int num_splits, int head_chunks, DecodeFusedArgs fa) {
+    float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa) {
   const int bs = 1 << bs_shift;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
@@ -182,16 +182,15 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
                  v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
   };
   KvTile<D> t[DEPTH];
-  // Without a window the first key of a split does not depend on the item's length: its tile is
-  // requested at once, beside the load of the length instead of behind it (one memory round trip less
-  // at the head of every block). A split that turns out to lie past the item's end has read a valid page
-  // (an entry of the table, or page 0) that it does not use.
-  const bool speculative = window <= 0;
-  if (speculative) fetch(t[0], split * split_keys);
+  // The keys of an item, from its window's first (rounded down to a tile of 16) to its newest, are dealt
+  // to the splits in equal runs of whole tiles: every split has work whatever the item's length is
+  // (the grid is sized for the longest context the step may hold, often many times the actual one).
   const int ctx = item_ctx[item];
   const int lo = window > 0 ? max(ctx - window, 0) : 0;
-  const int begin = max(split * split_keys, (lo / 16) * 16);
-  const int end = min((split + 1) * split_keys, ctx);
+  const int lo16 = (lo / 16) * 16;
+  const int tiles_per_split = ((ctx - lo16 + 15) / 16 + num_splits - 1) / num_splits;
+  const int begin = lo16 + split * tiles_per_split * 16;
+  const int end = min(begin + tiles_per_split * 16, ctx);
 
   float m[1] = {-INFINITY}, lsum[1] = {0.f};
   float4_t acc[1][D / 16];
@@ -199,10 +198,10 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   for (int dt = 0; dt < D / 16; ++dt) acc[0][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
   if (begin < end) {
-    // otherwise the first tile is requested before the query is prepared, unless it holds the slot that
-    // this block is about to write: then it is requested (again) after that write
+    // the first tile is requested before the query is prepared, unless it holds the slot that this
+    // block is about to write
     const bool early = !FUSED || begin + 16 < ctx;
-    if (early && !speculative) fetch(t[0], begin);
+    if (early) fetch(t[0], begin);
     Frag8 qf[1][D / 32];
     if (FUSED) {
       constexpr int HC = D / 64;  // chunks per half head
@@ -407,8 +406,8 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
   const int depth = split_keys <= 256 ? 2 : 1;
 #define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                                                                         \
   attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
-                                                                    nkv, bs_shift, window, scale_log2, split_keys,    \
-                                                                    num_splits, chunks, ARGS)
+                                                                    nkv, bs_shift, window, scale_log2, num_splits,    \
+                                                                    chunks, ARGS)
   if constexpr (D % 64 == 0) {
     if (fused) {
       if (depth == 2)
@@ -433,8 +432,9 @@ extern "C" int me_attention_mfma_supported(int d, int bs) {
 
 // q [items, nh, d] (one token per item), item_ctx[i] = keys of item i including the new one,
 // workspace: part_o float [items * nh * num_splits * d], part_ml float [items * nh * num_splits * 2].
-// Split s covers keys [s * split_keys, (s+1) * split_keys); num_splits * split_keys must cover every
-// context the step can hold (max_ctx).
+// Every item's keys are dealt to the num_splits splits in equal runs; split_keys (a multiple of 16) says
+// how long a run is at the longest context the step can hold (max_ctx): num_splits * split_keys must
+// cover it, and it decides how many tiles a wave keeps in flight.
 static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
