@@ -178,12 +178,16 @@ static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x
     launch_variant<1, 8, 8, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
   else if (mt == 1)
     launch_variant<1, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else if (mt == 2 && chunks > 8 * 2)
+    launch_variant<2, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
   else if (mt == 2)
     launch_variant<2, 8, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
   else if (mt == 3)
-    launch_variant<3, 4, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<3, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+  else if (swiglu)  // two accumulators per tile: eight waves' partial sums would not fit into 64 KB of LDS
+    launch_variant<4, 4, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
   else
-    launch_variant<4, 4, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<4, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
 }
 
 // C[M, N] = epilogue(prologue(input) . W^T).
