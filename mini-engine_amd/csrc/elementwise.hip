@@ -35,28 +35,40 @@ extern "C" int me_embed(void* x, const void* table, const int* ids, int num_toke
 //   s = x[src] + (delta ? delta[src] : 0);  if (write_x) x[src] = s;
 //   h[r] = s * rsqrt(mean(s^2) + eps) * w
 // One block per row; the sum of squares is reduced in a fixed order.
+// `parts` (float32 [num_parts, total rows, dim], or null) is a delta that still is a sum: partial
+// products over runs of k, added here in the order of the runs.
 template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ w,
-                                   T* __restrict__ h, const int* __restrict__ rows, int dim, float eps,
-                                   int write_x) {
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,
+                                   int num_parts, size_t part_stride, const float* __restrict__ w, T* __restrict__ h,
+                                   const int* __restrict__ rows, int dim, float eps, int write_x) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xr = x + (size_t)src * dim;
   const T* dr = delta ? delta + (size_t)src * dim : nullptr;
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+  const float* pr = parts ? parts + (size_t)src * dim : nullptr;
+  const bool adds = dr || pr;
+  auto sum_at = [&](int i) {
     float s = xr[i];
     if (dr) s += to_float(dr[i]);
-    if (write_x && dr) xr[i] = s;
+    if (pr) {
+      float d = pr[i];
+      for (int p = 1; p < num_parts; ++p) d += pr[p * part_stride + i];
+      s += d;
+    }
+    return s;
+  };
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    const float s = sum_at(i);
+    if (write_x && adds) xr[i] = s;
     ss += s * s;
   }
   const float total = block_sum(ss, scratch);
   const float inv = rsqrtf(total / (float)dim + eps);
   T* hr = h + (size_t)r * dim;
   for (int i = threadIdx.x; i < dim; i += blockDim.x) {
-    float s = xr[i];
-    if (dr && !write_x) s += to_float(dr[i]);
+    const float s = (adds && !write_x) ? sum_at(i) : xr[i];
     hr[i] = from_float<T>(s * inv * w[i]);
   }
 }
@@ -137,21 +149,25 @@ static bool launch_add_rmsnorm_rows(float* x, const T* delta, const float* w, T*
   return true;
 }
 
-extern "C" int me_add_rmsnorm(void* x, const void* delta, const float* w, void* h, const int* rows,
-                              int num_rows, int dim, float eps, int write_x, int dtype, hipStream_t stream) {
+extern "C" int me_add_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
+                              const float* w, void* h, const int* rows, int num_rows, int dim, float eps, int write_x,
+                              int dtype, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   if (dim <= 0) return me_fail("me_add_rmsnorm: dim=%d", dim);
+  if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_add_rmsnorm: %d partial sums", num_parts);
   // bfloat16 only: in float32 the order of a row's sum stays the same for every number of rows
-  if (dtype == ME_BF16 && launch_add_rmsnorm_rows<bf16_t>((float*)x, (const bf16_t*)delta, w, (bf16_t*)h, rows, num_rows,
-                                                          dim, eps, write_x, stream))
+  if (dtype == ME_BF16 && !parts &&
+      launch_add_rmsnorm_rows<bf16_t>((float*)x, (const bf16_t*)delta, w, (bf16_t*)h, rows, num_rows, dim, eps, write_x,
+                                      stream))
     return me_check_launch("me_add_rmsnorm");
   const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
   if (dtype == ME_F32)
-    add_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((float*)x, (const float*)delta, w, (float*)h, rows,
-                                                                dim, eps, write_x);
+    add_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((float*)x, (const float*)delta, parts, num_parts,
+                                                                (size_t)part_stride, w, (float*)h, rows, dim, eps, write_x);
   else
-    add_rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>((float*)x, (const bf16_t*)delta, w, (bf16_t*)h,
-                                                                 rows, dim, eps, write_x);
+    add_rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>((float*)x, (const bf16_t*)delta, parts, num_parts,
+                                                                 (size_t)part_stride, w, (bf16_t*)h, rows, dim, eps,
+                                                                 write_x);
   return me_check_launch("me_add_rmsnorm");
 }
 

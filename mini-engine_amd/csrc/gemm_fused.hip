@@ -24,7 +24,7 @@ template <int MT, int WAVES, int U, bool NORM, bool SWIGLU, typename OutT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
     const bf16_t* __restrict__ X, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
     const float* __restrict__ w_norm, float eps, float* __restrict__ x_out, const bf16_t* __restrict__ W,
-    OutT* __restrict__ C, int M, int N, int K) {
+    OutT* __restrict__ C, int M, int N, int K, int chunks_per_split) {
   constexpr int ACCS = SWIGLU ? 2 : 1;
   __shared__ float red[WAVES][MT * ACCS][64][4];
   __shared__ float ssq[WAVES][MT][64];
@@ -45,13 +45,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
   }
   const bool writes_x = NORM && delta != nullptr && blockIdx.x == 0;
 
-  const int chunks = (K + 31) / 32;
-  for (int c0 = wave; c0 < chunks; c0 += WAVES * U) {
+  // blockIdx.y > 0 only with k cut into splits: this block sums chunks [first, last) of 32 k and writes
+  // its partial result behind those of the splits before it
+  const int first = blockIdx.y * chunks_per_split;
+  const int last = min((K + 31) / 32, first + chunks_per_split);
+  C += (size_t)blockIdx.y * M * N;
+  for (int c0 = first + wave; c0 < last; c0 += WAVES * U) {
     bf16x8_t a[U][ACCS], b[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = (c0 + WAVES * u) * 32 + g * 8;
-      const bool k_ok = k < K;  // K % 8 == 0 is checked on the host
+      const bool k_ok = k < K && c0 + WAVES * u < last;  // K % 8 == 0 is checked on the host
       a[u][0] = bf16x8_t{};
       if (n_ok && k_ok) a[u][0] = *reinterpret_cast<const bf16x8_t*>(wrow + k);
       if (SWIGLU) {
@@ -62,7 +66,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = (c0 + WAVES * u) * 32 + g * 8;
-      const bool k_ok = k < K;
+      const bool k_ok = k < K && c0 + WAVES * u < last;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + r;
@@ -148,11 +152,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
 template <int MT, int WAVES, int U, typename OutT>
 static void launch_variant(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
                            const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
-                           hipStream_t stream) {
-  const unsigned blocks = (N + 15) / 16;
+                           int splits, hipStream_t stream) {
+  const dim3 blocks((N + 15) / 16, splits);
+  const int cps = ((K + 31) / 32 + splits - 1) / splits;
 #define ME_LAUNCH(NORM, SWI)                                                                                  \
   gemm_small_kernel<MT, WAVES, U, NORM, SWI, OutT><<<blocks, WAVES * 64, 0, stream>>>(X, x_in, delta, w_norm, eps, \
-                                                                                      x_out, W, C, M, N, K)
+                                                                                      x_out, W, C, M, N, K, cps)
   if (norm && swiglu)
     ME_LAUNCH(true, true);
   else if (norm)
@@ -167,27 +172,27 @@ static void launch_variant(bool norm, bool swiglu, const bf16_t* X, const float*
 template <typename OutT>
 static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
                          const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
-                         hipStream_t stream) {
+                         int splits, hipStream_t stream) {
   const int mt = (M + 15) / 16;
   // up to 16 rows: as many chunks of 32 k per wave and round as it takes to have all of k in flight at
   // once (a second round of loads costs a memory round trip, which is most of such a kernel's time)
-  const int chunks = (K + 31) / 32;
+  const int chunks = ((K + 31) / 32 + splits - 1) / splits;  // per block
   if (mt == 1 && chunks > 8 * 8)
-    launch_variant<1, 8, 12, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<1, 8, 12, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (mt == 1 && chunks > 8 * 4)
-    launch_variant<1, 8, 8, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<1, 8, 8, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (mt == 1)
-    launch_variant<1, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<1, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (mt == 2 && chunks > 8 * 2)
-    launch_variant<2, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<2, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (mt == 2)
-    launch_variant<2, 8, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<2, 8, 2, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (mt == 3)
-    launch_variant<3, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<3, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (swiglu)  // two accumulators per tile: eight waves' partial sums would not fit into 64 KB of LDS
-    launch_variant<4, 4, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<4, 4, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else
-    launch_variant<4, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, stream);
+    launch_variant<4, 8, 4, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
 }
 
 // C[M, N] = epilogue(prologue(input) . W^T).
@@ -196,10 +201,16 @@ static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x
 //   is given, x_in + delta is written to x_out (float32 [M, K], not aliasing x_in).
 //   swiglu == 0: W is [N, K].  swiglu == 1: W is [2 N, K] (gate rows, then up rows), C = silu(gate) * up.
 //   out_dtype: ME_BF16 or ME_F32. M <= 64, K % 8 == 0, pointers 16-byte aligned.
+//   k_splits > 1 (plain float32 products only): k is cut into that many runs of whole chunks of 32, each
+//   summed by blocks of its own, and C is [k_splits, M, N]: partial sums for the caller to add up (more
+//   blocks for products with few output columns, and each reads only its run of x).
 extern "C" int me_gemm_bf16_small(const void* X, const float* x_in, const void* delta, const float* w_norm, float eps,
                                   float* x_out, const void* W, void* C, int M, int N, int K, int norm, int swiglu,
-                                  int out_dtype, hipStream_t stream) {
+                                  int out_dtype, int k_splits, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
+  if (k_splits < 1 || k_splits > 64) return me_fail("me_gemm_bf16_small: %d splits of k", k_splits);
+  if (k_splits > 1 && (norm || swiglu || out_dtype != ME_F32))
+    return me_fail("me_gemm_bf16_small: partial sums over splits of k are plain float32 products");
   if (M > 64) return me_fail("me_gemm_bf16_small: M=%d exceeds 64 rows", M);
   if (K <= 0 || K % 8) return me_fail("me_gemm_bf16_small: K=%d must be a positive multiple of 8", K);
   if (norm) {
@@ -213,8 +224,8 @@ extern "C" int me_gemm_bf16_small(const void* X, const float* x_in, const void* 
   if (((uintptr_t)X | (uintptr_t)W) & 15) return me_fail("me_gemm_bf16_small: operands must be 16-byte aligned");
   const bf16_t *x = (const bf16_t*)X, *d = (const bf16_t*)delta, *w = (const bf16_t*)W;
   if (out_dtype == ME_F32)
-    launch_small<float>(norm, swiglu, x, x_in, d, w_norm, eps, x_out, w, (float*)C, M, N, K, stream);
+    launch_small<float>(norm, swiglu, x, x_in, d, w_norm, eps, x_out, w, (float*)C, M, N, K, k_splits, stream);
   else
-    launch_small<bf16_t>(norm, swiglu, x, x_in, d, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, stream);
+    launch_small<bf16_t>(norm, swiglu, x, x_in, d, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, 1, stream);
   return me_check_launch("me_gemm_bf16_small");
 }

@@ -65,9 +65,25 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = Non
     return out
 
 
+class PartialSums:
+    """A product that still is a sum: float32 ``parts`` [S, T, D], partial products over S runs of k.
+    It stands where a delta of the residual stream stands; :func:`add_rmsnorm` adds the parts up, in the
+    order of the runs, as it adds the delta."""
+
+    def __init__(self, parts: torch.Tensor):
+        self.parts = parts
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+    def to_tensor(self, dtype: torch.dtype) -> torch.Tensor:
+        return self.parts.sum(0).to(dtype)
+
+
 def add_rmsnorm(
     x: torch.Tensor,
-    delta: torch.Tensor | None,
+    delta: "torch.Tensor | PartialSums | None",
     weight: torch.Tensor,
     eps: float,
     dtype: torch.dtype,
@@ -76,12 +92,16 @@ def add_rmsnorm(
     write_x: bool = True,
 ) -> torch.Tensor:
     """Residual add then RMSNorm. ``x`` float32 [T, D] is the residual stream (updated in place when
-    ``write_x``), ``delta`` [T, D] in ``dtype`` or None, ``weight`` float32 [D]. With ``rows`` (int32
+    ``write_x``), ``delta`` [T, D] in ``dtype``, :class:`PartialSums` or None, ``weight`` float32 [D]. With ``rows`` (int32
     [R]) only those rows are read and the result is [R, D]. Returns the normed rows in ``dtype``."""
     _want(x, "x", torch.float32, (None, None))
     t, d = x.shape
     _want(weight, "weight", torch.float32, (d,))
-    if delta is not None:
+    parts = None
+    if isinstance(delta, PartialSums):
+        parts, delta = delta.parts, None
+        _want(parts, "partial sums", torch.float32, (None, t, d))
+    elif delta is not None:
         _want(delta, "delta", dtype, (t, d))
     n = t
     if rows is not None:
@@ -90,8 +110,9 @@ def add_rmsnorm(
     if out is None:
         out = torch.empty((n, d), dtype=dtype, device=x.device)
     _want(out, "out", dtype, (n, d))
-    check(lib().me_add_rmsnorm(_p(x), _p(delta), _p(weight), _p(out), _p(rows), _i(n), _i(d), _f(eps),
-                               _i(1 if write_x else 0), _i(_code(dtype)), _stream()))
+    check(lib().me_add_rmsnorm(_p(x), _p(delta), _p(parts), _i(0 if parts is None else parts.shape[0]),
+                               ctypes.c_longlong(0 if parts is None else t * d), _p(weight), _p(out), _p(rows), _i(n),
+                               _i(d), _f(eps), _i(1 if write_x else 0), _i(_code(dtype)), _stream()))
     return out
 
 
@@ -286,12 +307,13 @@ SMALL_FAST_ROWS = 16  # up to here it beats the GEMM library on every shape, wit
 
 
 def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
-                    out: torch.Tensor | None = None) -> torch.Tensor:
+                    out: torch.Tensor | None = None, k_splits: int = 1) -> torch.Tensor:
     """bfloat16 ``x @ weight.T`` for at most 64 rows on the matrix cores, float32 accumulation.
 
     ``x`` is a bfloat16 tensor [M, K] or a :class:`NormedInput` (then the residual add and the RMSNorm
     are the product's prologue). With ``swiglu`` the weight holds gate rows then up rows, [2N, K], and
-    the result is ``silu(gate) * up`` [M, N]."""
+    the result is ``silu(gate) * up`` [M, N]. With ``k_splits`` > 1 (plain float32 products) the result
+    is [k_splits, M, N]: partial sums over runs of k, each by blocks of its own."""
     normed = isinstance(x, NormedInput)
     m, k = x.shape
     _want(weight, "weight", torch.bfloat16, (None, k))
@@ -302,9 +324,16 @@ def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bflo
         n //= 2
     if m > SMALL_MAX_ROWS:
         raise ValueError(f"gemm_bf16_small takes at most {SMALL_MAX_ROWS} rows, got {m}")
-    if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=weight.device)
-    _want(out, "out", out_dtype, (m, n))
+    if k_splits > 1:
+        if normed or swiglu or out_dtype is not torch.float32:
+            raise ValueError("partial sums over splits of k are plain float32 products")
+        if out is None:
+            out = torch.empty((k_splits, m, n), dtype=torch.float32, device=weight.device)
+        _want(out, "out", torch.float32, (k_splits, m, n))
+    else:
+        if out is None:
+            out = torch.empty((m, n), dtype=out_dtype, device=weight.device)
+        _want(out, "out", out_dtype, (m, n))
     if normed:
         _want(x.x, "residual stream", torch.float32, (m, k))
         _want(x.weight, "norm weight", torch.float32, (k,))
@@ -317,13 +346,13 @@ def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bflo
             x_out = x.spare
         check(lib().me_gemm_bf16_small(_p(None), _p(x.x), _p(x.delta), _p(x.weight), _f(x.eps), _p(x_out), _p(weight),
                                        _p(out), _i(m), _i(n), _i(k), _i(1), _i(1 if swiglu else 0),
-                                       _i(_code(out_dtype)), _stream()))
+                                       _i(_code(out_dtype)), _i(1), _stream()))
         x.residual = x.x if x.delta is None else x.spare
     else:
         _want(x, "x", torch.bfloat16, (m, k))
         check(lib().me_gemm_bf16_small(_p(x), _p(None), _p(None), _p(None), _f(0.0), _p(None), _p(weight), _p(out),
                                        _i(m), _i(n), _i(k), _i(0), _i(1 if swiglu else 0), _i(_code(out_dtype)),
-                                       _stream()))
+                                       _i(k_splits), _stream()))
     return out
 
 
@@ -377,9 +406,22 @@ def small_ok(x, weight: torch.Tensor, gated: bool = False) -> bool:
     return x.shape[0] <= SMALL_MAX_ROWS and (gated or 2048 <= weight.shape[0] <= 16384)
 
 
-def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False) -> torch.Tensor:
+def delta_splits(rows: int, n: int, k: int) -> int:
+    """Into how many runs of k a product of 17 to 64 rows with few output columns is cut (1: not at all):
+    a block per 16 columns leaves most of the chip idle and makes each block read all of x, so k is
+    cut until about every compute unit has a block, each with at least 256 of k."""
+    if not SMALL_FAST_ROWS < rows <= SMALL_MAX_ROWS or n >= 2048 or k % 8:
+        return 1
+    return max(1, min(8, 256 // -(-n // 16), k // 256))
+
+
+def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False,
+           as_delta: bool = False):
     """``x @ weight.T`` for x [M, K], weight [N, K]; with ``gated`` the weight is [2N, K] (gate rows,
-    then up rows) and the result is ``silu(gate) * up``. ``x`` may be a :class:`NormedInput`.
+    then up rows) and the result is ``silu(gate) * up``. ``x`` may be a :class:`NormedInput`. With
+    ``as_delta`` the caller says that the result only ever is the pending delta of the residual stream
+    (what a mixer or a feed-forward returns): it may then come back as :class:`PartialSums`, which
+    :func:`add_rmsnorm` adds up on the way.
 
     float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16: the
     fused matrix-core kernel for up to 16 rows; the tiled matrix-core kernel with the SwiGLU as its
@@ -398,6 +440,10 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return swiglu(y) if gated else y
     if small_ok(x, weight, gated):
         return gemm_bf16_small(x, weight, out_dtype, gated)
+    if as_delta and not gated and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0:
+        splits = delta_splits(x.shape[0], weight.shape[0], x.shape[1])
+        if splits > 1:
+            return PartialSums(gemm_bf16_small(x, weight, torch.float32, k_splits=splits))
     if gated:
         if tiled_ok(x, weight) and out_dtype is torch.bfloat16:
             return gemm_bf16_tiled(x, weight, out_dtype, True)  # measured ahead of the library product + SwiGLU kernel

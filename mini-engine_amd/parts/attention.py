@@ -93,13 +93,13 @@ class Attention(Mixer):
             out = K.attention_decode_fused_bf16(
                 proj, self.q_norm_w, self.k_norm_w if owns else None, rope, eps, owns, b.k_cache, b.v_cache,
                 batch.item_ctx, table, self.nh, float(s.scale), int(s.window), batch.max_ctx)
-            return K.linear(out, self.w_o)
+            return K.linear(out, self.w_o, as_delta=True)
         q = K.qk_norm_rope_scatter(
             proj, self.q_norm_w, self.k_norm_w if owns else None, rope, batch.positions, batch.token_item,
             table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, eps, write_kv=owns,
             item_start=batch.item_start, starts=batch.starts, qlens=batch.qlens)
         out = self.attend(q, batch, table, b)
-        return K.linear(out, self.w_o)
+        return K.linear(out, self.w_o, as_delta=True)
 
     def attend(self, q: torch.Tensor, batch, table: torch.Tensor, b: KVBinding) -> torch.Tensor:
         """bfloat16 with sizes the matrix-core kernels take: the split-context kernel when every item

@@ -97,11 +97,16 @@ class Mixer(Part):
         return None
 
     def forward(self, h: torch.Tensor, batch: Any, cache: Any = None) -> torch.Tensor:
+        """``h`` is the normed input [T, H] (or a lazy one that a part may take as the prologue of its
+        first product); the result [T, H] is the delta that the block adds to the residual stream. It
+        may be any object that the add-and-norm kernel takes as a delta: a tensor in the compute dtype,
+        or partial sums that kernel adds up (see ``ops.kernels.linear(..., as_delta=True)``)."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, batch: Any) -> torch.Tensor:
+        """As :meth:`Mixer.forward`, without a cache."""
         raise NotImplementedError
 
 

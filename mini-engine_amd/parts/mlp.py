@@ -34,7 +34,7 @@ class GatedMlp(FeedForward):
 
     def forward(self, h, batch=None) -> torch.Tensor:
         act = K.linear(h, self.w_gate_up, gated=True)
-        return K.linear(act, self.w_down)
+        return K.linear(act, self.w_down, as_delta=True)
 
 
 FEED_FORWARDS.register("gated_mlp", GatedMlp)

@@ -108,6 +108,44 @@ def test_gemm_bf16_tiled(m, n, k, gated, shape):
         K().gemm_bf16_tiled(dev(x[:, : k - 8].contiguous()), dev(w[:, : k - 8].contiguous()), torch.bfloat16, gated)
 
 
+@pytest.mark.parametrize("m,n,k,splits", [(17, 1024, 2048, 4), (64, 1000, 3072, 4), (33, 48, 520, 2), (40, 16, 4096, 8)])
+def test_small_gemm_partial_sums_and_their_add_rmsnorm(m, n, k, splits):
+    """A product of 17 to 64 rows cut into runs of k: the parts add up to the product, and add_rmsnorm
+    takes them where it takes a delta."""
+    g = torch.Generator().manual_seed(k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    parts = K().gemm_bf16_small(dev(x), dev(w), torch.float32, k_splits=splits)
+    assert parts.shape == (splits, m, n)
+    want = x.float() @ w.float().T
+    torch.testing.assert_close(parts.sum(0).cpu(), want, rtol=1e-4, atol=1e-4 * max(1.0, want.abs().max().item()))
+    if k >= 64 * splits:
+        assert all(parts[i].abs().max() > 0 for i in range(splits))  # every run did some of the work
+    res = torch.randn(m, n, generator=g) * 2
+    wn = 1 + 0.1 * torch.randn(n, generator=g)
+    xd = dev(res.clone())
+    h = K().add_rmsnorm(xd, K().PartialSums(parts), dev(wn), 1e-5, torch.bfloat16)
+    s = res + want
+    torch.testing.assert_close(xd.cpu(), s, rtol=1e-4, atol=1e-4 * max(1.0, s.abs().max().item()))
+    torch.testing.assert_close(h.float().cpu(), plain.rms_norm(s, wn, 1e-5), **tol(torch.bfloat16))
+    pick = torch.tensor([m - 1, 0], dtype=torch.int32)
+    xd2 = dev(res.clone())
+    h2 = K().add_rmsnorm(xd2, K().PartialSums(parts), dev(wn), 1e-5, torch.bfloat16, rows=dev(pick), write_x=False)
+    assert torch.equal(xd2.cpu(), res)
+    torch.testing.assert_close(h2.float().cpu(), plain.rms_norm(s[pick.long()], wn, 1e-5), **tol(torch.bfloat16))
+
+
+def test_linear_hands_back_partial_sums_only_when_asked():
+    x = dev(torch.randn(40, 2048).bfloat16())
+    w = dev((torch.randn(1024, 2048) * 0.02).bfloat16())
+    plain_out = K().linear(x, w)
+    assert isinstance(plain_out, torch.Tensor)
+    delta = K().linear(x, w, as_delta=True)
+    assert isinstance(delta, K().PartialSums) and delta.shape == (40, 1024)
+    torch.testing.assert_close(delta.to_tensor(torch.bfloat16).float(), plain_out.float(), rtol=2e-2, atol=2e-2)
+    assert isinstance(K().linear(x[:8], w, as_delta=True), torch.Tensor)  # up to 16 rows: the fused kernel
+
+
 def test_gemm_f32_rows_do_not_depend_on_the_batch():
     """The value of a row is bit-identical whatever other rows are in the product."""
     x, w = torch.randn(90, 200), torch.randn(77, 200)
