@@ -73,19 +73,21 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
   }
 }
 
-// The same for many bfloat16 rows (256 or more): a wave per row, the row in registers (CHUNKS x 8 elements per lane), 16-byte
+// The same for more than 16 bfloat16 rows: a wave per row, the row in registers (CHUNKS x 8 elements per lane), 16-byte
 // loads and stores, no LDS and no barrier. dim is a multiple of 8 and at most 512 * CHUNKS.
 template <typename T, int CHUNKS>
 __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float* __restrict__ x, const T* __restrict__ delta,
-                                                                const float* __restrict__ w, T* __restrict__ h,
-                                                                const int* __restrict__ rows, int num_rows, int dim,
-                                                                float eps, int write_x) {
+                                                                const float* __restrict__ parts, int num_parts,
+                                                                size_t part_stride, const float* __restrict__ w,
+                                                                T* __restrict__ h, const int* __restrict__ rows,
+                                                                int num_rows, int dim, float eps, int write_x) {
   const int lane = threadIdx.x & (ME_WAVE - 1);
-  const int r = blockIdx.x * 4 + threadIdx.x / ME_WAVE;
+  const int r = blockIdx.x * (blockDim.x / ME_WAVE) + threadIdx.x / ME_WAVE;
   if (r >= num_rows) return;
   const int src = rows ? rows[r] : r;
   float* xr = x + (size_t)src * dim;
   const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+  const float* pr = parts ? parts + (size_t)src * dim : nullptr;
   float s[CHUNKS][8];
   float ss = 0.f;
 #pragma unroll
@@ -103,10 +105,20 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float* __restrict
         const Pack d = *reinterpret_cast<const Pack*>(dr + e);
 #pragma unroll
         for (int j = 0; j < 8; ++j) s[c][j] += to_float(d.v[j]);
-        if (write_x) {
-          *reinterpret_cast<float4*>(xr + e) = make_float4(s[c][0], s[c][1], s[c][2], s[c][3]);
-          *reinterpret_cast<float4*>(xr + e + 4) = make_float4(s[c][4], s[c][5], s[c][6], s[c][7]);
+      }
+      if (pr) {  // a delta that still is a sum of partial products: added in the order of the runs
+        float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < num_parts; ++p) {
+          const float4 pa = *reinterpret_cast<const float4*>(pr + p * part_stride + e);
+          const float4 pb = *reinterpret_cast<const float4*>(pr + p * part_stride + e + 4);
+          d[0] += pa.x, d[1] += pa.y, d[2] += pa.z, d[3] += pa.w, d[4] += pb.x, d[5] += pb.y, d[6] += pb.z, d[7] += pb.w;
         }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[c][j] += d[j];
+      }
+      if ((dr || pr) && write_x) {
+        *reinterpret_cast<float4*>(xr + e) = make_float4(s[c][0], s[c][1], s[c][2], s[c][3]);
+        *reinterpret_cast<float4*>(xr + e + 4) = make_float4(s[c][4], s[c][5], s[c][6], s[c][7]);
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) ss = fmaf(s[c][j], s[c][j], ss);
@@ -131,12 +143,16 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float* __restrict
 }
 
 template <typename T>
-static bool launch_add_rmsnorm_rows(float* x, const T* delta, const float* w, T* h, const int* rows, int num_rows, int dim,
-                                    float eps, int write_x, hipStream_t stream) {
-  if (num_rows < 256 || dim % 8 || dim > 4096) return false;
-  if (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)h) & 15) return false;
-  const unsigned blocks = (num_rows + 3) / 4;
-#define ME_ROWS_CASE(C) add_rmsnorm_rows_kernel<T, C><<<blocks, 256, 0, stream>>>(x, delta, w, h, rows, num_rows, dim, eps, write_x)
+static bool launch_add_rmsnorm_rows(float* x, const T* delta, const float* parts, int num_parts, size_t part_stride,
+                                    const float* w, T* h, const int* rows, int num_rows, int dim, float eps, int write_x,
+                                    hipStream_t stream) {
+  if (num_rows <= 16 || dim % 8 || dim > 4096) return false;
+  if (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)parts | (uintptr_t)w | (uintptr_t)h) & 15 || part_stride % 4) return false;
+  const int waves = num_rows >= 256 ? 4 : 1;  // few rows: a block each, on compute units of their own
+  const unsigned blocks = (num_rows + waves - 1) / waves;
+#define ME_ROWS_CASE(C)                                                                                             \
+  add_rmsnorm_rows_kernel<T, C><<<blocks, waves * 64, 0, stream>>>(x, delta, parts, num_parts, part_stride, w, h, rows, \
+                                                                   num_rows, dim, eps, write_x)
   if (dim <= 512)
     ME_ROWS_CASE(1);
   else if (dim <= 1024)
@@ -156,9 +172,9 @@ extern "C" int me_add_rmsnorm(void* x, const void* delta, const float* parts, in
   if (dim <= 0) return me_fail("me_add_rmsnorm: dim=%d", dim);
   if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_add_rmsnorm: %d partial sums", num_parts);
   // bfloat16 only: in float32 the order of a row's sum stays the same for every number of rows
-  if (dtype == ME_BF16 && !parts &&
-      launch_add_rmsnorm_rows<bf16_t>((float*)x, (const bf16_t*)delta, w, (bf16_t*)h, rows, num_rows, dim, eps, write_x,
-                                      stream))
+  if (dtype == ME_BF16 && launch_add_rmsnorm_rows<bf16_t>((float*)x, (const bf16_t*)delta, parts, num_parts,
+                                                          (size_t)part_stride, w, (bf16_t*)h, rows, num_rows, dim, eps,
+                                                          write_x, stream))
     return me_check_launch("me_add_rmsnorm");
   const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
   if (dtype == ME_F32)

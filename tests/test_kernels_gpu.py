@@ -42,7 +42,7 @@ def test_embed(dtype, hidden, vocab):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,dim", [(5, 72), (3, 1000), (2, 5120), (1, 16), (300, 1000), (257, 4096), (260, 72),
-                                      (256, 520)])
+                                      (256, 520), (17, 1024), (64, 1000), (40, 4100)])
 def test_add_rmsnorm(dtype, rows, dim):
     x, delta, w = torch.randn(rows, dim) * 3, torch.randn(rows, dim).to(dtype), 1 + 0.1 * torch.randn(dim)
     xd = dev(x.clone())
