@@ -159,6 +159,8 @@ struct DecodeFusedArgs {
   bf16_t* v_cache_w;
 };
 
+#define LONG_RUN 16  // tiles of a split from which on a wave fetches one tile at a time
+
 template <int D, bool FUSED, int DEPTH>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -303,16 +305,24 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     // splits (few waves, each waiting on memory) want two (four measured no better); with long splits the
     // chip is full of waves and fewer registers, one more wave per SIMD, serve better. A tile past `end` is a valid page that
     // nobody computes on.
+    if (DEPTH > 1 && tiles_per_split > LONG_RUN) {
+      // a long run of this wave's own (the chip is full of such waves): one tile at a time streams best
+      for (int k = begin; k < end; k += 16) {
+        if (k > begin) fetch(t[0], k);
+        compute_tile<D, 1>(t[0], k, lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc);
+      }
+    } else {
 #pragma unroll
-    for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], begin + 16 * j);
-    for (int key0 = begin; key0 < end; key0 += 16 * DEPTH) {
+      for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], begin + 16 * j);
+      for (int key0 = begin; key0 < end; key0 += 16 * DEPTH) {
 #pragma unroll
-      for (int j = 0; j < DEPTH; ++j) {
-        const int k = key0 + 16 * j;
-        if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], k + 16 * (DEPTH - 1));
-        else if (k > begin) fetch(t[0], k);
-        if (j == 0 || k < end)
-          compute_tile<D, 1>(t[j], k, lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc);
+        for (int j = 0; j < DEPTH; ++j) {
+          const int k = key0 + 16 * j;
+          if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], k + 16 * (DEPTH - 1));
+          else if (k > begin) fetch(t[0], k);
+          if (j == 0 || k < end)
+            compute_tile<D, 1>(t[j], k, lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc);
+        }
       }
     }
   }
@@ -403,7 +413,7 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
   dim3 grid(items, nkv * chunks, num_splits);
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-  const int depth = split_keys <= 256 ? 2 : 1;
+  const int depth = (split_keys <= 256 || (long long)items * nkv * chunks * num_splits <= 1024) ? 2 : 1;
 #define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                                                                         \
   attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
                                                                     nkv, bs_shift, window, scale_log2, num_splits,    \
