@@ -34,20 +34,35 @@ def _p(t: torch.Tensor | None) -> _vp:
     return _vp(None) if t is None else _vp(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> _vp:
+    """torch's current stream of the current device, as the handle the entry points take. An eager step
+    makes a few hundred of these calls: the raw getter, where this torch has it, costs a tenth of
+    building a Stream object."""
+    if _raw_stream is not None:
+        return _vp(_raw_stream(torch.cuda.current_device()))
     return _vp(torch.cuda.current_stream().cuda_stream)
 
 
 def _want(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: tuple | None = None) -> None:
-    if not t.is_cuda:
-        raise ValueError(f"{name} must be on the GPU")
-    if not t.is_contiguous():
-        raise ValueError(f"{name} must be contiguous")
+    """Host-side check of an operand: on the GPU, contiguous, of the wanted dtype and shape (None in the
+    shape: any size). What the kernels index with is checked here, before anything is launched."""
+    if not (t.is_cuda and t.is_contiguous()):
+        raise ValueError(f"{name} must be a contiguous tensor on the GPU")
     if dtype is not None and t.dtype is not dtype:
         raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
     if shape is not None:
-        if t.dim() != len(shape) or any(s is not None and s != g for s, g in zip(shape, t.shape)):
-            raise ValueError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+        got = t.shape
+        ok = len(got) == len(shape)
+        if ok:
+            for s, g in zip(shape, got):
+                if s is not None and s != g:
+                    ok = False
+                    break
+        if not ok:
+            raise ValueError(f"{name} must have shape {list(shape)}, got {list(got)}")
 
 
 # ------------------------------------------------------------------------------------ row-wise ops
