@@ -20,7 +20,7 @@ def pytest_configure(config):
 
 
 def tiny_configs():
-    """Two configurations that differ in every size and option."""
+    """Configurations that differ in every size and option."""
     from mini_engine_amd.models.qwen3 import Qwen3Config
 
     a = Qwen3Config(vocab_size=256, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
@@ -29,10 +29,15 @@ def tiny_configs():
     b = Qwen3Config(vocab_size=384, hidden_size=96, intermediate_size=160, num_hidden_layers=3,
                     num_attention_heads=6, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-5,
                     rope_theta=1e6, max_position_embeddings=1024, tie_word_embeddings=False)
-    return {"A": a, "B": b}
+    # a third one whose head size and page size take the bfloat16 path through the matrix-core attention
+    # kernels (A and B, with heads of 16 and pages of 8, run the general kernels)
+    c = Qwen3Config(vocab_size=320, hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                    num_attention_heads=4, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6,
+                    rope_theta=50000.0, max_position_embeddings=2048, tie_word_embeddings=True)
+    return {"A": a, "B": b, "C": c}
 
 
-BLOCK_SIZES = {"A": 16, "B": 8}
+BLOCK_SIZES = {"A": 16, "B": 8, "C": 16}
 
 
 def write_tiny(folder: str, cfg, seed: int = 0, std: float = 0.02, dtype=torch.bfloat16) -> str:

@@ -1,5 +1,5 @@
-"""Replay of the same requests under every way of cutting them, in float32 and bfloat16, on both
-tiny configurations, compared with the plain implementation position by position:
+"""Replay of the same requests under every way of cutting them, in float32 and bfloat16, on the
+tiny configurations (C reaches the matrix-core attention kernels in bfloat16), compared with the plain implementation position by position:
 whole; most in one step and the last 32 tokens one by one; portions of changing size down to two
 tokens; mixed with other requests in a pool so small that pages are used again."""
 
@@ -49,7 +49,7 @@ def plain_for(folders, name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_replay_matches_plain(tiny_folders, name, dtype, mode):
     reqs = requests_for(name)
