@@ -25,7 +25,8 @@ import numpy as np
 PAGE_ROUNDING = 64  # a request's token count is rounded up to this for the --max-tokens bound
 
 
-def build_session(model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8):
+def build_session(model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8,
+                  cuda_graphs: bool = True):
     from ..config.engine_config import EngineConfig
     from ..ops.library import lib
     from .llm_engine import LLMEngine
@@ -42,7 +43,7 @@ def build_session(model_dir: str, dtype: str, max_tokens: int, block_size: int =
         max_model_len=max(max_tokens, block_size),
         enable_prefix_caching=False,
         dtype=dtype,
-        cuda_graphs=True,
+        cuda_graphs=cuda_graphs,
     )
     return LLMEngine.from_pretrained(model_dir, config, progress=lambda m: print(f"[trace_run] {m}", file=sys.stderr, flush=True))
 

@@ -1,0 +1,59 @@
+"""The layer sizes of the benchmark's model (hidden 1024, 16 query and 8 kv heads of 128, feed-forward
+3072) with two layers and a small vocabulary, in bfloat16, against the plain implementation: the paths
+that only such sizes reach. A 700-token prompt in one step (the tiled matrix-core GEMM with the SwiGLU
+epilogue, prefill attention with tiles cut and packed into bundles), 24 short prompts in one step, then
+all 25 requests decoding side by side (17 to 64 rows: the small matrix-core GEMM, projections as partial
+sums over runs of k, the fused decode attention with its keys dealt to the splits), eagerly and as a
+replayed graph."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+import trace_helpers as th
+from conftest import random_prompt, write_tiny
+
+pytestmark = pytest.mark.gpu
+
+EXTRA = 6  # tokens each request is fed one by one after its prompt
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    from mini_engine_amd.models.qwen3 import Qwen3Config
+
+    cfg = Qwen3Config(vocab_size=512, hidden_size=1024, intermediate_size=3072, num_hidden_layers=2,
+                      num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+                      rope_theta=1e6, max_position_embeddings=4096, tie_word_embeddings=True)
+    folder = write_tiny(str(tmp_path_factory.mktemp("model_shape")), cfg, seed=5, std=0.03)
+    reqs = {"long": random_prompt(700 + EXTRA, cfg.vocab_size, seed=1)}
+    for i in range(24):
+        reqs[f"s{i}"] = random_prompt(20 + (7 * i) % 41 + EXTRA, cfg.vocab_size, seed=10 + i)
+    return folder, reqs, th.plain_logits(folder, reqs)
+
+
+def steps_for(reqs):
+    def entry(rid, lo, hi):
+        return {"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
+
+    steps = [{"step": 0, "entries": [entry("long", 0, len(reqs["long"]) - EXTRA)], "end": []},
+             {"step": 1, "entries": [entry(r, 0, len(t) - EXTRA) for r, t in reqs.items() if r != "long"], "end": []}]
+    for j in range(EXTRA):
+        steps.append({"step": 2 + j, "entries": [entry(r, len(t) - EXTRA + j, len(t) - EXTRA + j + 1) for r, t in reqs.items()],
+                      "end": list(reqs) if j == EXTRA - 1 else []})
+    return steps
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_benchmark_layer_sizes_against_plain(model, graphs):
+    from mini_engine_amd.engine.trace import TraceSession, build_session
+
+    folder, reqs, want = model
+    steps = steps_for(reqs)
+    session = TraceSession(build_session(folder, "bfloat16", 4096, block_size=16, max_live=32, cuda_graphs=graphs))
+    got = th.collect(steps, th.replay_in_process(session, steps))
+    for rid in reqs:
+        th.assert_logits_close(got[rid], want[rid], "bfloat16", f"graphs={graphs} request {rid}")
+    assert (session.engine.runner.graph_replays > 0) == graphs
+    assert all(len(p.free_pool) == p.num_blocks for p in session.bm.pools)
