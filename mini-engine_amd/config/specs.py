@@ -6,7 +6,7 @@ sizes. Nothing in here knows an architecture's name; an architecture module turn
 ``config.json`` keys into these specs (see ``models/qwen3.py``).
 
 Every spec is a frozen dataclass with a ``kind`` string. The part registries in
-``parts/registry.py`` map ``kind`` to the class that implements it, so a new kind of mixer,
+``parts/base.py`` map ``kind`` to the class that implements it, so a new kind of mixer,
 feed-forward, norm or position encoding is added by registering a (spec, implementation) pair; no
 spec in this file has to change for that.
 """

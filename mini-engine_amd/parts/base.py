@@ -6,7 +6,8 @@ it is in. The four interfaces:
 
 ``Norm``               ``weight_wants(name)``, ``load(tensors, name)``, ``weight`` / ``eps`` used by the
                        fused residual-add-and-norm of the block.
-``PositionEncoding``   ``tables(device)`` returns what the mixer's kernel needs (for rotary: inv_freq).
+``PositionEncoding``   ``tables(num_positions)`` returns what the mixer's kernels read (for rotating
+                       encodings: the float32 table of cosines and sines by position).
 ``Mixer``              ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``cache_need()``,
                        ``forward(h, batch, cache) -> [T, hidden]``.
 ``FeedForward``        ``weight_wants(prefix)``, ``load(tensors, prefix)``, ``forward(h, batch) -> [T, hidden]``.
@@ -84,7 +85,11 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    def tables(self) -> Any:
+    def tables(self, num_positions: int = 1) -> Any:
+        """What the mixer's kernels read for positions ``0 .. num_positions - 1``. For encodings that
+        rotate pairs ``(j, j + r/2)`` of the first ``r`` elements of each head: a contiguous float32
+        tensor ``[P >= num_positions, 2, r/2]`` of cosines and sines on the part's device. It is not
+        allocated anew inside a graph capture: keep and hand back a table that is large enough."""
         raise NotImplementedError
 
 

@@ -6,8 +6,10 @@ without a change to the framework's files. It keeps, per request, the running su
 
 The state must be carried from portion to portion, start from zero for a new request in a used slot,
 and not leak between requests that share a batch. A toy feed-forward with routing (two experts, top-1
-by a float32 router) and a toy position encoding (none; the mixer is order-aware by itself) show the
-other registries. None of this is a model of anyone's."""
+by a float32 router) and no position encoding on that layer (the mixer is order-aware by itself) show the
+other registries; a second test registers a toy position encoding (angles that grow with the square
+root of the position, over the first half of each head) for the framework's own attention mixer. None
+of this is a model of anyone's."""
 
 from __future__ import annotations
 
@@ -191,3 +193,100 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
     for k in reqs:
         torch.testing.assert_close(mixed[k], want[k], rtol=1e-4, atol=1e-4)
     assert bm.slots.in_use == set() and all(len(p.free_pool) == p.num_blocks for p in bm.pools)
+
+
+@dataclass(frozen=True)
+class SqrtAnglesSpec:
+    rotary_dim: int
+    rate: float
+    kind: str = "toy_sqrt_angles"
+
+
+def register_toy_position():
+    from mini_engine_amd.parts import POSITION_ENCODINGS, PositionEncoding
+
+    class SqrtAngles(PositionEncoding):
+        """angle[p, j] = rate * sqrt(p) / (j + 1): not a function of distances alone, so a table
+        read at a wrong row or a portion that restarts at zero changes the logits."""
+
+        def tables(self, num_positions=1):
+            rd = self.spec.rotary_dim
+            p = torch.arange(max(num_positions, 256), dtype=torch.float32, device=self.device)
+            angle = self.spec.rate * p.sqrt()[:, None] / torch.arange(1, rd // 2 + 1, device=self.device)
+            return torch.stack((angle.cos(), angle.sin()), dim=1).contiguous()
+
+    POSITION_ENCODINGS.register("toy_sqrt_angles", SqrtAngles)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_position_encoding_is_registered_and_used_by_the_attention_mixer(dtype):
+    import plain_qwen3 as plain
+    from mini_engine_amd import EngineConfig
+    from mini_engine_amd.config import AttentionSpec, GatedMlpSpec, LayerSpec, ModelPlan, NormSpec
+    from mini_engine_amd.engine.batch import StepItem
+    from mini_engine_amd.engine.runner import ModelRunner
+    from mini_engine_amd.engine.sequence import Sequence
+    from mini_engine_amd.parts import Decoder
+    from mini_engine_amd.weights import RandomSource
+
+    register_toy_position()
+    h, nh, nkv, d, rd = 64, 4, 2, 32, 16
+    norm = NormSpec(dim=h, eps=1e-5)
+    layer = LayerSpec(mixer=AttentionSpec(hidden_size=h, num_heads=nh, num_kv_heads=nkv, head_dim=d, scale=0.3,
+                                          qk_norm_eps=None, position=SqrtAnglesSpec(rd, 1.7)),
+                      ffn=GatedMlpSpec(hidden_size=h, intermediate_size=96), mixer_norm=norm, ffn_norm=norm,
+                      mixer_prefix="t.attn", ffn_prefix="t.mlp", mixer_norm_name="t.n1", ffn_norm_name="t.n2")
+    plan = ModelPlan(architecture="ToyPositionForTests", vocab_size=113, hidden_size=h, layers=(layer,), order=(0,),
+                     final_norm=norm, embed_name="t.embed", final_norm_name="t.norm", head_name="t.head",
+                     tie_word_embeddings=False, max_position_embeddings=256)
+    dec = Decoder(plan, dtype, "cuda")
+    wants = dec.weight_wants()
+    src = RandomSource(wants, seed=5, std=0.2, norm_std=0.1, device="cpu")
+    # matrices rounded to bfloat16, so that both dtypes and the plain implementation see the same values
+    weights = {n: (src.get(n).to(torch.bfloat16).float() if w.role == "matrix" else src.get(n))
+               for n, w in wants.items()}
+
+    class Source:
+        def shapes(self):
+            return {n: tuple(t.shape) for n, t in weights.items()}
+
+        def get(self, n):
+            return weights[n]
+
+    dec.load(Source())
+    runner = ModelRunner(dec, EngineConfig(block_size=16, num_blocks=16, max_num_seqs=2, dtype=str(dtype)[6:],
+                                           max_model_len=128))
+    bm = runner.new_block_manager()
+    tokens = torch.randint(0, 113, (70,), generator=torch.Generator().manual_seed(3)).tolist()
+
+    def rotate(x, cos, sin):  # the first rd elements of each head, pairs (j, j + rd/2)
+        return torch.cat((plain.apply_rope(x[..., :rd], cos, sin), x[..., rd:]), dim=-1)
+
+    w = {n: t.float() for n, t in weights.items()}
+    t = len(tokens)
+    x = w["t.embed"][torch.tensor(tokens)]
+    hn = plain.rms_norm(x, w["t.n1"], 1e-5)
+    q = (hn @ w["t.attn.q_proj.weight"].T).view(t, nh, d)
+    k = (hn @ w["t.attn.k_proj.weight"].T).view(t, nkv, d)
+    v = (hn @ w["t.attn.v_proj.weight"].T).view(t, nkv, d)
+    angle = 1.7 * torch.arange(t, dtype=torch.float32).sqrt()[:, None] / torch.arange(1, rd // 2 + 1)
+    cos, sin = torch.cat((angle, angle), -1).cos(), torch.cat((angle, angle), -1).sin()
+    a = plain.grouped_causal_attention(rotate(q, cos, sin), rotate(k, cos, sin), v, 0.3)
+    x = x + a.reshape(t, -1) @ w["t.attn.o_proj.weight"].T
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["t.n2"], 1e-5), w, "t.mlp")
+    want = plain.rms_norm(x, w["t.norm"], 1e-5) @ w["t.head"].T
+    no_rotation = plain.grouped_causal_attention(q, k, v, 0.3)
+    assert (a - no_rotation).abs().max() > 0.05  # the encoding matters at these sizes
+
+    seq, got = Sequence(tokens), []
+    for n in (33, 2, 19, 1, 1, 14):  # portions and single tokens
+        lo = seq.num_computed_tokens
+        assert bm.try_allocate(seq, lo + n)
+        got.append(runner.step([StepItem(seq, tokens[lo : lo + n], lo, list(range(n)))]).float().cpu())
+        seq.num_computed_tokens += n
+    bm.free(seq)
+    got = torch.cat(got)
+    if dtype is torch.float32:
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+    else:
+        assert (got - want).abs().max() < 0.04 * want.abs().max()
