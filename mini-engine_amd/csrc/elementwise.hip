@@ -388,23 +388,116 @@ __global__ __launch_bounds__(256) void qk_norm_rope_scatter_kernel(
   }
 }
 
-// The same work for the common geometry (head size a power of two from 16 to 256, rotary over the
-// whole head or none): a lane owns eight consecutive dims of the lower half of a head and their rotary
-// partners half a head away, so no value has to cross lanes for the rotation, loads and stores are
-// 8 elements wide (16 bytes in bfloat16), and a wave handles 64 / (d/16) heads at a time. Unit u of the
-// grid is (token, head) = (u / heads, u % heads).
+// Eight consecutive elements, moved as one access.
 template <typename T>
 struct alignas(sizeof(T) * 8) Pack8 {
   T v[8];
 };
 
+// Values of many consecutive tokens: one block per (16-slot segment of a page that the step's tokens
+// touch, kv head). The segment's tokens are read row by row into LDS and written transposed, 16 slots
+// (32 bytes) per head dimension, instead of one 2-byte store per (token, dimension). Segments are
+// numbered over all items; item i touches segments pos0/16 .. (pos0 + qlen - 1)/16 of its positions.
+template <typename T>
+struct VScatterLds {
+  T tile[16][ME_MAX_HEAD_DIM + 2];
+  int item, seg;
+};
+
+// The work of one block (256 threads, all of which call it): segment `segment` of the step, kv head `kvh`.
+template <typename T>
+__device__ __forceinline__ void v_scatter_segment(VScatterLds<T>& lds, int segment, int kvh, const T* __restrict__ qkv,
+                                                  const int* __restrict__ positions, const int* __restrict__ item_start,
+                                                  int num_items, const int* __restrict__ block_table, int table_width,
+                                                  T* __restrict__ v_cache, int nh, int nkv, int d, int bs) {
+  T(&tile)[16][ME_MAX_HEAD_DIM + 2] = lds.tile;
+  int& s_item = lds.item;
+  int& s_seg = lds.seg;
+  if (threadIdx.x == 0) {
+    int left = segment, it = 0;
+    for (; it < num_items; ++it) {
+      const int p0 = positions[item_start[it]], n = item_start[it + 1] - item_start[it];
+      const int segs = (p0 + n - 1) / 16 - p0 / 16 + 1;
+      if (left < segs) break;
+      left -= segs;
+    }
+    s_item = it;
+    s_seg = left;
+  }
+  __syncthreads();
+  const int item = s_item;
+  if (item >= num_items) return;
+  const int t0 = item_start[item], n = item_start[item + 1] - t0;
+  const int p0 = positions[t0];
+  const int seg_pos = (p0 / 16 + s_seg) * 16;           // first position of the segment
+  const int first = max(seg_pos, p0), last = min(seg_pos + 15, p0 + n - 1);  // positions present
+  const int width = (nh + 2 * nkv) * d;
+  const T* src = qkv + (size_t)(nh + nkv + kvh) * d;
+  const bool wide = d % 8 == 0 && (((uintptr_t)qkv | (uintptr_t)v_cache) & (sizeof(T) * 8 - 1)) == 0;
+  if (wide) {  // rows in pieces of eight elements
+    for (int idx = threadIdx.x; idx < (last - first + 1) * (d / 8); idx += blockDim.x) {
+      const int row = idx / (d / 8), col = idx % (d / 8) * 8;
+      const Pack8<T> v = *reinterpret_cast<const Pack8<T>*>(src + (size_t)(t0 + first - p0 + row) * width + col);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) tile[first - seg_pos + row][col + j] = v.v[j];
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < (last - first + 1) * d; idx += blockDim.x) {
+      const int row = idx / d, col = idx % d;
+      tile[first - seg_pos + row][col] = src[(size_t)(t0 + first - p0 + row) * width + col];
+    }
+  }
+  __syncthreads();
+  const int page = block_table[(size_t)item * table_width + seg_pos / bs];
+  if (page < 0) return;
+  T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + seg_pos % bs;
+  const int lo = first - seg_pos, hi = last - seg_pos;
+  if (wide && lo == 0 && hi == 15) {  // a whole segment: eight slots of one dimension per store
+    for (int idx = threadIdx.x; idx < d * 2; idx += blockDim.x) {
+      const int dim = idx >> 1, half = idx & 1;
+      Pack8<T> v;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v.v[j] = tile[half * 8 + j][dim];
+      *reinterpret_cast<Pack8<T>*>(dst + (size_t)dim * bs + half * 8) = v;
+    }
+    return;
+  }
+  for (int idx = threadIdx.x; idx < d * 16; idx += blockDim.x) {
+    const int dim = idx / 16, slot = idx % 16;
+    if (slot >= lo && slot <= hi) dst[(size_t)dim * bs + slot] = tile[slot][dim];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void v_scatter_tiles_kernel(const T* __restrict__ qkv, const int* __restrict__ positions,
+                                                              const int* __restrict__ item_start, int num_items,
+                                                              const int* __restrict__ block_table, int table_width,
+                                                              T* __restrict__ v_cache, int nh, int nkv, int d, int bs) {
+  __shared__ VScatterLds<T> lds;
+  v_scatter_segment<T>(lds, blockIdx.x, blockIdx.y, qkv, positions, item_start, num_items, block_table, table_width,
+                       v_cache, nh, nkv, d, bs);
+}
+
+// The same work for the common geometry (head size a power of two from 16 to 256, rotary over the
+// whole head or none): a lane owns eight consecutive dims of the lower half of a head and their rotary
+// partners half a head away, so no value has to cross lanes for the rotation, loads and stores are
+// 8 elements wide (16 bytes in bfloat16), and a wave handles 64 / (d/16) heads at a time. Unit u of the
+// grid is (token, head) = (u / heads, u % heads).
 template <typename T, int LPH>  // LPH = d / 16 lanes per head
 __global__ __launch_bounds__(256) void qk_norm_rope_scatter_wide_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
     const float* __restrict__ rope_table, const int* __restrict__ positions, const int* __restrict__ token_item,
     const int* __restrict__ block_table, int table_width, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, int num_tokens, int nh, int nkv, int bs, float eps, int write_kv, int skip_v) {
+    T* __restrict__ v_cache, int num_tokens, int nh, int nkv, int bs, float eps, int write_kv, int skip_v,
+    const int* __restrict__ item_start, int num_items, unsigned own_blocks) {
   constexpr int D = LPH * 16, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
+  if (blockIdx.x >= own_blocks) {  // the blocks behind this kernel's own write the values, a page segment each
+    __shared__ VScatterLds<T> lds;
+    const unsigned v = blockIdx.x - own_blocks;
+    v_scatter_segment<T>(lds, v / nkv, v % nkv, qkv, positions, item_start, num_items, block_table, table_width, v_cache,
+                         nh, nkv, D, bs);
+    return;
+  }
   const int lane = threadIdx.x & (ME_WAVE - 1);
   const int sub = lane / LPH, p = lane % LPH;
   const int heads_row = write_kv ? nh + 2 * nkv : nh;
@@ -488,19 +581,23 @@ template <typename T>
 static bool launch_wide(const T* qkv, const float* q_w, const float* k_w, const float* rope_table, const int* positions,
                         const int* token_item, const int* block_table, int table_width, T* q_out, T* k_cache,
                         T* v_cache, int num_tokens, int nh, int nkv, int d, int bs, float eps, int write_kv, int skip_v,
-                        hipStream_t stream) {
+                        const int* item_start, int num_items, int num_segments, hipStream_t stream) {
   // 8-element accesses need aligned bases (row lengths are multiples of the head size, itself one of 16)
   const uintptr_t align = sizeof(T) * 8 - 1;
   if (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache) & align) return false;
   if (((uintptr_t)q_w | (uintptr_t)k_w | (uintptr_t)rope_table) & 15) return false;
   const int heads = write_kv ? (skip_v ? nh + nkv : nh + 2 * nkv) : nh;
   const long long units = (long long)num_tokens * heads;
+  // with skip_v the values are written by blocks of the same launch, one per (page segment, kv head)
+  const long long value_blocks = skip_v ? (long long)num_segments * nkv : 0;
 #define ME_WIDE(LPH)                                                                                                  \
   {                                                                                                                   \
     const long long per_block = 4 * (64 / LPH);                                                                       \
-    qk_norm_rope_scatter_wide_kernel<T, LPH><<<(unsigned)((units + per_block - 1) / per_block), 256, 0, stream>>>(    \
+    const long long own = (units + per_block - 1) / per_block, all = own + value_blocks;                              \
+    if (all > 0x7fffffffLL) return false;                                                                             \
+    qk_norm_rope_scatter_wide_kernel<T, LPH><<<(unsigned)all, 256, 0, stream>>>(                                      \
         qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, q_out, k_cache, v_cache,          \
-        num_tokens, nh, nkv, bs, eps, write_kv, skip_v);                                                              \
+        num_tokens, nh, nkv, bs, eps, write_kv, skip_v, item_start, num_items, (unsigned)own);                        \
     return true;                                                                                                      \
   }
   switch (d) {
@@ -514,71 +611,24 @@ static bool launch_wide(const T* qkv, const float* q_w, const float* k_w, const 
   return false;
 }
 
-// Values of many consecutive tokens: one block per (16-slot segment of a page that the step's tokens
-// touch, kv head). The segment's tokens are read row by row into LDS and written transposed, 16 slots
-// (32 bytes) per head dimension, instead of one 2-byte store per (token, dimension). Segments are
-// numbered over all items; item i touches segments pos0/16 .. (pos0 + qlen - 1)/16 of its positions.
+// One launch where the wide kernel takes the geometry (it writes the values' page segments with blocks of
+// its own); else the general kernel, and the page-segment kernel behind it when `tiles`.
 template <typename T>
-__global__ __launch_bounds__(256) void v_scatter_tiles_kernel(const T* __restrict__ qkv, const int* __restrict__ positions,
-                                                              const int* __restrict__ item_start, int num_items,
-                                                              const int* __restrict__ block_table, int table_width,
-                                                              T* __restrict__ v_cache, int nh, int nkv, int d, int bs) {
-  __shared__ T tile[16][ME_MAX_HEAD_DIM + 2];
-  __shared__ int s_item, s_seg;
-  if (threadIdx.x == 0) {
-    int left = blockIdx.x, it = 0;
-    for (; it < num_items; ++it) {
-      const int p0 = positions[item_start[it]], n = item_start[it + 1] - item_start[it];
-      const int segs = (p0 + n - 1) / 16 - p0 / 16 + 1;
-      if (left < segs) break;
-      left -= segs;
-    }
-    s_item = it;
-    s_seg = left;
-  }
-  __syncthreads();
-  const int item = s_item;
-  if (item >= num_items) return;
-  const int kvh = blockIdx.y;
-  const int t0 = item_start[item], n = item_start[item + 1] - t0;
-  const int p0 = positions[t0];
-  const int seg_pos = (p0 / 16 + s_seg) * 16;           // first position of the segment
-  const int first = max(seg_pos, p0), last = min(seg_pos + 15, p0 + n - 1);  // positions present
-  const int width = (nh + 2 * nkv) * d;
-  const T* src = qkv + (size_t)(nh + nkv + kvh) * d;
-  const bool wide = d % 8 == 0 && (((uintptr_t)qkv | (uintptr_t)v_cache) & (sizeof(T) * 8 - 1)) == 0;
-  if (wide) {  // rows in pieces of eight elements
-    for (int idx = threadIdx.x; idx < (last - first + 1) * (d / 8); idx += blockDim.x) {
-      const int row = idx / (d / 8), col = idx % (d / 8) * 8;
-      const Pack8<T> v = *reinterpret_cast<const Pack8<T>*>(src + (size_t)(t0 + first - p0 + row) * width + col);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) tile[first - seg_pos + row][col + j] = v.v[j];
-    }
-  } else {
-    for (int idx = threadIdx.x; idx < (last - first + 1) * d; idx += blockDim.x) {
-      const int row = idx / d, col = idx % d;
-      tile[first - seg_pos + row][col] = src[(size_t)(t0 + first - p0 + row) * width + col];
-    }
-  }
-  __syncthreads();
-  const int page = block_table[(size_t)item * table_width + seg_pos / bs];
-  if (page < 0) return;
-  T* dst = v_cache + ((size_t)page * nkv + kvh) * d * bs + seg_pos % bs;
-  const int lo = first - seg_pos, hi = last - seg_pos;
-  if (wide && lo == 0 && hi == 15) {  // a whole segment: eight slots of one dimension per store
-    for (int idx = threadIdx.x; idx < d * 2; idx += blockDim.x) {
-      const int dim = idx >> 1, half = idx & 1;
-      Pack8<T> v;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) v.v[j] = tile[half * 8 + j][dim];
-      *reinterpret_cast<Pack8<T>*>(dst + (size_t)dim * bs + half * 8) = v;
-    }
+static void launch_qk_scatter(const T* qkv, const float* q_w, const float* k_w, const float* rope_table,
+                              const int* positions, const int* token_item, const int* block_table, int table_width,
+                              T* q_out, T* k_cache, T* v_cache, int num_tokens, int nh, int nkv, int d, int rd, int bs,
+                              float eps, int write_kv, bool wide, bool tiles, int hpb, dim3 grid, const int* item_start,
+                              int num_items, int num_segments, hipStream_t stream) {
+  if (wide && launch_wide<T>(qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, q_out, k_cache,
+                             v_cache, num_tokens, nh, nkv, d, bs, eps, write_kv, tiles ? 1 : 0, item_start, num_items,
+                             tiles ? num_segments : 0, stream))
     return;
-  }
-  for (int idx = threadIdx.x; idx < d * 16; idx += blockDim.x) {
-    const int dim = idx / 16, slot = idx % 16;
-    if (slot >= lo && slot <= hi) dst[(size_t)dim * bs + slot] = tile[slot][dim];
-  }
+  qk_norm_rope_scatter_kernel<T><<<grid, 256, 0, stream>>>(qkv, q_w, k_w, rope_table, positions, token_item, block_table,
+                                                           table_width, q_out, k_cache, v_cache, nh, nkv, d, rd, bs, eps,
+                                                           write_kv, hpb, tiles ? 1 : 0);
+  if (tiles)
+    v_scatter_tiles_kernel<T><<<dim3(num_segments, nkv), 256, 0, stream>>>(qkv, positions, item_start, num_items,
+                                                                         block_table, table_width, v_cache, nh, nkv, d, bs);
 }
 
 // rope_table: float32 [num_positions, 2, rd / 2] or null; every position of the step must be below
@@ -604,27 +654,13 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
   dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
   if (grid.y > 65535) return me_fail("me_qk_norm_rope_scatter: too many heads");
   const bool wide = (rd == d || rope_table == nullptr) && (d & (d - 1)) == 0 && d >= 16 && d <= 256;
-  if (dtype == ME_F32) {
-    if (!(wide && launch_wide<float>((const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
-                                     table_width, (float*)q_out, (float*)k_cache, (float*)v_cache, num_tokens, nh, nkv,
-                                     d, bs, eps, write_kv, tiles ? 1 : 0, stream)))
-      qk_norm_rope_scatter_kernel<float><<<grid, 256, 0, stream>>>(
-          (const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (float*)q_out,
-          (float*)k_cache, (float*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb, tiles ? 1 : 0);
-    if (tiles)
-      v_scatter_tiles_kernel<float><<<dim3(num_segments, nkv), 256, 0, stream>>>(
-          (const float*)qkv, positions, item_start, num_items, block_table, table_width, (float*)v_cache, nh, nkv, d, bs);
-  } else {
-    if (!(wide && launch_wide<bf16_t>((const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table,
-                                      table_width, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, num_tokens, nh,
-                                      nkv, d, bs, eps, write_kv, tiles ? 1 : 0, stream)))
-      qk_norm_rope_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
-          (const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width, (bf16_t*)q_out,
-          (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, rd, bs, eps, write_kv, hpb, tiles ? 1 : 0);
-    if (tiles)
-      v_scatter_tiles_kernel<bf16_t><<<dim3(num_segments, nkv), 256, 0, stream>>>(
-          (const bf16_t*)qkv, positions, item_start, num_items, block_table, table_width, (bf16_t*)v_cache, nh, nkv, d,
-          bs);
-  }
+  if (dtype == ME_F32)
+    launch_qk_scatter<float>((const float*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width,
+                             (float*)q_out, (float*)k_cache, (float*)v_cache, num_tokens, nh, nkv, d, rd, bs, eps,
+                             write_kv, wide, tiles, hpb, grid, item_start, num_items, num_segments, stream);
+  else
+    launch_qk_scatter<bf16_t>((const bf16_t*)qkv, q_w, k_w, rope_table, positions, token_item, block_table, table_width,
+                              (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, num_tokens, nh, nkv, d, rd, bs, eps,
+                              write_kv, wide, tiles, hpb, grid, item_start, num_items, num_segments, stream);
   return me_check_launch("me_qk_norm_rope_scatter");
 }
