@@ -207,10 +207,16 @@ class BlockManager:
         """
         while len(seq.block_tables) < len(self.pools):
             seq.block_tables.append([])
+        need = self.blocks_needed(num_tokens)
+        if not cached_blocks and (self.slots is None or seq.state_slot >= 0):
+            for table in seq.block_tables:
+                if len(table) < need:
+                    break
+            else:
+                return True  # the usual decode step: the last page still has room
         cached = self._per_group(cached_blocks)
         if any(cached) and any(seq.block_tables):
             raise ValueError("cached blocks can only seed an empty block table")
-        need = self.blocks_needed(num_tokens)
         plans = []
         for pool, table, hit in zip(self.pools, seq.block_tables, cached):
             num_new = need - len(table) - len(hit)
@@ -240,6 +246,7 @@ class BlockManager:
                 if b >= 0:
                     pool.release(b)
             table.clear()
+        seq.table_epoch += 1
         seq.block_hashes.clear()
         if self.slots is not None and seq.state_slot >= 0:
             self.slots.give_back(seq.state_slot)
@@ -257,6 +264,7 @@ class BlockManager:
                 if table[i] >= 0:
                     pool.release(table[i])
                     table[i] = -1
+                    seq.table_epoch += 1
                     freed += 1
         return freed
 

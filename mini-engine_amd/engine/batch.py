@@ -121,8 +121,16 @@ def pack_host(items: list[StepItem], num_groups: int, widths: list[int] | None =
     return arr, t, b, r, widths
 
 
-def validate_items(items: list[StepItem], vocab_size: int, block_size: int, groups, max_len: int | None = None) -> None:
-    """Host-side checks that make every index a kernel will form a valid one."""
+def check_pages(table: list[int], first: int, need: int, group: int) -> None:
+    """Entries ``first .. need - 1`` of a block table must name pages (not -1, a page given back)."""
+    if first < need and min(table[first:need]) < 0:
+        raise ValueError(f"group {group}: a page the step reads or writes was already given back")
+
+
+def validate_items(items: list[StepItem], vocab_size: int, block_size: int, groups, max_len: int | None = None,
+                   pages: bool = True) -> None:
+    """Host-side checks that make every index a kernel will form a valid one. ``pages=False`` leaves
+    the scan of the block tables' entries to the caller (:func:`check_pages`)."""
     if not items:
         raise ValueError("a step needs at least one item")
     for it in items:
@@ -139,15 +147,14 @@ def validate_items(items: list[StepItem], vocab_size: int, block_size: int, grou
         for w in it.want:
             if not 0 <= w < n:
                 raise ValueError(f"wanted place {w} is outside the item's {n} tokens")
+        need = -(-(it.start + n) // block_size)
         for g, spec in enumerate(groups):
             table = it.seq.block_tables[g]
-            need = -(-(it.start + n) // block_size)
             if len(table) < need:
                 raise ValueError(f"block table of group {g} has {len(table)} pages, {need} are needed")
-            first_key = max(0, it.start - spec.window + 1) if spec.window > 0 else 0
-            for page in table[first_key // block_size : need]:
-                if page < 0:
-                    raise ValueError(f"group {g}: a page the step reads or writes was already given back")
+            if pages:
+                first_key = max(0, it.start - spec.window + 1) if spec.window > 0 else 0
+                check_pages(table, first_key // block_size, need, g)
 
 
 def make_batch(items: list[StepItem], num_groups: int, device, spare_block: int = 0, spare_slot: int = 0) -> StepBatch:

@@ -17,7 +17,7 @@ from ..cache.block_manager import BlockManager
 from ..cache.storage import CacheStorage, plan_layout
 from ..config.engine_config import EngineConfig
 from ..parts.decoder import Decoder
-from .batch import StepBatch, StepItem, make_batch, pack_host, section_offsets, validate_items
+from .batch import StepBatch, StepItem, check_pages, make_batch, pack_host, section_offsets, validate_items
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
@@ -43,6 +43,8 @@ class ModelRunner:
         self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, StepBatch, torch.Tensor, torch.Tensor]] = {}
         self._graph_pool = None
         self._copy_done: dict[int, torch.cuda.Event] = {}
+        # per bucket and row: (sequence, its table_epoch, pages written per group) of the last replay
+        self._rows: dict[int, list] = {}
         self.graph_replays = 0
         self.eager_steps = 0
 
@@ -58,11 +60,13 @@ class ModelRunner:
 
         After a replayed step the result is a view of the graph's output buffer: read it before the
         next step."""
+        replay = self._graph_eligible(items)
+        # a replayed step checks the pages of its block tables while it writes them into the graph's buffer
         validate_items(items, self.decoder.plan.vocab_size, self.config.block_size, self.layout.groups,
-                       self.config.max_model_len)
+                       self.config.max_model_len, pages=not replay)
         if self.layout.has_state:
             self.storage.zero_state([it.seq.state_slot for it in items if it.start == 0 and it.seq.state_slot >= 0])
-        if self._graph_eligible(items):
+        if replay:
             return self._replay(items)
         self.eager_steps += 1
         batch = make_batch(items, self.num_groups, self.device, self.storage.spare_block, self.storage.spare_slot)
@@ -110,17 +114,62 @@ class ModelRunner:
             if b not in self._graphs:
                 self._capture(b)
 
+    def _refill(self, bucket: int, batch: StepBatch, host: torch.Tensor, items: list[StepItem]) -> None:
+        """Write this step's indices into the bucket's pinned host buffer, which still holds the last
+        replay's. Token, position, length and slot of every row are written anew. A row of a block
+        table is only extended by the pages its sequence has gained when the row held the same
+        sequence's table last time and nothing but appended pages has changed it since
+        (``Sequence.table_epoch``); tables of window groups, whose entries change as pages are given
+        back, are always written whole. Rows beyond the items point at the spare page and slot."""
+        a = host.numpy()
+        sec, n = batch.sections, len(items)
+        rows = self._rows.setdefault(bucket, [None] * bucket)
+        spare_block, spare_slot = self.storage.spare_block, self.storage.spare_slot
+        tok_o, pos_o, ctx_o, slot_o = (sec[k][0] for k in ("token_ids", "positions", "item_ctx", "state_slots"))
+        starts = [it.start for it in items]
+        pad = bucket - n
+        a[tok_o : tok_o + bucket] = [it.tokens[0] for it in items] + [0] * pad
+        a[pos_o : pos_o + bucket] = starts + [0] * pad
+        a[ctx_o : ctx_o + bucket] = [s + 1 for s in starts] + [1] * pad
+        a[slot_o : slot_o + bucket] = [it.seq.state_slot if it.seq.state_slot >= 0 else spare_slot for it in items] + [spare_slot] * pad
+        bases = [sec[f"table{g}"][0] for g in range(self.num_groups)]
+        windows = [g.window for g in self.layout.groups]
+        for i, it in enumerate(items):
+            seq, row = it.seq, rows[i]
+            same = row is not None and row[0] is seq and row[1] == seq.table_epoch
+            written = row[2] if same else [0] * self.num_groups
+            rows[i] = None  # until the row is complete, should a check below raise
+            need = it.start // self.config.block_size + 1
+            for g, table in enumerate(seq.block_tables):
+                w = batch.widths[g]
+                o = bases[g] + i * w
+                have = written[g] if same and windows[g] == 0 else -1
+                if have < 0:
+                    a[o : o + w] = spare_block
+                    have = 0
+                # pages this step reads or writes that were not checked when an earlier step wrote them
+                first_key = max(0, it.start - windows[g] + 1) if windows[g] > 0 else 0
+                check_pages(table, max(have, first_key // self.config.block_size), need, g)
+                if have < len(table):
+                    a[o + have : o + len(table)] = table[have:]
+                    written[g] = len(table)
+            rows[i] = (seq, seq.table_epoch, written)
+        for i in range(n, bucket):
+            if rows[i] is not None:
+                for g in range(self.num_groups):
+                    o = bases[g] + i * batch.widths[g]
+                    a[o : o + batch.widths[g]] = spare_block
+                rows[i] = None
+
     def _replay(self, items: list[StepItem]) -> torch.Tensor:
         n = len(items)
         bucket = next(b for b in batch_buckets(self.config.max_num_seqs) if b >= n)
         entry = self._graphs.get(bucket) or self._capture(bucket)
         graph, batch, host, logits = entry
-        arr, *_ = pack_host(items, self.num_groups, batch.widths, pad_items=bucket - n,
-                            spare_block=self.storage.spare_block, spare_slot=self.storage.spare_slot)
         done = self._copy_done.get(bucket)
         if done is not None:
             done.synchronize()  # the previous upload from this pinned buffer has been read
-        host.numpy()[:] = arr
+        self._refill(bucket, batch, host, items)
         batch.buf.copy_(host, non_blocking=True)
         done = done or torch.cuda.Event()
         done.record()
