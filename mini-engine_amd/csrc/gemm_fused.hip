@@ -10,7 +10,8 @@
 //   epilogue SWIGLU: W holds gate rows [0, N) and up rows [N, 2N); a block computes 16 gate columns and
 //                    the 16 matching up columns and writes silu(gate) * up.
 //
-// A block owns 16 output columns and all M rows; its WAVES waves split k in interleaved chunks of 32
+// A block owns 16 output columns (64 for products with very many columns, whose blocks then share the
+// loads of x among four tiles of columns) and all M rows; its WAVES waves split k in interleaved chunks of 32
 // and add their partial sums through LDS in wave order. Products use v_mfma_f32_16x16x32_bf16 with
 // the transposed arrangement (C^T[n, m] = sum_k W[n, k] X[m, k]): lane l feeds W[n0 + l%16][8 k] and
 // X[m0 + l%16][8 k] (k = 32 c + 8 (l/16) ..), both contiguous in memory, and receives
@@ -20,21 +21,28 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, int WAVES, int U, bool NORM, bool SWIGLU, typename OutT>
+template <int MT, int WAVES, int U, bool NORM, bool SWIGLU, typename OutT, int NT = 1>
 __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
     const bf16_t* __restrict__ X, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
     const float* __restrict__ w_norm, float eps, float* __restrict__ x_out, const bf16_t* __restrict__ W,
     OutT* __restrict__ C, int M, int N, int K, int chunks_per_split) {
-  constexpr int ACCS = SWIGLU ? 2 : 1;
+  // ACCS tiles of 16 weight rows per block: gate and up rows of the same 16 columns (SWIGLU), or NT
+  // neighbouring tiles of 16 columns, which share the loads of x (products with very many columns)
+  static_assert(!SWIGLU || NT == 1, "the gated form computes one tile of columns per block");
+  constexpr int ACCS = SWIGLU ? 2 : NT;
   __shared__ float red[WAVES][MT * ACCS][64][4];
   __shared__ float ssq[WAVES][MT][64];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int r = lane & 15, g = lane >> 4;
-  const int n = n0 + r;
-  const bool n_ok = n < N;
-  const bf16_t* wrow = W + (size_t)(n_ok ? n : 0) * K;
-  const bf16_t* wrow_up = SWIGLU ? W + ((size_t)N + (n_ok ? n : 0)) * K : nullptr;
+  const bf16_t* wrow[ACCS];
+  bool n_ok[ACCS];
+#pragma unroll
+  for (int a = 0; a < ACCS; ++a) {
+    const int n = SWIGLU ? n0 + r : n0 + a * 16 + r;
+    n_ok[a] = n < N;
+    wrow[a] = W + ((SWIGLU && a ? (size_t)N : 0) + (size_t)(n_ok[a] ? n : 0)) * K;
+  }
   float4_t acc[MT][ACCS];
   float ss[MT];
 #pragma unroll
@@ -56,11 +64,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
     for (int u = 0; u < U; ++u) {
       const int k = (c0 + WAVES * u) * 32 + g * 8;
       const bool k_ok = k < K && c0 + WAVES * u < last;  // K % 8 == 0 is checked on the host
-      a[u][0] = bf16x8_t{};
-      if (n_ok && k_ok) a[u][0] = *reinterpret_cast<const bf16x8_t*>(wrow + k);
-      if (SWIGLU) {
-        a[u][ACCS - 1] = bf16x8_t{};
-        if (n_ok && k_ok) a[u][ACCS - 1] = *reinterpret_cast<const bf16x8_t*>(wrow_up + k);
+#pragma unroll
+      for (int aa = 0; aa < ACCS; ++aa) {
+        a[u][aa] = bf16x8_t{};
+        if (n_ok[aa] && k_ok) a[u][aa] = *reinterpret_cast<const bf16x8_t*>(wrow[aa] + k);
       }
     }
 #pragma unroll
@@ -135,16 +142,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
       scale = rsqrtf(total / (float)K + eps);
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float v0 = 0.f, v1 = 0.f;
-      for (int w = 0; w < WAVES; ++w) {
-        v0 += red[w][t * ACCS][l][j];
-        if (SWIGLU) v1 += red[w][t * ACCS + 1][l][j];
+    for (int tile = 0; tile < (SWIGLU ? 1 : NT); ++tile) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v0 = 0.f, v1 = 0.f;
+        for (int w = 0; w < WAVES; ++w) {
+          v0 += red[w][t * ACCS + tile][l][j];
+          if (SWIGLU) v1 += red[w][t * ACCS + 1][l][j];
+        }
+        v0 *= scale;
+        float y = v0;
+        if (SWIGLU) y = v0 / (1.f + expf(-v0)) * (v1 * scale);
+        const int col = nb + tile * 16 + j;
+        if (col < N) C[(size_t)m * N + col] = from_float<OutT>(y);
       }
-      v0 *= scale;
-      float y = v0;
-      if (SWIGLU) y = v0 / (1.f + expf(-v0)) * (v1 * scale);
-      if (nb + j < N) C[(size_t)m * N + nb + j] = from_float<OutT>(y);
     }
   }
 }
@@ -169,6 +180,8 @@ static void launch_variant(bool norm, bool swiglu, const bf16_t* X, const float*
 #undef ME_LAUNCH
 }
 
+#define WIDE_MIN_COLUMNS 32768
+
 template <typename OutT>
 static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
                          const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
@@ -177,6 +190,13 @@ static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x
   // up to 16 rows: as many chunks of 32 k per wave and round as it takes to have all of k in flight at
   // once (a second round of loads costs a memory round trip, which is most of such a kernel's time)
   const int chunks = ((K + 31) / 32 + splits - 1) / splits;  // per block
+  if (mt == 1 && M > 2 && !norm && !swiglu && splits == 1 && N >= WIDE_MIN_COLUMNS) {
+    // very many columns (the output head) and more than a row or two: a block computes 64 columns from
+    // one set of loads of x (at 8 rows and 151,936 columns 63 us against 69; at one row it is slower)
+    gemm_small_kernel<1, 8, 4, false, false, OutT, 4><<<dim3((N + 63) / 64), 8 * 64, 0, stream>>>(
+        X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, chunks);
+    return;
+  }
   if (mt == 1 && chunks > 8 * 8)
     launch_variant<1, 8, 12, OutT>(norm, swiglu, X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, splits, stream);
   else if (mt == 1 && chunks > 8 * 4)

@@ -191,6 +191,22 @@ def test_gemm_bf16_small_with_norm_prologue_and_swiglu_epilogue(m, n, k, with_de
         assert h.residual is xd and torch.equal(spare.cpu(), torch.full((m, k), 7.0))
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 32768, 64), (2, 33001, 520), (8, 40010, 1024), (16, 33001, 2056), (3, 32768 + 17, 72)])
+def test_gemm_bf16_small_with_very_many_columns(m, n, k):
+    """From 32,768 columns on (an output head) and three rows on, a block computes four tiles of 16
+    columns from one set of loads of x: column counts that are no multiple of 64, k over several rounds, both output types."""
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    w[-1] *= 5  # the last column stands out: a tile that stops short of it, or runs past it, shows
+    want = x.float() @ w.float().T
+    for out_dtype in (torch.float32, torch.bfloat16):
+        got = K().gemm_bf16_small(dev(x), dev(w), out_dtype).float().cpu()
+        scale = max(1.0, want.abs().max().item())
+        tol_abs = (2**-7 if out_dtype is torch.bfloat16 else 1e-4) * scale
+        assert (got - want).abs().max().item() <= tol_abs, (out_dtype, (got - want).abs().max().item(), scale)
+
+
 def test_normed_input_falls_back_to_the_separate_kernels():
     """More than 64 rows or float32: the add-and-norm kernel runs, in place, and the product follows."""
     for dtype, m in ((torch.bfloat16, 100), (torch.float32, 5)):
