@@ -954,32 +954,36 @@ __global__ __launch_bounds__(256) void attention_prefill_combine_kernel(const fl
   }
 }
 
-#define PF_NB 1
 #define PF_WAVES 8
-#define PF_COLUMNS (PF_NB * PF_WAVES * 16)  // query columns (token, head of the group) per block
+// Query columns (token, head of the group) per block: 16 or 32 per wave. The wider block reads each key
+// and value fragment once for two products and stages half as many tiles per product, which pays when a
+// step still gives every compute unit several blocks (long prompts).
+#define PF_COLUMNS_NARROW (PF_WAVES * 16)
+#define PF_COLUMNS_WIDE (2 * PF_WAVES * 16)
 
-extern "C" int me_attention_prefill_columns() { return PF_COLUMNS; }
+extern "C" int me_attention_prefill_columns(int wide) { return wide ? PF_COLUMNS_WIDE : PF_COLUMNS_NARROW; }
 
-template <int D>
+template <int D, int NB>
 static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const PrefillWork* work,
                           const int* bundle_first, const int* table, int width, bf16_t* out,
                           float* part_o, float* part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window,
                           float sl, int tpb, hipStream_t stream) {
   static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, PF_NB, PF_WAVES>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, NB, PF_WAVES>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, PrefillLds<D>::BYTES);
     if (e != hipSuccess) return me_fail("me_attention_prefill_bf16: cannot reserve %d bytes of LDS: %s",
                                         PrefillLds<D>::BYTES, hipGetErrorString(e));
     configured = true;
   }
-  attention_prefill_kernel<D, PF_NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
+  attention_prefill_kernel<D, NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
       q, kc, vc, work, bundle_first, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb);
   return 0;
 }
 
-// q [T, nh, d], packed new tokens. work: entries of eight ints laid out by the caller (item, first token and
-// number of tokens of the tile (at most me_attention_prefill_columns() / group), position of the first
+// q [T, nh, d], packed new tokens. columns: query columns per block, me_attention_prefill_columns(0) or (1).
+// work: entries of eight ints laid out by the caller (item, first token and
+// number of tokens of the tile (at most columns / group), position of the first
 // token, first key (a multiple of 64), last key, chunk or -1, 1 on the last entry of a bundle);
 // bundle_first int [num_bundles]: the first entry of each bundle. Every bundle is run by one block per kv
 // head. When a tile's keys are cut into chunks (max_chunks > 1), part_o float [T, nh, max_chunks, d] and
@@ -989,7 +993,7 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
                                          const int* block_table, int table_width, void* out, const int* work,
                                          const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
                                          const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
-                                         int d, int bs, int window, float scale, hipStream_t stream) {
+                                         int d, int bs, int window, float scale, int columns, hipStream_t stream) {
   const int num_work = num_bundles;
   if (num_items <= 0 || num_work <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
@@ -1002,7 +1006,10 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   if (!work || !bundle_first) return me_fail("me_attention_prefill_bf16: no work list");
   if (max_chunks < 1 || (max_chunks > 1 && (!part_o || !part_ml || !token_chunks || num_tokens <= 0)))
     return me_fail("me_attention_prefill_bf16: %d chunks need the partial buffers and the chunk counts", max_chunks);
-  const int tpb = PF_COLUMNS / group;
+  if (columns != PF_COLUMNS_NARROW && columns != PF_COLUMNS_WIDE)
+    return me_fail("me_attention_prefill_bf16: %d query columns per block (%d or %d)", columns, PF_COLUMNS_NARROW, PF_COLUMNS_WIDE);
+  const bool wide = columns == PF_COLUMNS_WIDE;
+  const int tpb = columns / group;
   const float sl = scale * LOG2E;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
@@ -1011,9 +1018,12 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   int rc = 0;
 #define ME_PREFILL_CASE(DD)                                                                                        \
   case DD:                                                                                                         \
-    rc = launch_prefill<DD>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table, table_width,    \
-                            (bf16_t*)out,                                                                          \
-                            part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb, stream);              \
+    rc = wide ? launch_prefill<DD, 2>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
+                                      table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
+                                      window, sl, tpb, stream)                                                     \
+              : launch_prefill<DD, 1>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
+                                      table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
+                                      window, sl, tpb, stream);                                                    \
     break;
   switch (d) {
     ME_PREFILL_CASE(32)

@@ -600,9 +600,11 @@ class PrefillPlan:
     attention's window, not on the layer, so a step builds it once."""
 
     def __init__(self, work: torch.Tensor, bundle_first: torch.Tensor, token_chunks: torch.Tensor | None,
-                 num_bundles: int, max_chunks: int):
+                 num_bundles: int, max_chunks: int, columns: int | None = None):
         self.work, self.bundle_first, self.token_chunks = work, bundle_first, token_chunks
         self.num_bundles, self.max_chunks = num_bundles, max_chunks
+        # query columns (token, head of the kv group) per block that the tiles were cut for
+        self.columns = lib().me_attention_prefill_columns(0) if columns is None else columns
 
 
 PIECE_OVERHEAD = 2  # what starting another piece of work costs a block, in key tiles (3 us against 1.5 us)
@@ -700,24 +702,55 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
 _PLANS: dict = {}  # the last plans made, by what they were made from: steps of a serving loop repeat
 
 
-def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device) -> PrefillPlan:
-    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device))
+def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,
+                 wide: bool | None = None) -> PrefillPlan:
+    """``wide``: blocks of twice as many query columns or not; None lets the step's size decide."""
+    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device), wide)
     plan = _PLANS.get(key)
     if plan is None:
         if len(_PLANS) >= 64:
             _PLANS.pop(next(iter(_PLANS)))
-        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device)
+        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device, wide)
     return plan
 
 
-def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device) -> PrefillPlan:
-    tpb = lib().me_attention_prefill_columns() // (nh // nkv)
+# Blocks of twice as many query columns read each key and value tile once for twice the work, but a step
+# has half as many of them. They are taken when every compute unit still gets a whole one, or when the step
+# has so many key tiles to walk that tiles are cut into key ranges anyway (measured on 256 compute units:
+# from 4,096 tokens of whole prompts on, or a 2,048-token portion behind 2,048 tokens, 8-24% faster;
+# three prompts of 1,024 tokens, a third slower).
+PREFILL_WIDE_MIN_BLOCKS = 1.0
+PREFILL_WIDE_MIN_KEY_TILES = 20.0  # per compute unit
+
+
+def wide_blocks_pay(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int) -> bool:
+    # not when the wide blocks would be a third emptier than the narrow ones (many items of few tokens)
+    half = max(1, tpb // 2)
+    if 3 * sum(-(-n // tpb) * tpb for n in qlens) > 4 * sum(-(-n // half) * half for n in qlens):
+        return False
+    blocks = key_tiles = 0
+    for start, n in zip(starts, qlens):
+        for t0 in range(0, n, tpb):
+            last = start + min(t0 + tpb, n) - 1
+            first = max(0, start + t0 - window + 1) if window > 0 else 0
+            blocks += 1
+            key_tiles += last // 64 - first // 64 + 1
+    return blocks * nkv >= PREFILL_WIDE_MIN_BLOCKS * slots or key_tiles * nkv >= PREFILL_WIDE_MIN_KEY_TILES * slots
+
+
+def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,
+                       wide: bool | None = None) -> PrefillPlan:
+    group = nh // nkv
     slots = torch.cuda.get_device_properties(device).multi_processor_count
+    if wide is None:
+        wide = wide_blocks_pay(starts, qlens, max(1, lib().me_attention_prefill_columns(1) // group), window, nkv, slots)
+    columns = lib().me_attention_prefill_columns(1 if wide else 0)
+    tpb = columns // group
     work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4)
     parts = [work.reshape(-1), first] + ([token_chunks] if max_chunks > 1 else [])
     both = torch.from_numpy(np.concatenate(parts)).to(device)  # one upload
     a, b = work.size, work.size + first.size
-    return PrefillPlan(both[:a], both[a:b], both[b:] if max_chunks > 1 else None, first.size, max_chunks)
+    return PrefillPlan(both[:a], both[a:b], both[b:] if max_chunks > 1 else None, first.size, max_chunks, columns)
 
 
 def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: list[int], block_table, scale: float,
@@ -757,6 +790,6 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
         _p(q), _p(k_cache), _p(v_cache), _i(items), _p(block_table),
         _i(block_table.shape[1]), _p(out), _p(plan.work), _p(plan.bundle_first), _i(plan.num_bundles), _p(part_o), _p(part_ml),
         _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
-        _stream()))
+        _i(plan.columns), _stream()))
     return out
 

@@ -5,7 +5,7 @@ import random
 
 import numpy as np
 
-from mini_engine_amd.ops.kernels import prefill_work_list
+from mini_engine_amd.ops.kernels import prefill_work_list, wide_blocks_pay
 
 
 def check_plan(starts, qlens, tpb, window, nkv, slots):
@@ -77,3 +77,16 @@ def test_random_steps():
         qlens = [rng.choice([1, 2, 7, 64, 65, 200, 700]) for _ in range(n_items)]
         check_plan(starts, qlens, rng.choice([8, 32, 64, 128]), rng.choice([0, 0, 37, 500]), rng.choice([1, 2, 8]),
                    rng.choice([16, 256]))
+
+
+def test_wide_blocks_are_taken_for_full_steps_and_long_contexts_only():
+    """128 tokens per wide block (a kv group of two heads), 8 kv heads, 256 compute units."""
+    pay = lambda starts, qlens, window=0: wide_blocks_pay(starts, qlens, 128, window, 8, 256)
+    assert not pay([0], [2048])            # 16 blocks per kv head: half the compute units
+    assert pay([0], [4096])                # a whole block for every compute unit
+    assert pay([0] * 32, [256] * 32)       # many short prompts fill the chip as well
+    assert not pay([0] * 3, [1024] * 3)    # neither: few blocks, few keys
+    assert pay([2048], [2048])             # few blocks, but a long walk over the keys for each
+    assert pay([8192] * 2, [512] * 2)
+    assert not pay([0] * 64, [64] * 64)    # wide blocks would be half empty
+    assert not pay([8192] * 2, [512] * 2, window=256)  # a window takes the long walk away
