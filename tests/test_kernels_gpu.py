@@ -86,7 +86,7 @@ def test_gemm_f32(m, n, k):
 
 @pytest.mark.parametrize("m,n,k,gated", [(130, 200, 128, False), (257, 96, 192, True), (2048, 1024, 1024, False),
                                          (77, 50, 64, True), (300, 333, 256, False), (513, 1000, 320, True), (1100, 200, 128, True)])
-@pytest.mark.parametrize("shape", [0, 1, 2, 6, 7, 8, 9])
+@pytest.mark.parametrize("shape", [0, 1, 2, 6, 7, 8, 9, 12])
 def test_gemm_bf16_tiled(m, n, k, gated, shape):
     """The LDS-tiled matrix-core product at sizes that are no multiple of its tiles, against a float32
     product of the same bfloat16 inputs; every block tile shape, plain and with the SwiGLU epilogue."""
