@@ -166,7 +166,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
     float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int bs_shift, int window,
-    float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa) {
+    float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa, const int* __restrict__ live_items,
+    int waves_wanted) {
   const int bs = 1 << bs_shift;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
@@ -188,9 +189,17 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   // to the splits in equal runs of whole tiles: every split has work whatever the item's length is
   // (the grid is sized for the longest context the step may hold, often many times the actual one).
   const int ctx = item_ctx[item];
+  // A launch that was laid out for fewer items than the grid holds (a replayed graph whose last items
+  // are padding) has more splits than this step needs: the live items share `waves_wanted` waves, and
+  // the splits beyond that come out empty.
+  int splits = num_splits;
+  if (live_items) {
+    const int units = max(live_items[0], 1) * (int)gridDim.y;
+    splits = min(num_splits, max(1, (waves_wanted + units - 1) / units));
+  }
   const int lo = window > 0 ? max(ctx - window, 0) : 0;
   const int lo16 = (lo / 16) * 16;
-  const int tiles_per_split = ((ctx - lo16 + 15) / 16 + num_splits - 1) / num_splits;
+  const int tiles_per_split = ((ctx - lo16 + 15) / 16 + splits - 1) / splits;
   const int begin = lo16 + split * tiles_per_split * 16;
   const int end = min(begin + tiles_per_split * 16, ctx);
 
@@ -407,17 +416,16 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
 template <int D>
 static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* item_ctx, const int* table,
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
-                          float scale_log2, int split_keys, int num_splits, const DecodeFusedArgs* fused,
-                          hipStream_t stream) {
+                          float scale_log2, int depth, int num_splits, const DecodeFusedArgs* fused,
+                          const int* live_items, int waves_wanted, hipStream_t stream) {
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits);
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-  const int depth = (split_keys <= 256 || (long long)items * nkv * chunks * num_splits <= 1024) ? 2 : 1;
 #define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                                                                         \
   attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
                                                                     nkv, bs_shift, window, scale_log2, num_splits,    \
-                                                                    chunks, ARGS)
+                                                                    chunks, ARGS, live_items, waves_wanted)
   if constexpr (D % 64 == 0) {
     if (fused) {
       if (depth == 2)
@@ -444,19 +452,24 @@ extern "C" int me_attention_mfma_supported(int d, int bs) {
 // workspace: part_o float [items * nh * num_splits * d], part_ml float [items * nh * num_splits * 2].
 // Every item's keys are dealt to the num_splits splits in equal runs; split_keys (a multiple of 16) says
 // how long a run is at the longest context the step can hold (max_ctx): num_splits * split_keys must
-// cover it, and it decides how many tiles a wave keeps in flight.
+// cover it. live_items (device, or null): how many of the items are live, for a launch whose grid was
+// laid out for fewer items than it holds; then full_splits is the number of splits of a step with every
+// item live and waves_wanted the number of waves that the live items' splits should come to.
 static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
-                         int max_ctx, const DecodeFusedArgs* fused, hipStream_t stream);
+                         int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
+                         int waves_wanted, hipStream_t stream);
 
 extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                                         const int* block_table, int table_width, void* out, float* part_o,
                                         float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
                                         float scale, int split_keys, int num_splits, int max_ctx,
+                                        const int* live_items, int full_splits, int waves_wanted,
                                         hipStream_t stream) {
   return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
-                       bs, window, scale, split_keys, num_splits, max_ctx, nullptr, stream);
+                       bs, window, scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted,
+                       stream);
 }
 
 // Head sizes and groupings for which the decode kernel can take the norm, the rotary encoding and
@@ -474,6 +487,7 @@ extern "C" int me_attention_decode_fused_bf16(const void* qkv, const float* q_w,
                                               const int* block_table, int table_width, void* out, float* part_o,
                                               float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
                                               float scale, int split_keys, int num_splits, int max_ctx,
+                                              const int* live_items, int full_splits, int waves_wanted,
                                               hipStream_t stream) {
   if (nkv <= 0 || nh <= 0 || nh % nkv || !me_attention_decode_fused_supported(d, bs, rope_table ? rotary_dim : 0, nh / nkv))
     return me_fail("me_attention_decode_fused_bf16: head_dim=%d block_size=%d rotary_dim=%d heads=%d/%d not supported", d,
@@ -487,13 +501,14 @@ extern "C" int me_attention_decode_fused_bf16(const void* qkv, const float* q_w,
   fa.k_cache_w = (bf16_t*)k_cache;
   fa.v_cache_w = (bf16_t*)v_cache;
   return decode_common(qkv, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
-                       bs, window, scale, split_keys, num_splits, max_ctx, &fa, stream);
+                       bs, window, scale, split_keys, num_splits, max_ctx, &fa, live_items, full_splits, waves_wanted, stream);
 }
 
 static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
-                         int max_ctx, const DecodeFusedArgs* fused, hipStream_t stream) {
+                         int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
+                         int waves_wanted, hipStream_t stream) {
   if (items <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_decode_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
@@ -504,12 +519,21 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
     return me_fail("me_attention_decode_bf16: block table of %d pages of %d cannot hold %d keys", table_width, bs, max_ctx);
   if (num_splits > ME_MAX_SPLITS) return me_fail("me_attention_decode_bf16: %d splits exceed %d", num_splits, ME_MAX_SPLITS);
   if (num_splits > 65535 || nkv * ((nh / nkv + 15) / 16) > 65535) return me_fail("me_attention_decode_bf16: grid too large");
+  // How many tiles a wave keeps in flight goes by the splits that a step with every item live uses
+  // (full_splits; the grid's num_splits when no count of live items is given).
+  if (live_items && (full_splits <= 0 || full_splits > num_splits || waves_wanted <= 0))
+    return me_fail("me_attention_decode_bf16: %d splits for a full step out of %d, %d waves wanted", full_splits, num_splits,
+                   waves_wanted);
+  const int run_splits = live_items ? full_splits : num_splits;
+  const int run_keys = (((max_ctx + run_splits - 1) / run_splits + 15) / 16) * 16;
+  const long long run_waves = (long long)items * nkv * ((nh / nkv + 15) / 16) * run_splits;
+  const int depth = (run_keys <= 256 || run_waves <= 1024) ? 2 : 1;
   const float sl = scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
 #define ME_DECODE_CASE(DD)                                                                                      \
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
-                      split_keys, num_splits, fused, stream);                                                   \
+                      depth, num_splits, fused, live_items, waves_wanted, stream);                              \
     break;
   switch (d) {
     ME_DECODE_CASE(32)

@@ -31,7 +31,7 @@ class StepItem:
 def section_offsets(t: int, b: int, r: int, widths: list[int]) -> dict[str, tuple[int, int]]:
     off, out = 0, {}
     for name, n in (("token_ids", t), ("positions", t), ("token_item", t), ("want_rows", r),
-                    ("item_start", b + 1), ("item_ctx", b), ("state_slots", b)):
+                    ("item_start", b + 1), ("item_ctx", b), ("state_slots", b), ("live_items", 1)):
         out[name] = (off, n)
         off += n
     for g, w in enumerate(widths):
@@ -59,6 +59,8 @@ class StepBatch:
         self.item_start = view("item_start")
         self.item_ctx = view("item_ctx")
         self.state_slots = view("state_slots")
+        self.live_items = view("live_items")  # how many of the items are requests; the rest is padding
+        self.least_live = b  # the fewest live items a (replayed) batch of this layout will ever hold
         self._tables = [view(f"table{g}").view(b, w) for g, w in enumerate(self.widths)]
         # host-side description, filled by pack(); static graph batches keep the capture-time values
         self.starts: list[int] = []
@@ -118,6 +120,7 @@ def pack_host(items: list[StepItem], num_groups: int, widths: list[int] | None =
             arr[o : o + widths[g]] = spare_block
         cursor += 1
     arr[start_o + b] = cursor
+    arr[sec["live_items"][0]] = len(items)
     return arr, t, b, r, widths
 
 

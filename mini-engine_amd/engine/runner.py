@@ -94,6 +94,8 @@ class ModelRunner:
         batch = StepBatch(buf, bucket, bucket, bucket, widths)
         batch.starts, batch.qlens, batch.slots_host = [0] * bucket, [1] * bucket, [-1] * bucket
         batch.max_ctx = self.config.max_model_len
+        smaller = [b for b in batch_buckets(self.config.max_num_seqs) if b < bucket]
+        batch.least_live = smaller[-1] + 1 if smaller else 1  # fewer items replay a smaller bucket's graph
         stream = torch.cuda.Stream()
         stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream):
@@ -132,6 +134,7 @@ class ModelRunner:
         a[pos_o : pos_o + bucket] = starts + [0] * pad
         a[ctx_o : ctx_o + bucket] = [s + 1 for s in starts] + [1] * pad
         a[slot_o : slot_o + bucket] = [it.seq.state_slot if it.seq.state_slot >= 0 else spare_slot for it in items] + [spare_slot] * pad
+        a[sec["live_items"][0]] = n
         bases = [sec[f"table{g}"][0] for g in range(self.num_groups)]
         windows = [g.window for g in self.layout.groups]
         for i, it in enumerate(items):

@@ -512,19 +512,36 @@ def attention_mfma_supported(head_dim: int, block_size: int, group: int = 1) -> 
 def decode_splits(items: int, kv_units: int, max_ctx: int, target_waves: int = 1024) -> tuple[int, int]:
     """(keys per split, number of splits) for the decode kernel: enough waves to fill the chip,
     splits of at least 64 keys, boundaries at multiples of 64."""
-    want = max(1, target_waves // max(1, items * kv_units))
-    splits = 1
-    while splits * 2 <= want and splits * 2 * 64 <= max(max_ctx, 64):
-        splits *= 2
+    units = max(1, items * kv_units)
+    splits = max(1, min(-(-target_waves // units), max(max_ctx, 64) // 64))
     split_keys = -(-max_ctx // splits)
     split_keys = -(-split_keys // 64) * 64
     return split_keys, -(-max_ctx // split_keys)
 
 
+DECODE_WAVES = 1024  # waves that a decode attention launch aims at (four per compute unit of 256)
+
+
+def _decode_split_plan(items: int, kv_units: int, max_ctx: int, live):
+    """(split_keys, num_splits, live pointer, splits of a full step) for a decode launch. ``live`` is
+    None or ``(count, least)``: a device int32 with the number of live items (the others are padding)
+    and the fewest live items the launch will ever see; the grid is then laid out for ``least`` items,
+    and the kernel takes as many of its splits as the live items need."""
+    _, full = decode_splits(items, kv_units, max_ctx, DECODE_WAVES)
+    if live is None or live[1] >= items:
+        keys, splits = decode_splits(items, kv_units, max_ctx, DECODE_WAVES)
+        return keys, splits, None, splits
+    count, least = live
+    _want(count, "live item count", torch.int32, (1,))
+    keys, splits = decode_splits(max(1, least), kv_units, max_ctx, DECODE_WAVES)
+    return keys, splits, count, min(full, splits)
+
+
 def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: float, window: int, max_ctx: int,
-                          out: torch.Tensor | None = None) -> torch.Tensor:
+                          out: torch.Tensor | None = None, live=None) -> torch.Tensor:
     """Attention of one new token per item over its cached keys: q [items, nh, d] bfloat16,
-    item_ctx int32 [items] (keys per item, the new one included, each <= max_ctx)."""
+    item_ctx int32 [items] (keys per item, the new one included, each <= max_ctx). ``live``: see
+    :func:`_decode_split_plan`."""
     _want(q, "q", torch.bfloat16, (None, None, None))
     items, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -534,7 +551,7 @@ def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: flo
     if block_table.shape[1] * bs < max_ctx:
         raise ValueError(f"block table of {block_table.shape[1]} pages cannot hold {max_ctx} keys")
     chunks = -(-(nh // nkv) // 16)
-    split_keys, num_splits = decode_splits(items, nkv * chunks, max_ctx)
+    split_keys, num_splits, live_count, full_splits = _decode_split_plan(items, nkv * chunks, max_ctx, live)
     part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=q.device)
     if out is None:
@@ -543,7 +560,7 @@ def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: flo
     check(lib().me_attention_decode_bf16(
         _p(q), _p(k_cache), _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out),
         _p(part_o), _p(part_ml), _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys),
-        _i(num_splits), _i(max_ctx), _stream()))
+        _i(num_splits), _i(max_ctx), _p(live_count), _i(full_splits), _i(DECODE_WAVES), _stream()))
     return out
 
 
@@ -554,10 +571,10 @@ def attention_decode_fused_supported(head_dim: int, block_size: int, rotary_dim:
 
 def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write_kv: bool, k_cache, v_cache, item_ctx,
                                 block_table, num_heads: int, scale: float, window: int, max_ctx: int,
-                                out: torch.Tensor | None = None) -> torch.Tensor:
+                                out: torch.Tensor | None = None, live=None) -> torch.Tensor:
     """One new token per item, from the raw q/k/v projection: what :func:`qk_norm_rope_scatter` followed
     by :func:`attention_decode_bf16` compute, in one launch. qkv [items, (nh + 2 nkv) d] bfloat16
-    (or [items, nh d] with ``write_kv`` off)."""
+    (or [items, nh d] with ``write_kv`` off). ``live``: see :func:`_decode_split_plan`."""
     nkv, bs, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     nh = num_heads
     _want(qkv, "qkv", torch.bfloat16, (None, ((nh + 2 * nkv) if write_kv else nh) * d))
@@ -577,7 +594,7 @@ def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write
         if rope.shape[0] < max_ctx:
             raise ValueError(f"the rotary table covers {rope.shape[0]} positions, the step may reach {max_ctx}")
     chunks = -(-(nh // nkv) // 16)
-    split_keys, num_splits = decode_splits(items, nkv * chunks, max_ctx)
+    split_keys, num_splits, live_count, full_splits = _decode_split_plan(items, nkv * chunks, max_ctx, live)
     part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=qkv.device)
     part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=qkv.device)
     if out is None:
@@ -587,7 +604,7 @@ def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write
         _p(qkv), _p(q_weight), _p(k_weight), _p(rope), _i(rd), _f(eps), _i(1 if write_kv else 0), _p(k_cache),
         _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out), _p(part_o), _p(part_ml),
         _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys), _i(num_splits), _i(max_ctx),
-        _stream()))
+        _p(live_count), _i(full_splits), _i(DECODE_WAVES), _stream()))
     return out
 
 

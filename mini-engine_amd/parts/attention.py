@@ -92,7 +92,8 @@ class Attention(Mixer):
             # one new token per item: norm, rotary, page write and attention in one launch
             out = K.attention_decode_fused_bf16(
                 proj, self.q_norm_w, self.k_norm_w if owns else None, rope, eps, owns, b.k_cache, b.v_cache,
-                batch.item_ctx, table, self.nh, float(s.scale), int(s.window), batch.max_ctx)
+                batch.item_ctx, table, self.nh, float(s.scale), int(s.window), batch.max_ctx,
+                live=(batch.live_items, batch.least_live))
             return K.linear(out, self.w_o, as_delta=True)
         q = K.qk_norm_rope_scatter(
             proj, self.q_norm_w, self.k_norm_w if owns else None, rope, batch.positions, batch.token_item,
@@ -110,7 +111,7 @@ class Attention(Mixer):
         if self.dtype is torch.bfloat16 and K.attention_mfma_supported(self.d, b.block_size, self.nh // self.nkv):
             if batch.decode_only:
                 return K.attention_decode_bf16(q, b.k_cache, b.v_cache, batch.item_ctx, table, scale, window,
-                                               batch.max_ctx)
+                                               batch.max_ctx, live=(batch.live_items, batch.least_live))
             key = ("prefill_plan", self.nh, self.nkv, self.d, window)
             plan = batch.derived.get(key)
             if plan is None:  # the same for every layer of this shape: made once per step

@@ -492,6 +492,37 @@ def test_attention_decode_mfma(nh, nkv, d, bs, window):
         torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs", [(16, 8, 128, 16), (4, 2, 64, 16), (6, 1, 96, 32)])
+def test_attention_decode_with_fewer_live_items_than_the_grid_holds(nh, nkv, d, bs):
+    """A launch laid out for as few as `least` live items (a replayed graph: the rest is padding) has
+    more splits than a fuller step needs; the kernel takes as many as the live items call for. Every
+    count of live items from `least` to all gives the same result as a launch without padding."""
+    dtype = torch.bfloat16
+    ctxs = [700, 16, 17, 333, 1000, 255, 64, 65, 1, 1, 1, 1, 130, 1, 1, 1]
+    items = [(c - 1, 1) for c in ctxs]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=260)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(4)
+    qs = [torch.randn(1, nh, d, generator=g).to(dtype) for _ in items]
+    scale = d**-0.5
+    want = dense_reference(qs, ks, vs, items, scale, 0)
+    item_ctx = torch.tensor(ctxs, dtype=torch.int32)
+    max_ctx = 4096
+    wide = torch.zeros(len(items), max_ctx // bs, dtype=torch.int32)
+    wide[:, : table_t.shape[1]] = table_t
+    args = (dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide), scale, 0, max_ctx)
+    plain_out = K().attention_decode_bf16(*args)
+    torch.testing.assert_close(plain_out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    least = 9
+    chunks = -(-(nh // nkv) // 16)
+    grid_splits, full_splits = (K().decode_splits(n, nkv * chunks, max_ctx)[1] for n in (least, len(items)))
+    assert grid_splits >= full_splits and (grid_splits > full_splits or nkv < 8)
+    for live in (9, 12, 16):
+        count = dev(torch.tensor([live], dtype=torch.int32))
+        out = K().attention_decode_bf16(*args, live=(count, least))
+        torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
 def test_attention_decode_many_splits():
     """A long context of one item is cut into more splits than a wave has lanes; a far key is made to
     dominate so that a split that is dropped or weighted wrongly shows."""
