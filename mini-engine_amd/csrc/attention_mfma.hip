@@ -362,6 +362,20 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
   const size_t unit = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & (ME_WAVE - 1), wave = tid / ME_WAVE;
   const float* ml = part_ml + unit * num_splits * 2;
+  // the first partial results of this thread are requested before the weights are known: their loads
+  // and those of the statistics are in flight together
+  constexpr int EARLY = 8;
+  const int quads = d / 4;          // d is a multiple of 32, so quads <= 64
+  const int groups = 256 / quads;   // groups of splits handled side by side
+  const int qd = tid % quads, grp = tid / quads;
+  const float* po = part_o + unit * num_splits * d + qd * 4;
+  float4_t early[EARLY];
+#pragma unroll
+  for (int i = 0; i < EARLY; ++i) {
+    const int sp = grp + i * groups;
+    early[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    if (grp < groups && sp < num_splits) early[i] = *reinterpret_cast<const float4_t*>(po + (size_t)sp * d);
+  }
   float big = -INFINITY;
   for (int s = tid; s < num_splits; s += 256)
     if (ml[s * 2 + 1] > 0.f) big = fmaxf(big, ml[s * 2]);
@@ -381,13 +395,18 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
   __syncthreads();
   const float denom = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]);
 
-  const int quads = d / 4;          // d is a multiple of 32, so quads <= 64
-  const int groups = 256 / quads;   // groups of splits handled side by side
-  const int qd = tid % quads, grp = tid / quads;
   float4_t accv = {0.f, 0.f, 0.f, 0.f};
   if (grp < groups) {
-    const float* po = part_o + unit * num_splits * d + qd * 4;
-    for (int s = grp; s < num_splits; s += groups) {
+#pragma unroll
+    for (int i = 0; i < EARLY; ++i) {
+      const int sp = grp + i * groups;
+      const float w = sp < num_splits ? wgt[sp] : 0.f;
+      accv[0] += w * early[i][0];
+      accv[1] += w * early[i][1];
+      accv[2] += w * early[i][2];
+      accv[3] += w * early[i][3];
+    }
+    for (int s = grp + EARLY * groups; s < num_splits; s += groups) {
       const float w = wgt[s];
       const float4_t v = *reinterpret_cast<const float4_t*>(po + (size_t)s * d);
       accv[0] += w * v[0];
