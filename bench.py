@@ -170,7 +170,7 @@ def main() -> int:
     if max_batch >= 64 and not args.zero_context:
         pts["throughput_64x256in_128out"] = round(reference_workload(), 1)
     line = {
-        "metric": "decode tok/s at batch 8 (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights"
