@@ -166,7 +166,10 @@ def main() -> int:
         return sum(len(o) for o in outs) / (time.perf_counter() - t0)
 
     tok_s, ms_per_step, gbs = decode(args.batch)
-    pts = {f"decode_b{b}": round(decode(b)[0], 1) for b in points}
+    measured = {b: decode(b) for b in points}
+    pts = {f"decode_b{b}": round(m[0], 1) for b, m in measured.items()}
+    # the same bound as `roofline`, for the other batch sizes: bytes a step must read / its time / the HBM peak
+    pts_frac = {f"decode_b{b}": round(m[2] / HBM_PEAK_GBS, 4) for b, m in measured.items()}
     if max_batch >= 64 and not args.zero_context:
         pts["throughput_64x256in_128out"] = round(reference_workload(), 1)
     line = {
@@ -184,6 +187,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4)},
         "points": pts,
+        "points_roofline_frac": pts_frac,
     }
     print(json.dumps(line))
     return 0
