@@ -28,6 +28,9 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+# The GEMM library that plain products of prompts go to (csrc/gemm_library.hip calls it directly).
+ROCM_LIB = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
+LINK_LIBS = [f"-L{ROCM_LIB}", f"-Wl,-rpath,{ROCM_LIB}", "-lhipblaslt"]
 
 
 def sources() -> list[str]:
@@ -92,7 +95,7 @@ def build(out_dir: str | None = None, quiet: bool = False, jobs: int | None = No
             _say(f"  {os.path.basename(futures[fut])} done ({len(objs)}/{len(srcs)}, {time.time() - t0:.0f}s)", quiet)
     lib = os.path.join(out_dir, LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
-    r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *sorted(objs)],
+    r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *sorted(objs), *LINK_LIBS],
                        capture_output=True, text=True, env=env)
     if r.returncode != 0:
         raise RuntimeError(f"linking {LIB_NAME} failed:\n{r.stderr[-4000:]}")

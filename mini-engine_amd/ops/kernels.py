@@ -18,7 +18,7 @@ from .library import check, lib
 
 _F32, _BF16 = 0, 1
 _vp = ctypes.c_void_p
-_i = ctypes.c_int
+_i = int  # a Python int goes to a C int as it is; wrapping it in a ctypes object only costs time
 _f = ctypes.c_float
 
 
@@ -53,7 +53,7 @@ def _want(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: t
         raise ValueError(f"{name} must be a contiguous tensor on the GPU")
     if dtype is not None and t.dtype is not dtype:
         raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
-    if shape is not None:
+    if shape is not None and t.shape != shape:  # equal tuples: the usual case, one comparison
         got = t.shape
         ok = len(got) == len(shape)
         if ok:
@@ -463,17 +463,40 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         if tiled_ok(x, weight) and out_dtype is torch.bfloat16:
             return gemm_bf16_tiled(x, weight, out_dtype, True)  # measured ahead of the library product + SwiGLU kernel
         return swiglu(linear(x, weight, out_dtype))
+    return gemm_bf16_library(x, weight, out_dtype)
+
+
+_LIBRARY_REFUSED: set = set()  # (N, K, output type) of products the direct library call has no algorithm for
+
+
+def gemm_bf16_library(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                      out: torch.Tensor | None = None) -> torch.Tensor:
+    """bfloat16 ``x @ weight.T`` through the GEMM library with float32 accumulation, as bfloat16 or as
+    float32 (logits, not rounded to bfloat16). The library is called directly (a third of the host time
+    of a call through torch); where it has no algorithm for the sizes (widths that are no multiple of
+    8), torch's product stands in, and for float32 results slices of 64 rows through the matrix-core kernel."""
+    _want(x, "x", torch.bfloat16, (None, None))
+    m, k = x.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _want(out, "out", out_dtype, (m, n))
+    shape_class = (n, k, out_dtype)
+    if shape_class not in _LIBRARY_REFUSED:
+        if lib().me_gemm_bf16_library(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(_code(out_dtype)), _stream()) == 0:
+            return out
+        _LIBRARY_REFUSED.add(shape_class)
     if out_dtype is torch.float32:
         try:
-            return torch.mm(x, weight.t(), out_dtype=torch.float32)  # float32 logits, not rounded to bfloat16
+            return torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
         except (TypeError, RuntimeError):
-            if x.shape[1] % 8 == 0:  # slices of 64 rows through the matrix-core kernel
-                out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
-                for lo in range(0, x.shape[0], SMALL_MAX_ROWS):
-                    gemm_bf16_small(x[lo:lo + SMALL_MAX_ROWS], weight, torch.float32, False, out[lo:lo + SMALL_MAX_ROWS])
-                return out
-    y = torch.matmul(x, weight.t())
-    return y if out_dtype is y.dtype else y.to(out_dtype)
+            if k % 8:
+                raise
+            for lo in range(0, m, SMALL_MAX_ROWS):
+                gemm_bf16_small(x[lo:lo + SMALL_MAX_ROWS], weight, torch.float32, False, out[lo:lo + SMALL_MAX_ROWS])
+            return out
+    return torch.matmul(x, weight.t(), out=out)
 
 
 # -------------------------------------------------------------------------------------- sampling

@@ -108,6 +108,34 @@ def test_gemm_bf16_tiled(m, n, k, gated, shape):
         K().gemm_bf16_tiled(dev(x[:, : k - 8].contiguous()), dev(w[:, : k - 8].contiguous()), torch.bfloat16, gated)
 
 
+@pytest.mark.parametrize("m,n,k", [(130, 200, 128), (2048, 1024, 1024), (70, 50, 72), (300, 333, 75), (65, 1001, 40), (1, 64, 64)])
+def test_gemm_bf16_library(m, n, k):
+    """Plain products through the GEMM library, called directly where it has an algorithm for the sizes
+    and through torch where not (odd widths), as bfloat16 and as float32, also replayed from a graph."""
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    want = x.float() @ w.float().T
+    scale = max(1.0, want.abs().max().item())
+    xd, wd = dev(x), dev(w)
+    for out_dtype in (torch.bfloat16, torch.float32):
+        got = K().gemm_bf16_library(xd, wd, out_dtype)
+        assert got.dtype is out_dtype
+        tol_abs = (2**-7 if out_dtype is torch.bfloat16 else 1e-4) * scale
+        assert (got.float().cpu() - want).abs().max().item() <= tol_abs, (out_dtype, (got.float().cpu() - want).abs().max().item(), scale)
+    out = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        K().gemm_bf16_library(xd, wd, torch.bfloat16, out=out)
+    for _ in range(2):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert (out.float().cpu() - want).abs().max().item() <= 2**-7 * scale
+
+
 @pytest.mark.parametrize("m,n,k,splits", [(17, 1024, 2048, 4), (64, 1000, 3072, 4), (33, 48, 520, 2), (40, 16, 4096, 8)])
 def test_small_gemm_partial_sums_and_their_add_rmsnorm(m, n, k, splits):
     """A product of 17 to 64 rows cut into runs of k: the parts add up to the product, and add_rmsnorm
