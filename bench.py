@@ -152,18 +152,37 @@ def main() -> int:
         step_bytes = weight_bytes + (tokens_before + tokens_after) / 2 * kv_per_token
         return (tokens_after - tokens_before) / dt, ms, step_bytes / (dt / k) / 1e9
 
-    def reference_workload():
-        """The reference's own throughput workload (benchmarks/bench.py:52-62, :113-123): 64 requests of
-        256 random prompt ids and 128 greedy output tokens, all submitted at once; output tokens over
-        the wall time of the whole run, prefill and scheduling included."""
+    def reference_workloads():
+        """The reference's own two serving workloads, with its engine options (benchmarks/bench.py:52-62,
+        :86-93, :113-123: pages of 16, 2,048 pages, 64 sequences, 8,192 tokens a step, prefix cache on).
+        Throughput: 64 requests of 256 random prompt ids and 128 greedy output tokens, all submitted at
+        once. Shared prefix: 64 requests of a common 512-token prefix and 32 tokens of their own, 64
+        output tokens, the first request run alone so that the others find its pages. Output tokens
+        over the wall time of the whole run, prefill and scheduling included."""
+        ref = LLMEngine.from_random("Qwen3ForCausalLM", cfg, EngineConfig(
+            block_size=16, num_blocks=2048, max_num_seqs=64, max_num_batched_tokens=8192, max_model_len=2048,
+            enable_prefix_caching=True, dtype=args.dtype, seed=0, cuda_graphs=True), seed=0)
+        ref.runner.capture_all()
+
+        def timed(run):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = run()
+            torch.cuda.synchronize()
+            return sum(len(o) for o in outs) / (time.perf_counter() - t0)
+
         params = SamplingParams(max_tokens=128, temperature=0.0, ignore_eos=True)
+        ref.generate([prompt(256) for _ in range(2)], params)  # code objects, the GEMM library's plans
         prompts = [prompt(256) for _ in range(64)]
-        engine.generate([prompt(256) for _ in range(2)], params)  # graphs of the smaller buckets, code objects
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        outs = engine.generate(prompts, params)
-        torch.cuda.synchronize()
-        return sum(len(o) for o in outs) / (time.perf_counter() - t0)
+        throughput = timed(lambda: ref.generate(prompts, params))
+        ref.block_manager.reset_prefix_cache()
+        shared = prompt(512)
+        prompts = [shared + prompt(32) for _ in range(64)]
+        params = SamplingParams(max_tokens=64, temperature=0.0, ignore_eos=True)
+        cached_before = ref.scheduler.num_cached_tokens
+        prefix = timed(lambda: ref.generate(prompts[:1], params) + ref.generate(prompts[1:], params))
+        assert ref.scheduler.num_cached_tokens - cached_before == 63 * 512, "the shared prefix was not served from the cache"
+        return throughput, prefix
 
     tok_s, ms_per_step, gbs = decode(args.batch)
     measured = {b: decode(b) for b in points}
@@ -171,7 +190,9 @@ def main() -> int:
     # the same bound as `roofline`, for the other batch sizes: bytes a step must read / its time / the HBM peak
     pts_frac = {f"decode_b{b}": round(m[2] / HBM_PEAK_GBS, 4) for b, m in measured.items()}
     if max_batch >= 64 and not args.zero_context:
-        pts["throughput_64x256in_128out"] = round(reference_workload(), 1)
+        throughput, prefix = reference_workloads()
+        pts["throughput_64x256in_128out"] = round(throughput, 1)
+        pts["shared_prefix_64x544in_64out"] = round(prefix, 1)
     line = {
         "metric": f"decode tok/s at batch {args.batch} (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,

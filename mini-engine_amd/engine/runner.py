@@ -110,6 +110,7 @@ class ModelRunner:
         self._graphs[bucket] = (graph, batch, host, logits)
         return self._graphs[bucket]
 
+    @torch.inference_mode()
     def capture_all(self) -> None:
         """Capture every bucket, largest first so that smaller graphs fit into its memory pool."""
         for b in reversed(batch_buckets(self.config.max_num_seqs)):
