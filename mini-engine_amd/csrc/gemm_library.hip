@@ -69,6 +69,8 @@ extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M
   if (K <= 0) return me_fail("me_gemm_bf16_library: K=%d", K);
   if (!X || !W || !C) return me_fail("me_gemm_bf16_library: null operand");
   if (out_dtype != ME_BF16 && out_dtype != ME_F32) return me_fail("me_gemm_bf16_library: unknown output type %d", out_dtype);
+  if ((uint32_t)M >= (1u << 21) || (uint32_t)N >= (1u << 21) || (uint32_t)K >= (1u << 21))  // the plans' key packs 21 bits each
+    return me_fail("me_gemm_bf16_library: sizes %d x %d x %d are beyond 2^21", M, N, K);
   LibraryPlan plan;
   {
     std::lock_guard<std::mutex> lock(g_mutex);
@@ -86,8 +88,6 @@ extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M
     const uint64_t key = ((uint64_t)(uint32_t)M << 42) ^ ((uint64_t)(uint32_t)N << 21) ^ (uint64_t)(uint32_t)K;
     auto it = plans.find(key);
     if (it == plans.end()) {
-      if ((uint32_t)M >= (1u << 21) || (uint32_t)N >= (1u << 21) || (uint32_t)K >= (1u << 21))
-        return me_fail("me_gemm_bf16_library: sizes %d x %d x %d are beyond 2^21", M, N, K);
       LibraryPlan fresh;
       if (make_plan(fresh, M, N, K, out_dtype)) return 1;
       it = plans.emplace(key, fresh).first;
