@@ -161,19 +161,27 @@ struct DecodeFusedArgs {
 
 #define LONG_RUN 16  // tiles of a split from which on a wave fetches one tile at a time
 
+// Most splits that one block takes on, a wave each. Heads beyond 128 need more than 256 registers a lane
+// with two tiles in flight, which only blocks of at most four waves (one per SIMD) may have.
+#define DECODE_BLOCK_WAVES(D) ((D) <= 128 ? 8 : 4)
+
 template <int D, bool FUSED, int DEPTH>
-__global__ __launch_bounds__(64) void attention_decode_kernel(
+__global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int bs_shift, int window,
-    float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa, const int* __restrict__ live_items,
-    int waves_wanted) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
+    int window, float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa,
+    const int* __restrict__ live_items, int waves_wanted) {
+  extern __shared__ float decode_lds[];  // only with several waves a block: their results, to be added up
   const int bs = 1 << bs_shift;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
-  const int split = blockIdx.z;
+  // the wave's number as a scalar: everything that follows from it (the split, its keys, the loop over them)
+  // stays uniform for the compiler
+  const int block_waves = blockDim.x / ME_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / ME_WAVE);
+  const int split = blockIdx.z * block_waves + wave;  // num_splits = gridDim.z * block_waves
   const int group = nh / nkv;
-  const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+  const int lane = threadIdx.x & (ME_WAVE - 1), r = lane & 15, g = lane >> 4;
   const int heads_here = min(16, group - chunk * 16);
   const int head0 = kvh * group + chunk * 16;
   const int* table = block_table + (size_t)item * table_width;
@@ -335,16 +343,67 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
       }
     }
   }
-  if (r < heads_here) {
-    const size_t slot = ((size_t)item * nh + head0 + r) * num_splits + split;
-    if (g == 0) {
-      part_ml[slot * 2] = m[0];
-      part_ml[slot * 2 + 1] = lsum[0];
+  if (block_waves == 1) {
+    if (r < heads_here) {
+      const size_t slot = ((size_t)item * nh + head0 + r) * num_splits + split;
+      if (g == 0) {
+        part_ml[slot * 2] = m[0];
+        part_ml[slot * 2 + 1] = lsum[0];
+      }
+      float* po = part_o + slot * D;
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt)
+        *reinterpret_cast<float4_t*>(po + dt * 16 + g * 4) = acc[0][dt];
     }
-    float* po = part_o + slot * D;
+    return;
+  }
+  // Several waves a block, each with a split of its own: their results meet in LDS and are added up
+  // here, with the weights 2^(m_w - M). A block that holds all splits of its heads (gridDim.z == 1)
+  // writes the finished output; else one partial result for the block, as a single wave would.
+  float* lds_o = decode_lds;                                        // [waves][heads_here][D]
+  float* lds_ml = decode_lds + (size_t)block_waves * heads_here * D;  // [waves][heads_here][2]
+  if (r < heads_here) {
+    float* po = lds_o + ((size_t)wave * heads_here + r) * D;
 #pragma unroll
     for (int dt = 0; dt < D / 16; ++dt)
       *reinterpret_cast<float4_t*>(po + dt * 16 + g * 4) = acc[0][dt];
+    if (g == 0) {
+      lds_ml[(wave * heads_here + r) * 2] = m[0];
+      lds_ml[(wave * heads_here + r) * 2 + 1] = lsum[0];
+    }
+  }
+  __syncthreads();
+  const int blocks_z = gridDim.z;
+  for (int idx = threadIdx.x; idx < heads_here * (D / 4); idx += blockDim.x) {
+    const int hr = idx / (D / 4), quad = idx % (D / 4);
+    float big = -INFINITY;
+    for (int w = 0; w < block_waves; ++w)
+      if (lds_ml[(w * heads_here + hr) * 2 + 1] > 0.f) big = fmaxf(big, lds_ml[(w * heads_here + hr) * 2]);
+    float denom = 0.f;
+    float4_t total = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < block_waves; ++w) {
+      const float l = lds_ml[(w * heads_here + hr) * 2 + 1];
+      const float wgt = l > 0.f ? fast_exp2(lds_ml[(w * heads_here + hr) * 2] - big) : 0.f;  // an empty split has no weight
+      denom += wgt * l;
+      const float4_t v = *reinterpret_cast<const float4_t*>(lds_o + ((size_t)w * heads_here + hr) * D + quad * 4);
+      total[0] += wgt * v[0];
+      total[1] += wgt * v[1];
+      total[2] += wgt * v[2];
+      total[3] += wgt * v[3];
+    }
+    const size_t head = (size_t)item * nh + head0 + hr;
+    if (blocks_z == 1) {
+      const float inv = 1.f / denom;
+      *reinterpret_cast<short4_t*>(out + head * D + quad * 4) =
+          pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
+    } else {
+      const size_t slot = head * blocks_z + blockIdx.z;
+      *reinterpret_cast<float4_t*>(part_o + slot * D + quad * 4) = total;
+      if (quad == 0) {
+        part_ml[slot * 2] = big;
+        part_ml[slot * 2 + 1] = denom;
+      }
+    }
   }
 }
 
@@ -435,16 +494,18 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
 template <int D>
 static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* item_ctx, const int* table,
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
-                          float scale_log2, int depth, int num_splits, const DecodeFusedArgs* fused,
-                          const int* live_items, int waves_wanted, hipStream_t stream) {
+                          float scale_log2, int depth, int num_splits, int block_waves, bf16_t* out,
+                          const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, hipStream_t stream) {
   const int chunks = (nh / nkv + 15) / 16;
-  dim3 grid(items, nkv * chunks, num_splits);
+  dim3 grid(items, nkv * chunks, num_splits / block_waves);  // num_splits is a multiple of block_waves
+  const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
+  const size_t lds = block_waves > 1 ? (size_t)block_waves * heads_most * (D + 2) * sizeof(float) : 0;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
 #define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                                                                         \
-  attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64, 0, stream>>>(q, kc, vc, item_ctx, table, width, part_o, part_ml, nh, \
-                                                                    nkv, bs_shift, window, scale_log2, num_splits,    \
-                                                                    chunks, ARGS, live_items, waves_wanted)
+  attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64 * block_waves, lds, stream>>>(                                       \
+      q, kc, vc, item_ctx, table, width, part_o, part_ml, out, nh, nkv, bs_shift, window, scale_log2, num_splits, chunks,  \
+      ARGS, live_items, waves_wanted)
   if constexpr (D % 64 == 0) {
     if (fused) {
       if (depth == 2)
@@ -547,12 +608,17 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   const int run_keys = (((max_ctx + run_splits - 1) / run_splits + 15) / 16) * 16;
   const long long run_waves = (long long)items * nkv * ((nh / nkv + 15) / 16) * run_splits;
   const int depth = (run_keys <= 256 || run_waves <= 1024) ? 2 : 1;
+  // Few splits (a step of many items): one block takes all splits of its heads, a wave each, adds their
+  // results up itself and writes the output; the second kernel is not needed then.
+  int block_waves = (num_splits > 1 && num_splits <= DECODE_BLOCK_WAVES(d)) ? num_splits : 1;
+  const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
+  if ((size_t)block_waves * heads_most * (d + 2) * sizeof(float) > 48 * 1024) block_waves = 1;  // LDS for the sum
   const float sl = scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
 #define ME_DECODE_CASE(DD)                                                                                      \
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
-                      depth, num_splits, fused, live_items, waves_wanted, stream);                              \
+                      depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, stream);   \
     break;
   switch (d) {
     ME_DECODE_CASE(32)
@@ -564,6 +630,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   }
 #undef ME_DECODE_CASE
   if (me_check_launch("me_attention_decode_bf16")) return 1;
+  if (block_waves > 1) return 0;  // the blocks held all splits of their heads and wrote the output themselves
   attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d);
   return me_check_launch("me_attention_decode_combine");
 }

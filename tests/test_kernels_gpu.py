@@ -551,6 +551,38 @@ def test_attention_decode_with_fewer_live_items_than_the_grid_holds(nh, nkv, d, 
         torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs", [(16, 8, 128, 16), (4, 2, 64, 16), (6, 1, 96, 32), (8, 8, 256, 16), (32, 2, 64, 16)])
+@pytest.mark.parametrize("window", [0, 100])
+def test_attention_decode_with_few_splits_in_one_block(nh, nkv, d, bs, window):
+    """Steps of many items have few splits per item: one block then takes all splits of its heads, a wave
+    each, and writes the finished output (no second kernel). Items of very different lengths, among them
+    some shorter than the number of splits, with and without the norm / rotary / page-write prologue."""
+    dtype = torch.bfloat16
+    ctxs = [500, 16, 17, 333, 450, 255, 64, 65, 1, 2, 3, 40] * 3
+    items = [(c - 1, 1) for c in ctxs]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=700)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(6)
+    qs = [torch.randn(1, nh, d, generator=g).to(dtype) for _ in items]
+    scale = d**-0.5
+    want = dense_reference(qs, ks, vs, items, scale, window)
+    item_ctx = torch.tensor(ctxs, dtype=torch.int32)
+    max_ctx = 512
+    chunks = -(-(nh // nkv) // 16)
+    splits = K().decode_splits(len(items), nkv * chunks, max_ctx)[1]
+    assert 1 < splits <= (8 if d <= 128 else 4), splits  # few enough for one block
+    wide = torch.zeros(len(items), max_ctx // bs, dtype=torch.int32)
+    wide[:, : table_t.shape[1]] = table_t
+    out = K().attention_decode_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide), scale,
+                                    window, max_ctx)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    # padding behind the live items: fewer live items, more of the block's waves at work
+    count = dev(torch.tensor([len(items) - 7], dtype=torch.int32))
+    out = K().attention_decode_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide), scale,
+                                    window, max_ctx, live=(count, len(items) - 10))
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
 def test_attention_decode_many_splits():
     """A long context of one item is cut into more splits than a wave has lanes; a far key is made to
     dominate so that a split that is dropped or weighted wrongly shows."""
