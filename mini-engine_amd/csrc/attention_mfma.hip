@@ -393,7 +393,7 @@ __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_k
     }
     const size_t head = (size_t)item * nh + head0 + hr;
     if (blocks_z == 1) {
-      const float inv = 1.f / denom;
+      const float inv = denom > 0.f ? 1.f / denom : 0.f;  // no visible key at all: zeros, not NaN
       *reinterpret_cast<short4_t*>(out + head * D + quad * 4) =
           pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
     } else {
