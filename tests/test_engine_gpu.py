@@ -136,6 +136,41 @@ def test_long_decoding(peaked, graphs):
     assert (eng.runner.graph_replays > 250) == graphs
 
 
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_random_workload_is_the_same_replayed_and_eager(peaked, name):
+    """Sixty requests of random lengths, some with a common prefix, through so few pages that requests
+    are preempted and re-admitted, eight at a time: the float32 outputs of an engine that replays its
+    decode steps from graphs (index buffer refilled in place, block-table rows extended or rewritten as
+    sequences come, go and come back) equal those of an engine that runs every step eagerly, token by
+    token, and every page is back in its pool at the end."""
+    import random
+
+    from mini_engine_amd import SamplingParams
+
+    folder, pcfg, _ = peaked[name]
+    rng = random.Random(5)
+    shared = [rng.randrange(1, pcfg.vocab_size) for _ in range(48)]
+    work = []
+    for _ in range(60):
+        p = [rng.randrange(1, pcfg.vocab_size) for _ in range(rng.choice([1, 2, 5, 17, 33, 64, 100]))]
+        if rng.random() < 0.4:
+            p = shared[: rng.choice([16, 32, 48])] + p
+        work.append((p, rng.choice([1, 3, 8, 20, 45])))
+    outs = {}
+    for graphs in (True, False):
+        eng = engine(folder, name, block_size=16, num_blocks=24, max_num_seqs=8, max_num_batched_tokens=96,
+                     max_model_len=256, cuda_graphs=graphs)
+        seqs = [eng.add_request(p, SamplingParams(max_tokens=m, temperature=0.0, ignore_eos=True)) for p, m in work]
+        while eng.scheduler.has_unfinished():
+            eng.step()
+        outs[graphs] = [s.output_token_ids for s in seqs]
+        assert all(len(o) == m for o, (_, m) in zip(outs[graphs], work))
+        assert eng.scheduler.num_preemptions > 0 and eng.scheduler.num_cached_tokens > 0
+        assert (eng.runner.graph_replays > 50) == graphs
+        assert all(len(pool.free_pool) == pool.num_blocks for pool in eng.block_manager.pools)
+    assert outs[True] == outs[False]
+
+
 def test_bfloat16_generation_stays_close(peaked):
     """bfloat16 cannot promise equal tokens (near-ties flip, reference DECISIONS.md:80-82): the first
     tokens agree, and each engine token is one the plain logits rank near the top."""
