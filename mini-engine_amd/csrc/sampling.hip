@@ -109,3 +109,54 @@ extern "C" int me_sample(const float* logits, int num_rows, int vocab, const flo
   sample_stage2_kernel<<<num_rows, 64, 0, stream>>>((const Best*)workspace, chunks, out);
   return me_check_launch("me_sample stage 2");
 }
+
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// me_sample_static: me_sample without a workspace argument. The (value, index) pairs that stage 1
+// hands to stage 2 live in a file-scope device array instead of memory the caller allocates. See
+// no_alloc.h for who this is for and what it asks of the caller.
+#include "no_alloc.h"
+
+#include <mutex>
+
+static __device__ __align__(256) unsigned char scratch[ME_SAMPLE_STATIC_SCRATCH_BYTES];
+
+#define ME_MAX_DEVICES 64
+static void* g_scratch_ptr[ME_MAX_DEVICES];  // this library's copy of `scratch` on each device, once looked up
+static std::mutex g_scratch_mutex;
+
+// The device address of `scratch` on the current device. In host code the array's name is only a
+// handle for this lookup; kernels and copies get the address it returns.
+static int static_scratch(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return me_fail("me_sample_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= ME_MAX_DEVICES) return me_fail("me_sample_static: device %d is beyond %d", dev, ME_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return me_fail("me_sample_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int me_sample_static_max_pairs() { return ME_SAMPLE_STATIC_SCRATCH_BYTES / (int)sizeof(Best); }
+
+extern "C" int me_sample_static(const float* logits, int num_rows, int vocab, const float* temperatures,
+                                const uint64_t* keys, int* out, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  if (vocab <= 0) return me_fail("me_sample_static: vocab=%d", vocab);
+  const int chunks = me_sample_chunks(vocab);
+  if ((long long)num_rows * chunks > me_sample_static_max_pairs())
+    return me_fail("me_sample_static: %d rows of %d vocabulary slices need %lld pairs of scratch, the static "
+                   "buffer holds %d (use me_sample with a workspace of your own)",
+                   num_rows, chunks, (long long)num_rows * chunks, me_sample_static_max_pairs());
+  void* ws = nullptr;
+  if (static_scratch(&ws)) return 1;
+  // Stage 1 writes every pair that stage 2 reads (rows x chunks of them), so what the last call left
+  // in the buffer needs no clearing.
+  return me_sample(logits, num_rows, vocab, temperatures, keys, out, ws, stream);
+}
