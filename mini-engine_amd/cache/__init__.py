@@ -1,3 +1,3 @@
-from .block_manager import ROOT_HASH, BlockManager, GroupSpec, PagePool, StateSlots, hash_block
+from .block_manager import ROOT_HASH, BlockManager, GroupSpec, PoolView, SlotsView, hash_block
 
-__all__ = ["ROOT_HASH", "BlockManager", "GroupSpec", "PagePool", "StateSlots", "hash_block"]
+__all__ = ["ROOT_HASH", "BlockManager", "GroupSpec", "PoolView", "SlotsView", "hash_block"]

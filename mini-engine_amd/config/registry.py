@@ -1,8 +1,9 @@
 """One registry from an architecture's name to the functions that describe it.
 
 The name is ``config.json``'s ``architectures[0]``. When that key is absent the ``model_type`` key
-is looked up instead (the reference keys on ``model_type`` and takes ``qwen3`` when it is absent too,
-``src/mini_engine/model.py:37``).
+is looked up among the model types that the registered entries claim (the reference keys on
+``model_type``, ``src/mini_engine/model.py:37``); an entry may also claim configs that name neither
+(``default_for_unnamed``, as the reference takes a config without ``model_type`` for its one model).
 """
 
 from __future__ import annotations
@@ -22,17 +23,20 @@ class ArchitectureEntry:
     config_from_folder: Callable[[str], Any]
     plan_from_config: Callable[[Any], ModelPlan]
     model_types: tuple[str, ...] = field(default_factory=tuple)
+    default_for_unnamed: bool = False  # takes a config.json that names neither architectures nor model_type
 
 
 _ARCHITECTURES: dict[str, ArchitectureEntry] = {}
-_DEFAULT_MODEL_TYPE = "qwen3"
-_MODEL_TYPE_TO_NAME = {"qwen3": "Qwen3ForCausalLM"}
+_MODEL_TYPE_TO_NAME: dict[str, str] = {}
+_UNNAMED: list[str] = []
 
 
 def register_architecture(entry: ArchitectureEntry) -> None:
     _ARCHITECTURES[entry.name] = entry
     for t in entry.model_types:
         _MODEL_TYPE_TO_NAME[t] = entry.name
+    if entry.default_for_unnamed and entry.name not in _UNNAMED:
+        _UNNAMED.append(entry.name)
 
 
 def architecture_names() -> list[str]:
@@ -51,7 +55,11 @@ def architecture_name_of(cfg: dict[str, Any]) -> str:
     archs = cfg.get("architectures")
     if archs:
         return str(archs[0])
-    model_type = cfg.get("model_type", _DEFAULT_MODEL_TYPE)
+    model_type = cfg.get("model_type")
+    if model_type is None:
+        if len(_UNNAMED) != 1:
+            raise ValueError("config.json names neither an architecture nor a model_type")
+        return _UNNAMED[0]
     if model_type not in _MODEL_TYPE_TO_NAME:
         raise ValueError(f"config.json names no architecture and model_type={model_type!r} is unknown")
     return _MODEL_TYPE_TO_NAME[model_type]

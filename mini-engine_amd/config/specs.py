@@ -60,6 +60,11 @@ class AttentionSpec:
     cache_from: int | None = None
     kind: str = "attention"
 
+    @property
+    def kv_elements_per_token(self) -> int:
+        """Key and value elements one token occupies in this layer's own pages (none when it reads another's)."""
+        return 0 if self.cache_from is not None else 2 * self.num_kv_heads * self.head_dim
+
 
 @dataclass(frozen=True)
 class GatedMlpSpec:

@@ -1,6 +1,7 @@
-"""Compile the HIP sources of this folder into one shared library for gfx950.
+"""Compile the HIP sources of this folder and the C++ sources of ``host/`` into one shared library.
 
-``build()`` compiles every ``*.hip`` file with ``hipcc`` (objects in parallel, then one link) and
+``build()`` compiles every ``*.hip`` file for gfx950 and every ``host/*.cpp`` file (plain C++: requests,
+page pools, scheduler, step packing) with ``hipcc`` (objects in parallel, then one link) and
 returns the path of ``libmini_engine_hip.so``. It prints a line per finished object, so a caller
 that waits for a first-time build sees progress. No GPU is needed to compile.
 """
@@ -33,8 +34,11 @@ ROCM_LIB = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
 LINK_LIBS = [f"-L{ROCM_LIB}", f"-Wl,-rpath,{ROCM_LIB}", "-lhipblaslt"]
 
 
+HOST_FLAGS = ["-x", "c++", "-O2", "-std=c++17", "-fPIC", "-Wall"]
+
+
 def sources() -> list[str]:
-    return sorted(glob.glob(os.path.join(HERE, "*.hip")))
+    return sorted(glob.glob(os.path.join(HERE, "*.hip"))) + sorted(glob.glob(os.path.join(HERE, "host", "*.cpp")))
 
 
 def default_lib_path() -> str:
@@ -52,7 +56,7 @@ def is_current(lib_path: str) -> bool:
     if not os.path.exists(lib_path):
         return False
     t = os.path.getmtime(lib_path)
-    deps = sources() + glob.glob(os.path.join(HERE, "*.h"))
+    deps = sources() + glob.glob(os.path.join(HERE, "*.h")) + glob.glob(os.path.join(HERE, "host", "*.h"))
     return all(os.path.getmtime(s) <= t for s in deps)
 
 
@@ -77,11 +81,12 @@ def build(out_dir: str | None = None, quiet: bool = False, jobs: int | None = No
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())  # hipcc wants a home for its caches
     t0 = time.time()
-    _say(f"compiling {len(srcs)} HIP sources for {ARCH} with {jobs} jobs", quiet)
+    _say(f"compiling {len(srcs)} sources (HIP for {ARCH}, C++ host) with {jobs} jobs", quiet)
 
     def compile_one(src: str) -> str:
-        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
-        cmd = [hipcc, *FLAGS, "-I", HERE, "-c", src, "-o", obj]
+        obj = os.path.join(obj_dir, os.path.basename(src).replace(".", "_") + ".o")
+        flags = HOST_FLAGS if src.endswith(".cpp") else FLAGS
+        cmd = [hipcc, *flags, "-I", HERE, "-c", src, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True, env=env)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {os.path.basename(src)}:\n{r.stderr[-4000:]}")

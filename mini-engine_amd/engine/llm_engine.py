@@ -1,5 +1,9 @@
-"""The engine loop: schedule -> step function -> sample -> postprocess
-(reference: ``src/mini_engine/engine.py:59-300``, without its speculative-decoding branches)."""
+"""The engine: a model, its runner and the loop ``plan a step -> run it -> draw tokens -> settle``
+(reference: ``src/mini_engine/engine.py:59-300``, without its speculative-decoding branches). The
+planning and the settling happen in the native host core; this class wires the parts together and
+keeps the reference's Python API: ``from_pretrained``, ``add_request``, ``generate``, ``step``,
+``stats``.
+"""
 
 from __future__ import annotations
 
@@ -7,6 +11,7 @@ import os
 from collections.abc import Iterable
 from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
 from .. import models as _models  # noqa: F401  (registers the architectures)
@@ -17,28 +22,32 @@ from ..parts.decoder import Decoder
 from ..sampling.sampler import Sampler
 from ..weights.loader import FolderSource
 from ..weights.random_init import RandomSource
-from .batch import StepItem
 from .runner import TORCH_DTYPES, ModelRunner
-from .scheduler import ScheduledSeq, Scheduler, SchedulerConfig
+from .scheduler import Scheduler, SchedulerConfig
 from .sequence import SamplingParams, Sequence
 
 
 @dataclass
 class EngineStats:
+    """Counters of the loop, under the reference's names (``engine.py:39-45``)."""
+
     steps: int = 0
-    prompt_tokens: int = 0  # cached hits are in `scheduler.num_cached_tokens`
-    computed_tokens: int = 0  # tokens actually run through the model
+    prompt_tokens: int = 0  # all prompt tokens submitted, whether computed or found in the prefix cache
+    computed_tokens: int = 0  # tokens that went through the model
     generated_tokens: int = 0
     step_batch_sizes: list[int] = field(default_factory=list)
+    # seconds spent in each phase of the steps so far
+    phase_seconds: dict[str, float] = field(default_factory=lambda: {"schedule": 0.0, "forward": 0.0, "sample": 0.0,
+                                                                     "postprocess": 0.0})
 
 
 def kv_cache_bytes_per_token(plan: ModelPlan, dtype: str) -> int:
-    """``2 * kv_heads * head_dim * element size`` summed over the runs of attention layers that own
-    a cache (reference: ``engine.py:54-56``, where that is ``2 * layers * kv_heads * head_dim``)."""
+    """Bytes of keys and values that one token occupies over all layers of ``plan`` in ``dtype``
+    (reference: ``engine.py:54-56``, where it is ``2 * layers * kv_heads * head_dim * element size``).
+    Every mixer says what it keeps through its spec's ``kv_elements_per_token``; one without that
+    attribute keeps no keys."""
     elem = 4 if dtype == "float32" else 2
-    runs = [plan.layers[i].mixer for i in plan.order]
-    return sum(2 * m.num_kv_heads * m.head_dim * elem for m in runs
-               if getattr(m, "kind", "") == "attention" and m.cache_from is None)
+    return elem * sum(int(getattr(plan.layers[i].mixer, "kv_elements_per_token", 0)) for i in plan.order)
 
 
 class LLMEngine:
@@ -47,15 +56,16 @@ class LLMEngine:
             raise ValueError(f"the model was built for {model.dtype}, the engine config says {config.dtype}")
         self.config = config
         self.model = model
-        self.runner = ModelRunner(model, config)
+        eos = set(eos_token_ids)
+        self.runner = ModelRunner(model, config, eos)
+        self.core = self.runner.core
         self.block_manager = self.runner.new_block_manager()
         self.scheduler = Scheduler(
             SchedulerConfig(config.max_num_seqs, config.max_num_batched_tokens, config.max_model_len),
-            self.block_manager,
-            set(eos_token_ids),
-        )
-        self.sampler = Sampler(config.seed, model.device)
+            self.block_manager, eos)
+        self.sampler = Sampler()
         self.stats = EngineStats()
+        self.time_phases = False  # synchronise after each phase of a step and add its time to the stats
 
     @property
     def kv_caches(self):
@@ -88,54 +98,58 @@ class LLMEngine:
     # -------------------------------------------------------------------- API
 
     def add_request(self, prompt_token_ids: list[int], params: SamplingParams | None = None) -> Sequence:
-        seq = Sequence(prompt_token_ids, params or SamplingParams())
+        tokens = [int(t) for t in prompt_token_ids]
         vocab = self.model.plan.vocab_size
-        if min(seq.token_ids) < 0 or max(seq.token_ids) >= vocab:
+        if tokens and (min(tokens) < 0 or max(tokens) >= vocab):
             raise ValueError(f"prompt holds a token id outside the vocabulary of {vocab}")
+        seq = Sequence(tokens, params, core=self.core)
         self.scheduler.add(seq)
-        self.stats.prompt_tokens += len(seq)
+        self.stats.prompt_tokens += len(tokens)
         return seq
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
-        """Run all prompts to completion as one continuously batched workload."""
-        seqs = [self.add_request(p, params) for p in prompts]
+        """Run all prompts to completion as one continuously batched workload; output ids per prompt."""
+        requests = [self.add_request(p, params) for p in prompts]
         while self.scheduler.has_unfinished():
             self.step()
-        return [s.output_token_ids for s in seqs]
+        return [r.output_token_ids for r in requests]
 
     def step(self) -> list[Sequence]:
-        batch = self.scheduler.schedule()
-        if not batch:
+        """One step of the loop; returns the requests that finished in it."""
+        timed = self.time_phases
+        clock = _PhaseClock(self.stats.phase_seconds) if timed else None
+        if self.core.plan() == 0:
             raise RuntimeError("scheduler produced an empty batch with work pending")
-        items = self._prepare(batch)
-        logits = self.runner.step(items)
-        sampling = [item for item in batch if item.samples]
-        sampled = self.sampler.sample(
-            logits,
-            [i.seq.params.temperature for i in sampling],
-            [i.seq.seq_id for i in sampling],
-            [i.seq.num_output_tokens for i in sampling],
-        )
-        it = iter(sampled)
-        next_tokens = [next(it) if item.samples else None for item in batch]
-        self._update_stats(batch)
-        return self.scheduler.postprocess(batch, next_tokens)
-
-    # ---------------------------------------------------------------- private
-
-    @staticmethod
-    def _prepare(batch: list[ScheduledSeq]) -> list[StepItem]:
-        items = []
-        for item in batch:
-            start = item.seq.num_computed_tokens
-            tokens = item.seq.token_ids[start : start + item.num_tokens]
-            items.append(StepItem(item.seq, tokens, start, [item.num_tokens - 1] if item.samples else []))
-        return items
-
-    def _update_stats(self, batch: list[ScheduledSeq]) -> None:
+        tokens, items, rows, *_, warm = (int(v) for v in self.core.step_summary())
+        if timed:
+            clock.lap("schedule")
+        logits = self.runner.run_planned()
+        if timed:
+            clock.lap("forward")
+        drawn = self.sampler.draw(logits, self.runner.batch, rows, bool(warm))
+        if timed:
+            clock.lap("sample")
+        finished = self.scheduler.settle_rows(drawn)
         s = self.stats
         s.steps += 1
-        s.step_batch_sizes.append(len(batch))
-        for item in batch:
-            s.computed_tokens += item.num_tokens
-            s.generated_tokens += int(item.samples)
+        s.step_batch_sizes.append(items)
+        s.computed_tokens += tokens
+        s.generated_tokens += rows
+        if timed:
+            clock.lap("postprocess")
+        return finished
+
+
+class _PhaseClock:
+    def __init__(self, totals: dict[str, float]):
+        import time
+
+        self._now, self.totals = time.perf_counter, totals
+        torch.cuda.synchronize()
+        self.t = self._now()
+
+    def lap(self, phase: str) -> None:
+        torch.cuda.synchronize()
+        t = self._now()
+        self.totals[phase] += t - self.t
+        self.t = t

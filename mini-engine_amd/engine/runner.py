@@ -1,12 +1,12 @@
 """The step function: run a batch of (request, next tokens) through the model from the cache and
 return the logits at the wanted places.
 
-:class:`ModelRunner` owns the decoder, the cache storage and the geometry of the page pools. A step
-runs only the tokens it is given: portions of prompts beside single decoded tokens, cut anywhere
-(reference: ``src/mini_engine/engine.py:158-226``). Steps in which every item is one decoded token
-can be replayed from a HIP graph captured per batch-size bucket (reference:
-``src/mini_engine/cuda_graphs.py``): the graph reads its indices from one static buffer that is
-refilled with a single copy before each replay.
+:class:`ModelRunner` owns the decoder, the cache storage and the native host core (requests, page
+pools, scheduler, step packing). A step runs only the tokens it is given: portions of prompts beside
+single decoded tokens, cut anywhere (reference: ``src/mini_engine/engine.py:158-226``). Steps in
+which every item is one decoded token can be replayed from a HIP graph captured per batch-size
+bucket (reference: ``src/mini_engine/cuda_graphs.py``): the graph reads its indices from one static
+buffer whose pinned source the core refills in place before each replay.
 """
 
 from __future__ import annotations
@@ -17,82 +17,95 @@ from ..cache.block_manager import BlockManager
 from ..cache.storage import CacheStorage, plan_layout
 from ..config.engine_config import EngineConfig
 from ..parts.decoder import Decoder
-from .batch import StepBatch, StepItem, check_pages, make_batch, pack_host, section_offsets, validate_items
+from .batch import StepBatch, StepItem, batch_from_core
+from .core import HostCore, step_layout
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
 def batch_buckets(max_batch: int) -> list[int]:
-    """Batch sizes a decode graph is captured for (reference: ``cuda_graphs.py:28-30``)."""
-    small = [b for b in (1, 2, 4, 8) if b < max_batch]
-    return small + list(range(16, max_batch, 16)) + [max_batch]
+    """Batch sizes a decode graph is captured for: 1, 2, 4, 8 below the cap, then every 16, then the
+    cap itself (reference: ``cuda_graphs.py:28-30``)."""
+    buckets = [b for b in (1, 2, 4, 8) if b < max_batch]
+    buckets += range(16, max_batch, 16)
+    return buckets + [max_batch]
 
 
 class ModelRunner:
-    def __init__(self, decoder: Decoder, config: EngineConfig):
+    def __init__(self, decoder: Decoder, config: EngineConfig, eos_token_ids=()):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible: this engine runs on the GPU only")
         self.decoder, self.config = decoder, config
         self.device = decoder.device
         self.dtype = decoder.dtype
         self.layout = plan_layout(decoder)
+        # slots exist only for models whose layers keep per-request state
+        self.num_state_slots = config.max_num_seqs if self.layout.has_state else 0
         self.storage = CacheStorage(decoder, self.layout, config.num_blocks, config.block_size,
-                                    config.max_num_seqs, self.dtype, self.device)
+                                    self.num_state_slots, self.dtype, self.device)
         self.num_groups = len(self.layout.groups)
         self.max_blocks_per_seq = -(-config.max_model_len // config.block_size)
+        self.core = HostCore(config.block_size, [(g.window, g.num_blocks or config.num_blocks) for g in self.layout.groups],
+                             config.enable_prefix_caching, self.num_state_slots, self.layout.has_state, config.max_num_seqs,
+                             config.max_num_batched_tokens, config.max_model_len, eos_token_ids, config.seed)
         self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, StepBatch, torch.Tensor, torch.Tensor]] = {}
         self._graph_pool = None
         self._copy_done: dict[int, torch.cuda.Event] = {}
-        # per bucket and row: (sequence, its table_epoch, pages written per group) of the last replay
-        self._rows: dict[int, list] = {}
+        self.batch: StepBatch | None = None  # the batch of the last step (its sampling inputs are read from it)
         self.graph_replays = 0
         self.eager_steps = 0
 
     def new_block_manager(self) -> BlockManager:
         c = self.config
         return BlockManager(c.num_blocks, c.block_size, c.enable_prefix_caching, self.layout.groups,
-                            num_state_slots=c.max_num_seqs, has_state=self.layout.has_state)
+                            num_state_slots=self.num_state_slots, has_state=self.layout.has_state, core=self.core)
 
     # ------------------------------------------------------------------------------------ step
-    @torch.inference_mode()
     def step(self, items: list[StepItem]) -> torch.Tensor:
         """Logits float32 [R, V]: for every item in order, for every place in its ``want``.
 
         After a replayed step the result is a view of the graph's output buffer: read it before the
         next step."""
-        replay = self._graph_eligible(items)
-        # a replayed step checks the pages of its block tables while it writes them into the graph's buffer
-        validate_items(items, self.decoder.plan.vocab_size, self.config.block_size, self.layout.groups,
-                       self.config.max_model_len, pages=not replay)
+        core = self.core
+        core.step_clear()
+        try:
+            for it in items:
+                it.seq.bind(core)
+                n = len(it.tokens)
+                if it.start < 0 or it.start + n > len(it.seq) or it.seq.tokens(it.start, n) != [int(t) for t in it.tokens]:
+                    raise ValueError("an item's tokens must be its request's tokens at the item's positions")
+                core.step_add(it.seq._handle, it.start, n, it.want)
+            return self.run_planned()
+        finally:
+            core.step_clear()
+
+    @torch.inference_mode()
+    def run_planned(self) -> torch.Tensor:
+        """Run the step that the core holds (planned by the scheduler or listed by :meth:`step`)."""
+        core = self.core
+        tokens, items, rows, longest, ctx, decode_only, last_only, _ = (int(v) for v in core.step_summary())
+        replay = bool(self.config.cuda_graphs and not self.layout.has_state and decode_only and last_only
+                      and 0 < items <= self.config.max_num_seqs)
+        # a replayed step checks the pages of its block tables while they are written into the graph's buffer
+        core.step_check(self.decoder.plan.vocab_size, scan_pages=not replay)
         if self.layout.has_state:
-            self.storage.zero_state([it.seq.state_slot for it in items if it.start == 0 and it.seq.state_slot >= 0])
+            _, starts, _, _, slots = core.step_items()
+            self.storage.zero_state([s for s, p0 in zip(slots, starts) if p0 == 0 and s >= 0])
         if replay:
             return self._replay(items)
         self.eager_steps += 1
-        batch = make_batch(items, self.num_groups, self.device, self.storage.spare_block, self.storage.spare_slot)
-        return self.decoder.forward(batch)
+        self.batch = batch_from_core(core, self.device, self.storage.spare_block, self.storage.spare_slot)
+        return self.decoder.forward(self.batch)
 
     # ---------------------------------------------------------------------------------- graphs
-    def _graph_eligible(self, items: list[StepItem]) -> bool:
-        if not self.config.cuda_graphs or self.layout.has_state or len(items) > self.config.max_num_seqs:
-            return False
-        for it in items:
-            if len(it.tokens) != 1 or it.want != [0]:
-                return False
-            if any(len(tb) > self.max_blocks_per_seq for tb in it.seq.block_tables):
-                return False
-        return True
-
     def _capture(self, bucket: int):
         widths = [self.max_blocks_per_seq] * self.num_groups
-        total = section_offsets(bucket, bucket, bucket, widths)["_total"][1]
-        host = torch.empty(total, dtype=torch.int32, pin_memory=True)
-        arr, *_ = pack_host([], self.num_groups, widths, pad_items=bucket, spare_block=self.storage.spare_block,
-                            spare_slot=self.storage.spare_slot)
-        host.numpy()[:] = arr
+        layout = step_layout(bucket, bucket, bucket, widths)
+        host = torch.empty(layout["total"], dtype=torch.int32, pin_memory=True)
+        self.core.pack_padding(host.numpy(), widths, bucket, self.storage.spare_block, self.storage.spare_slot)
+        self.core.forget_rows(bucket)
         buf = host.to(self.device)
-        batch = StepBatch(buf, bucket, bucket, bucket, widths)
-        batch.starts, batch.qlens, batch.slots_host = [0] * bucket, [1] * bucket, [-1] * bucket
+        batch = StepBatch(buf, layout).describe([0] * bucket, [1] * bucket, [-1] * bucket)
         batch.max_ctx = self.config.max_model_len
         smaller = [b for b in batch_buckets(self.config.max_num_seqs) if b < bucket]
         batch.least_live = smaller[-1] + 1 if smaller else 1  # fewer items replay a smaller bucket's graph
@@ -117,67 +130,18 @@ class ModelRunner:
             if b not in self._graphs:
                 self._capture(b)
 
-    def _refill(self, bucket: int, batch: StepBatch, host: torch.Tensor, items: list[StepItem]) -> None:
-        """Write this step's indices into the bucket's pinned host buffer, which still holds the last
-        replay's. Token, position, length and slot of every row are written anew. A row of a block
-        table is only extended by the pages its sequence has gained when the row held the same
-        sequence's table last time and nothing but appended pages has changed it since
-        (``Sequence.table_epoch``); tables of window groups, whose entries change as pages are given
-        back, are always written whole. Rows beyond the items point at the spare page and slot."""
-        a = host.numpy()
-        sec, n = batch.sections, len(items)
-        rows = self._rows.setdefault(bucket, [None] * bucket)
-        spare_block, spare_slot = self.storage.spare_block, self.storage.spare_slot
-        tok_o, pos_o, ctx_o, slot_o = (sec[k][0] for k in ("token_ids", "positions", "item_ctx", "state_slots"))
-        starts = [it.start for it in items]
-        pad = bucket - n
-        a[tok_o : tok_o + bucket] = [it.tokens[0] for it in items] + [0] * pad
-        a[pos_o : pos_o + bucket] = starts + [0] * pad
-        a[ctx_o : ctx_o + bucket] = [s + 1 for s in starts] + [1] * pad
-        a[slot_o : slot_o + bucket] = [it.seq.state_slot if it.seq.state_slot >= 0 else spare_slot for it in items] + [spare_slot] * pad
-        a[sec["live_items"][0]] = n
-        bases = [sec[f"table{g}"][0] for g in range(self.num_groups)]
-        windows = [g.window for g in self.layout.groups]
-        for i, it in enumerate(items):
-            seq, row = it.seq, rows[i]
-            same = row is not None and row[0] is seq and row[1] == seq.table_epoch
-            written = row[2] if same else [0] * self.num_groups
-            rows[i] = None  # until the row is complete, should a check below raise
-            need = it.start // self.config.block_size + 1
-            for g, table in enumerate(seq.block_tables):
-                w = batch.widths[g]
-                o = bases[g] + i * w
-                have = written[g] if same and windows[g] == 0 else -1
-                if have < 0:
-                    a[o : o + w] = spare_block
-                    have = 0
-                # pages this step reads or writes that were not checked when an earlier step wrote them
-                first_key = max(0, it.start - windows[g] + 1) if windows[g] > 0 else 0
-                check_pages(table, max(have, first_key // self.config.block_size), need, g)
-                if have < len(table):
-                    a[o + have : o + len(table)] = table[have:]
-                    written[g] = len(table)
-            rows[i] = (seq, seq.table_epoch, written)
-        for i in range(n, bucket):
-            if rows[i] is not None:
-                for g in range(self.num_groups):
-                    o = bases[g] + i * batch.widths[g]
-                    a[o : o + batch.widths[g]] = spare_block
-                rows[i] = None
-
-    def _replay(self, items: list[StepItem]) -> torch.Tensor:
-        n = len(items)
+    def _replay(self, n: int) -> torch.Tensor:
         bucket = next(b for b in batch_buckets(self.config.max_num_seqs) if b >= n)
-        entry = self._graphs.get(bucket) or self._capture(bucket)
-        graph, batch, host, logits = entry
+        graph, batch, host, logits = self._graphs.get(bucket) or self._capture(bucket)
         done = self._copy_done.get(bucket)
         if done is not None:
             done.synchronize()  # the previous upload from this pinned buffer has been read
-        self._refill(bucket, batch, host, items)
+        self.core.step_refill(bucket, host.numpy(), batch.widths, self.storage.spare_block, self.storage.spare_slot)
         batch.buf.copy_(host, non_blocking=True)
         done = done or torch.cuda.Event()
         done.record()
         self._copy_done[bucket] = done
         graph.replay()
         self.graph_replays += 1
+        self.batch = batch
         return logits[:n]

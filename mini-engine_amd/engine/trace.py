@@ -19,6 +19,7 @@ import argparse
 import json
 import os
 import sys
+import tempfile
 
 import numpy as np
 
@@ -26,21 +27,26 @@ PAGE_ROUNDING = 64  # a request's token count is rounded up to this for the --ma
 
 
 def build_session(model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8,
-                  cuda_graphs: bool = True):
+                  cuda_graphs: bool = True, num_blocks: int | None = None):
+    """An engine for replay: a pool of ``num_blocks`` pages (default: what ``max_tokens`` tokens need),
+    no prefix cache. ``max_live`` bounds the batch a decode graph is captured for and, for models whose
+    layers keep per-request state, the number of state slots; a model without such state can have any
+    number of live requests."""
     from ..config.engine_config import EngineConfig
     from ..ops.library import lib
     from .llm_engine import LLMEngine
 
     lib()  # compile (first call in a fresh checkout) or load the kernels before anything else
-    if PAGE_ROUNDING % block_size:
-        raise ValueError(f"block_size={block_size} must divide {PAGE_ROUNDING}")
-    num_blocks = max(1, -(-max_tokens // block_size))
+    if num_blocks is None:
+        if PAGE_ROUNDING % block_size:
+            raise ValueError(f"block_size={block_size} must divide {PAGE_ROUNDING} when --max-tokens sizes the pool")
+        num_blocks = max(1, -(-max_tokens // block_size))
     config = EngineConfig(
         block_size=block_size,
         num_blocks=num_blocks,
         max_num_seqs=max_live,
-        max_num_batched_tokens=max(max_tokens, 1),
-        max_model_len=max(max_tokens, block_size),
+        max_num_batched_tokens=max(num_blocks * block_size, 1),
+        max_model_len=max(num_blocks * block_size, block_size),
         enable_prefix_caching=False,
         dtype=dtype,
         cuda_graphs=cuda_graphs,
@@ -69,24 +75,28 @@ class TraceSession:
                 raise ValueError(f"step {record.get('step')}: request {rid!r} brings no tokens")
             seq = self.live.get(rid)
             if seq is None:
-                seq = self._Sequence(tokens)
-                seq.token_ids = []
-                self.live[rid] = seq
+                seq = self.live[rid] = self._Sequence(tokens, core=self.engine.core)
+            else:
+                seq.extend(tokens)
             start = seq.num_computed_tokens
-            seq.token_ids.extend(tokens)
             if not self.bm.try_allocate(seq, start + len(tokens)):
+                slots = self.bm.slots
+                if slots is not None and seq.state_slot < 0 and not slots.free:
+                    raise RuntimeError(
+                        f"step {record.get('step')}: no state slot is free for request {rid!r} "
+                        f"({slots.num_slots} requests are live); --max-live is too small")
                 raise RuntimeError(
                     f"step {record.get('step')}: out of cache pages for request {rid!r} "
                     f"({self.bm.num_free_blocks} pages of {self.bm.block_size} tokens free); --max-tokens is too small")
             items.append(self._StepItem(seq, tokens, start, want))
-            touched.append((seq, len(tokens)))
+            touched.append((seq, start + len(tokens)))
         out = None
         if items:
             logits = self.engine.runner.step(items)
             if logits.shape[0]:
                 out = logits.float().cpu().numpy()
-            for seq, n in touched:
-                seq.num_computed_tokens += n
+            for seq, computed in touched:
+                seq.num_computed_tokens = computed
                 self.bm.release_passed(seq)
         for rid in record.get("end", []):
             seq = self.live.pop(str(rid), None)
@@ -95,17 +105,54 @@ class TraceSession:
         return out
 
 
+def random_model_folder(spec: str, seed: int, dtype: str) -> str:
+    """Write a model folder with seeded random weights for ``ARCHITECTURE:key=value,...`` (the keys of
+    that architecture's config.json) into a temporary folder and return its path."""
+    import torch
+
+    from .. import models as _models  # noqa: F401
+    from ..config.registry import get_architecture
+    from ..parts.decoder import Decoder
+    from ..weights import write_model_folder
+
+    name, _, rest = spec.partition(":")
+    values: dict = {}
+    for pair in filter(None, rest.split(",")):
+        key, _, value = pair.partition("=")
+        values[key.strip()] = json.loads(value) if value.strip() not in ("True", "False") else value.strip() == "True"
+    values.setdefault("architectures", [name])
+    entry = get_architecture(name)
+    arch_config = entry.config_from_dict(values)
+    folder = tempfile.mkdtemp(prefix="trace_model_")
+    wants = Decoder(entry.plan_from_config(arch_config), torch.float32, "cpu").weight_wants()
+    write_model_folder(folder, arch_config.to_config_json(), wants, seed=seed,
+                       dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    return folder
+
+
 def main(argv: list[str] | None = None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    src = ap.add_mutually_exclusive_group(required=True)
+    src.add_argument("--model", help="folder with config.json and model.safetensors")
+    src.add_argument("--random-shape", metavar="ARCH:key=value,...",
+                     help="instead of a folder: an architecture name and its config.json keys; weights are drawn from --seed")
+    ap.add_argument("--seed", type=int, default=0, help="seed of the random weights of --random-shape")
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder the logits files are written to")
-    ap.add_argument("--max-tokens", type=int, required=True,
+    ap.add_argument("--max-tokens", type=int, default=None,
                     help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache pool")
+    ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--num-blocks", type=int, default=None, help="pages of the cache pool (instead of --max-tokens)")
+    ap.add_argument("--max-live", type=int, default=8,
+                    help="largest batch a decode graph is captured for; state slots of models with per-request state")
     args = ap.parse_args(argv)
+    if args.max_tokens is None and args.num_blocks is None:
+        ap.error("one of --max-tokens and --num-blocks is needed")
     os.makedirs(args.out, exist_ok=True)
     print("[trace_run] loading kernels and model", file=sys.stderr, flush=True)
-    session = TraceSession(build_session(args.model, args.dtype, args.max_tokens))
+    model_dir = args.model or random_model_folder(args.random_shape, args.seed, args.dtype)
+    session = TraceSession(build_session(model_dir, args.dtype, args.max_tokens or 0, args.block_size, args.max_live,
+                                         num_blocks=args.num_blocks))
     print("[trace_run] ready", file=sys.stderr, flush=True)
     for line in sys.stdin:
         line = line.strip()

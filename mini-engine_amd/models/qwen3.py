@@ -183,5 +183,7 @@ register_architecture(
         config_from_dict=Qwen3Config.from_dict,
         config_from_folder=Qwen3Config.from_folder,
         plan_from_config=plan_from_config,
+        model_types=("qwen3",),
+        default_for_unnamed=True,
     )
 )

@@ -4,8 +4,10 @@ Greedy rows take the argmax. A row with temperature ``t > 0`` draws from
 ``softmax(logits / max(t, 1e-5))``; the draw is made on the GPU by adding Gumbel noise to the scaled
 logits and taking the argmax, which has exactly that distribution. The reference draws the whole
 batch from one generator, so its samples depend on what else is in the batch; here the noise of a
-draw is a function of (engine seed, request id, index of the output token) alone, so a request's
-sampled tokens are the same under every way of batching it.
+draw is a function of (engine seed, number of the request within its engine, index of the output
+token) alone, so a request's sampled tokens are the same under every way of batching it and in a
+second engine with the same seed. The native host core derives the keys and packs them, with the
+temperatures, into the step's index buffer.
 """
 
 from __future__ import annotations
@@ -26,26 +28,20 @@ def mix64(z: int) -> int:
     return z ^ (z >> 31)
 
 
-def draw_key(seed: int, request_id: int, output_index: int) -> int:
-    """Key of one draw, as a signed 64-bit integer (the kernel reads the bit pattern)."""
-    k = mix64(mix64(mix64(seed & _MASK) ^ (request_id & _MASK)) ^ (output_index & _MASK))
+def draw_key(seed: int, request_number: int, output_index: int) -> int:
+    """Key of one draw as the host core derives it, as a signed 64-bit integer (the kernel reads the bits)."""
+    k = mix64(mix64(mix64(seed & _MASK) ^ (request_number & _MASK)) ^ (output_index & _MASK))
     return k - (1 << 64) if k >= (1 << 63) else k
 
 
 class Sampler:
-    def __init__(self, seed: int, device: torch.device):
-        self.seed, self.device = seed, device
-
-    def sample(self, logits: torch.Tensor, temperatures: list[float], request_ids: list[int],
-               output_indices: list[int]) -> list[int]:
-        """One token id per row of float32 ``logits`` [R, V]."""
-        if logits.shape[0] == 0:
-            return []
-        if all(t == 0 for t in temperatures):
-            return K.sample(logits).tolist()
-        meta = np.zeros((2, len(temperatures)), dtype=np.int64)
-        meta[0] = np.asarray(temperatures, dtype=np.float32).view(np.int32).astype(np.int64)
-        meta[1] = [draw_key(self.seed, r, i) for r, i in zip(request_ids, output_indices)]
-        dev = torch.from_numpy(meta).to(self.device)
-        temps = dev[0].to(torch.int32).view(torch.float32).contiguous()
-        return K.sample(logits, temps, dev[1].contiguous()).tolist()
+    def draw(self, logits: torch.Tensor, batch, rows: int, tempered: bool) -> np.ndarray:
+        """One token id per wanted row of the step (int32), read back to the host. ``batch`` is the
+        step's batch: its ``temperatures`` and ``sample_keys`` sections hold what each row is drawn with."""
+        if rows == 0:
+            return np.zeros(0, dtype=np.int32)
+        if tempered:
+            out = K.sample(logits[:rows], batch.temperatures[:rows], batch.sample_keys[:rows])
+        else:
+            out = K.sample(logits[:rows])
+        return out.cpu().numpy()

@@ -1,66 +1,142 @@
-"""Packing of a step's batch on the host, and the host-side checks that guard the kernels' indices."""
+"""Packing of a step's batch by the native host core, and its checks that guard the kernels' indices."""
 
 from __future__ import annotations
 
 import numpy as np
 import pytest
 
-from mini_engine_amd.cache import GroupSpec
-from mini_engine_amd.engine.batch import StepItem, pack_host, section_offsets, validate_items
+from mini_engine_amd.engine.core import HostCore, step_layout
 from mini_engine_amd.engine.runner import batch_buckets
-from mini_engine_amd.engine.sequence import Sequence
+from mini_engine_amd.engine.sequence import SamplingParams, Sequence
+from mini_engine_amd.sampling.sampler import draw_key
+from raw_batch import RawItem, pack_raw, raw_layout
+
+BS = 4
 
 
-def seq_with(tables, slot=-1):
-    s = Sequence([1])
-    s.block_tables = [list(t) for t in tables]
-    s.state_slot = slot
-    return s
+def held(core: HostCore, tokens: list[int], computed: int = 0, params=None) -> Sequence:
+    """A request of ``core`` with pages for all its tokens (a fresh pool hands out pages 0, 1, 2, ...)."""
+    seq = Sequence(tokens, params, core=core)
+    assert core.grow(seq._handle, len(tokens))
+    seq.num_computed_tokens = computed
+    return seq
+
+
+def section(arr, lay, name, n):
+    return arr[lay[name]:lay[name] + n].tolist()
+
+
+def test_layout_is_the_documented_order_of_sections():
+    lay = step_layout(5, 2, 3, [4, 2])
+    assert lay == raw_layout(5, 2, 3, [4, 2])
+    assert lay["sample_keys"] % 2 == 0 and lay["total"] == lay["tables"][1] + 2 * 2
 
 
 def test_pack_layout_of_a_mixed_batch():
-    a, b = seq_with([[5, 2]], slot=1), seq_with([[7]])
-    items = [StepItem(a, [11, 12, 13], 4, [0, 2]), StepItem(b, [21], 0, [0])]
-    arr, t, nb, r, widths = pack_host(items, 1, spare_block=9, spare_slot=3)
-    sec = section_offsets(t, nb, r, widths)
-    get = lambda name: arr[sec[name][0] : sec[name][0] + sec[name][1]].tolist()
-    assert (t, nb, r, widths) == (4, 2, 3, [2])
-    assert get("token_ids") == [11, 12, 13, 21] and get("positions") == [4, 5, 6, 0]
-    assert get("token_item") == [0, 0, 0, 1] and get("want_rows") == [0, 2, 3]
-    assert get("item_start") == [0, 3, 4] and get("item_ctx") == [7, 1] and get("state_slots") == [1, 3]
-    assert get("table0") == [5, 2, 7, 9]  # short tables are padded with the spare page
+    core = HostCore(BS, [(0, 16)], num_state_slots=4, has_state=True, seed=11)
+    a = held(core, list(range(30, 37)), computed=4, params=SamplingParams(temperature=0.5))  # pages 0, 1; slot 0
+    b = held(core, [21])  # page 2; slot 1
+    core.step_add(a._handle, 4, 3, [0, 2])
+    core.step_add(b._handle, 0, 1, [0])
+    lay = core.step_layout()
+    arr = np.full(lay["total"], -7, dtype=np.int32)
+    core.step_pack(arr, None, 0, spare_page=9, spare_slot=3)
+    assert (lay["tokens"], lay["items"], lay["rows"], lay["widths"]) == (4, 2, 3, [2])
+    assert section(arr, lay, "token_ids", 4) == [34, 35, 36, 21] and section(arr, lay, "positions", 4) == [4, 5, 6, 0]
+    assert section(arr, lay, "token_item", 4) == [0, 0, 0, 1] and section(arr, lay, "want_rows", 3) == [0, 2, 3]
+    assert section(arr, lay, "item_start", 3) == [0, 3, 4] and section(arr, lay, "item_ctx", 2) == [7, 1]
+    assert section(arr, lay, "state_slots", 2) == [0, 1] and section(arr, lay, "live_items", 1) == [2]
+    assert arr[lay["tables"][0]:lay["tables"][0] + 4].tolist() == [0, 1, 2, 9]  # short tables end in the spare page
+    # the independent packer of the tests agrees on everything but the sampling inputs
+    raw, raw_lay = pack_raw([RawItem([[0, 1]], [34, 35, 36], 4, [0, 2], 0), RawItem([[2]], [21], 0, [0], 1)], 1,
+                            spare_block=9, spare_slot=3)
+    assert raw_lay == lay
+    keep = np.ones(lay["total"], dtype=bool)
+    keep[lay["temperatures"]:lay["sample_keys"] + 2 * lay["rows"]] = False
+    assert np.array_equal(arr[keep], raw[keep])
+    # sampling inputs: only a wanted place that is its request's last token is drawn from
+    temps = arr[lay["temperatures"]:lay["temperatures"] + 3].view(np.float32).tolist()
+    keys = arr[lay["sample_keys"]:lay["sample_keys"] + 6].view(np.int64).tolist()
+    assert temps == [0.0, 0.5, 0.0]
+    assert keys == [0, draw_key(11, 0, 0), draw_key(11, 1, 0)]  # (seed, number of the request, index of the output)
 
 
 def test_padding_items_write_to_the_spare_page():
-    a = seq_with([[4]])
-    arr, t, nb, r, widths = pack_host([StepItem(a, [8], 2, [0])], 1, widths=[3], pad_items=2, spare_block=6, spare_slot=5)
-    sec = section_offsets(t, nb, r, widths)
-    get = lambda name: arr[sec[name][0] : sec[name][0] + sec[name][1]].tolist()
-    assert (t, nb, r) == (3, 3, 3)
-    assert get("positions") == [2, 0, 0] and get("item_ctx") == [3, 1, 1] and get("want_rows") == [0, 1, 2]
-    assert get("table0") == [4, 6, 6, 6, 6, 6, 6, 6, 6] and get("state_slots") == [5, 5, 5]
+    core = HostCore(BS, [(0, 16)])
+    a = held(core, [5, 6, 8], computed=2)
+    core.step_add(a._handle, 2, 1, [0])
+    lay = core.step_layout([3], pad_items=2)
+    arr = np.zeros(lay["total"], dtype=np.int32)
+    core.step_pack(arr, [3], 2, spare_page=6, spare_slot=5)
+    assert (lay["tokens"], lay["items"], lay["rows"]) == (3, 3, 3)
+    assert section(arr, lay, "positions", 3) == [2, 0, 0] and section(arr, lay, "item_ctx", 3) == [3, 1, 1]
+    assert section(arr, lay, "want_rows", 3) == [0, 1, 2] and section(arr, lay, "state_slots", 3) == [5, 5, 5]
+    assert arr[lay["tables"][0]:lay["tables"][0] + 9].tolist() == [0, 6, 6, 6, 6, 6, 6, 6, 6]
+    only_padding = np.zeros(step_layout(2, 2, 2, [3])["total"], dtype=np.int32)
+    core.pack_padding(only_padding, [3], 2, 6, 5)
+    raw, _ = pack_raw([], 1, widths=[3], pad_items=2, spare_block=6, spare_slot=5)
+    assert np.array_equal(only_padding, raw)
+    assert core.step_summary()[1] == 1  # the step itself is untouched by packing padding beside it
 
 
-def test_validation_catches_what_would_make_a_kernel_fault():
-    g = (GroupSpec(),)
-    ok = StepItem(seq_with([[0, 1]]), [1, 2, 3], 2, [2])
-    validate_items([ok], 10, 4, g)
+def test_checks_catch_what_would_make_a_kernel_fault():
+    def check(tokens, start, count, want, pages_for=None, vocab=10, window=0, computed=0, passed=False):
+        core = HostCore(BS, [(window, 32)], max_model_len=64)
+        seq = Sequence(tokens, core=core)
+        assert core.grow(seq._handle, len(tokens) if pages_for is None else pages_for)
+        if passed:
+            seq.num_computed_tokens = computed
+            core.drop_passed(seq._handle)
+        core.step_add(seq._handle, start, count, want)
+        core.step_check(vocab)
+
+    check([1, 2, 3, 4, 5], 2, 3, [2])
     with pytest.raises(ValueError, match="vocabulary"):
-        validate_items([StepItem(seq_with([[0]]), [10], 0, [])], 10, 4, g)
+        check([10], 0, 1, [])
     with pytest.raises(ValueError, match="vocabulary"):
-        validate_items([StepItem(seq_with([[0]]), [-1], 0, [])], 10, 4, g)
+        check([-1], 0, 1, [])
     with pytest.raises(ValueError, match="pages"):
-        validate_items([StepItem(seq_with([[0]]), [1, 2, 3], 2, [])], 10, 4, g)
+        check([1, 2, 3, 4, 5], 2, 3, [], pages_for=4)
     with pytest.raises(ValueError, match="wanted place"):
-        validate_items([StepItem(seq_with([[0]]), [1], 0, [1])], 10, 4, g)
+        check([1], 0, 1, [1])
+    with pytest.raises(ValueError, match="beyond its request"):
+        check([1, 2], 1, 2, [])
+    with pytest.raises(ValueError, match="beyond the limit"):
+        check([1] * 80, 0, 80, [])
     with pytest.raises(ValueError, match="at least one"):
-        validate_items([], 10, 4, g)
-    with pytest.raises(ValueError, match="given back"):
-        validate_items([StepItem(seq_with([[-1, 3]]), [1], 4, [])], 10, 4, g)
-    # in a window group only pages the window still covers have to be there
-    validate_items([StepItem(seq_with([[-1, 3]]), [1], 6, [])], 10, 4, (GroupSpec(window=3),))
-    with pytest.raises(ValueError, match="given back"):
-        validate_items([StepItem(seq_with([[-1, 3]]), [1], 6, [])], 10, 4, (GroupSpec(window=4),))
+        HostCore(BS, [(0, 4)]).step_check(10)
+    # in a window group only pages the window still covers have to be there: with 6 tokens computed and a
+    # window of 3 the first page is given back; a step at position 6 needs keys from 4 on
+    check([1] * 7, 6, 1, [], window=3, computed=6, passed=True)
+    with pytest.raises(ValueError, match="given back"):  # position 4 sees keys from 2 on, which are gone
+        check([1] * 7, 4, 1, [], window=3, computed=6, passed=True)
+
+
+def test_refill_extends_rows_and_rewrites_what_changed():
+    core = HostCore(BS, [(0, 32)], seed=3)
+    a, b = held(core, [1] * 5, computed=4), held(core, [2] * 9, computed=8)
+    widths, lay = [4], step_layout(2, 2, 2, [4])
+    buf = np.zeros(lay["total"], dtype=np.int32)
+    core.pack_padding(buf, widths, 2, 31, 0)
+
+    def replay(seqs):
+        core.step_clear()
+        for s in seqs:
+            core.step_add(s._handle, s.num_computed_tokens, 1, [0])
+        core.step_refill(2, buf, widths, 31, 0)
+        return buf[lay["tables"][0]:lay["tables"][0] + 8].reshape(2, 4).tolist()
+
+    assert replay([a, b]) == [[0, 1, 31, 31], [2, 3, 4, 31]]
+    assert section(buf, lay, "token_ids", 2) == [1, 2] and section(buf, lay, "item_ctx", 2) == [5, 9]
+    buf[lay["tables"][0]] = 77  # the row of a is not rewritten while it only gains pages ...
+    a.extend([1] * 4)
+    assert core.grow(a._handle, 9)
+    a.num_computed_tokens = 8
+    assert replay([a, b])[0] == [77, 1, 5, 31]
+    core.drop(a._handle)  # ... and written whole once its table was cleared
+    assert core.grow(a._handle, 9)
+    assert replay([a, b])[0] == a.block_table + [31]
+    assert replay([b]) == [[2, 3, 4, 31], [31, 31, 31, 31]] and section(buf, lay, "live_items", 1) == [1]
 
 
 def test_buckets_match_the_reference():  # cuda_graphs.py:28-30, tests/test_gpu.py:47

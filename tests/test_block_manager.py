@@ -1,7 +1,7 @@
-"""The cache manager without tensors. The first part restates the vectors the reference's own tests
-hold (``/root/reference/tests/test_block_manager.py``, cited per test); the second part covers what
-is added here: groups with windows, state slots, and random orders of requests under which no page
-may be lost, held twice or freed twice."""
+"""The cache manager (the native host core behind its Python view) without tensors. The first part
+restates the vectors the reference's own tests hold (``tests/test_block_manager.py``, cited per
+test); the second part covers what is added here: groups with windows, state slots, and random
+orders of requests under which no page may be lost, held twice or freed twice."""
 
 from __future__ import annotations
 
@@ -142,7 +142,8 @@ def test_duplicate_content_is_not_double_registered():  # :121-133
     for s in (a, b):
         s.num_computed_tokens = len(s)
         bm.register_computed_blocks(s)
-    assert bm.hash_to_block[a.block_hashes[0]] == a.block_table[0]
+    assert a.num_block_hashes == b.num_block_hashes == 1
+    assert bm.hash_to_block[hash_block(ROOT_HASH, [7] * BS)] == a.block_table[0]
     assert bm.block_hash[b.block_table[0]] is None
     bm.free(a)
     bm.free(b)
@@ -152,11 +153,11 @@ def test_duplicate_content_is_not_double_registered():  # :121-133
 def test_decode_tokens_get_hashed_as_blocks_fill():  # :136-144
     bm = BlockManager(num_blocks=8, block_size=BS)
     seq = computed(bm, [1, 2, 3])
-    assert seq.block_hashes == []
-    seq.token_ids.append(4)
+    assert seq.num_block_hashes == 0
+    seq.extend([4])
     seq.num_computed_tokens = 4
     bm.register_computed_blocks(seq)
-    assert len(seq.block_hashes) == 1
+    assert seq.num_block_hashes == 1
     assert bm.match_prefix([1, 2, 3, 4, 5]) == [seq.block_table[0]]
 
 
@@ -174,11 +175,12 @@ def test_double_free_is_detected():  # :161-169
     bm = BlockManager(num_blocks=4, block_size=BS)
     seq = Sequence([1])
     bm.try_allocate(seq, 1)
-    table = list(seq.block_table)
+    (page,) = seq.block_table
     bm.free(seq)
-    seq.block_table = table
-    with pytest.raises(AssertionError):
-        bm.free(seq)
+    bm.free(seq)  # a request that holds nothing gives nothing back
+    with pytest.raises(AssertionError, match="double free"):
+        bm.core.release_page(0, page)  # a holder that does not exist cannot let go
+    check_invariants(bm, [])
 
 
 def test_cached_blocks_only_seed_an_empty_table():  # block_manager.py:90-91
@@ -268,7 +270,7 @@ def test_random_orders_keep_every_page_accounted_for(seed, windowed):
         elif op < 0.8 and live:
             seq = rng.choice(live)
             if seq.num_computed_tokens == len(seq):
-                seq.token_ids.append(rng.randrange(50))
+                seq.extend([rng.randrange(50)])
             n = rng.randint(1, len(seq) - seq.num_computed_tokens)
             before = [list(t) for t in seq.block_tables]
             if bm.try_allocate(seq, seq.num_computed_tokens + n):
@@ -285,3 +287,28 @@ def test_random_orders_keep_every_page_accounted_for(seed, windowed):
         bm.free(seq)
     check_invariants(bm, [])
     assert all(len(p.free_pool) == p.num_blocks for p in bm.pools)
+
+
+def test_nine_requests_live_at_once_without_state_slots():
+    """A model without per-request state has no slots, so the number of live requests is bound by pages alone."""
+    bm = BlockManager(num_blocks=1000, block_size=BS, num_state_slots=0)
+    live = [Sequence([1, 2, 3]) for _ in range(12)]
+    assert all(bm.try_allocate(s, 3) for s in live) and bm.num_free_blocks == 988
+    check_invariants(bm, live)
+    with_slots = BlockManager(num_blocks=1000, block_size=BS, num_state_slots=8, has_state=True)
+    nine = [Sequence([1, 2, 3]) for _ in range(9)]
+    got = [with_slots.try_allocate(s, 3) for s in nine]
+    assert got == [True] * 8 + [False]  # the ninth lacks a slot, not a page
+    del nine[0]  # a request nobody names any more gives back what it held
+    assert with_slots.try_allocate(nine[-1], 3)
+
+
+def test_a_window_group_refuses_what_its_pool_can_never_hold():
+    """A step's portion needs the window and the portion at once in a window group's pool."""
+    from mini_engine_amd.engine.core import HostCore
+
+    core = HostCore(BS, [(8, 3)], max_num_batched_tokens=16)
+    assert core.can_ever_hold(8)  # two pages
+    assert not core.can_ever_hold(40)  # window 8 + portion 16 = 6 pages + 1 > 3
+    roomy = HostCore(BS, [(8, 7)], max_num_batched_tokens=16)
+    assert roomy.can_ever_hold(4000)

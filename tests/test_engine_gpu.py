@@ -205,10 +205,6 @@ def test_tiny_b_workload_with_temperature_and_shared_prefix(peaked):
     params = SamplingParams(max_tokens=12, temperature=0.8)
 
     def run(stage, **over):
-        import mini_engine_amd.engine.sequence as seqmod
-        import itertools
-
-        seqmod._seq_counter = itertools.count(1000)  # the same request ids in every run
         eng = LLMEngine.from_pretrained(folder, EngineConfig(**{"block_size": 8, "dtype": "float32", "seed": 5, **over}))
         outs = []
         for group in stage:

@@ -30,16 +30,11 @@ def close(got, want, dtype):
     torch.testing.assert_close(got, want, rtol=t["rtol"], atol=t["atol"] * max(1.0, want.abs().max().item()))
 
 
-class FakeSeq:
-    def __init__(self, tables, slot=-1):
-        self.block_tables, self.state_slot = tables, slot
-
-
 def batch_for(items, device="cuda", groups=1):
     """items: list of (tables per group, start, n tokens)."""
-    from mini_engine_amd.engine.batch import StepItem, make_batch
+    from raw_batch import RawItem, make_raw_batch
 
-    return make_batch([StepItem(FakeSeq(t), [0] * n, s, list(range(n))) for t, s, n in items], groups, device)
+    return make_raw_batch([RawItem(t, [0] * n, s, list(range(n))) for t, s, n in items], groups, device)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
