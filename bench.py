@@ -54,9 +54,6 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--skip-prefill", action="store_true", help="profiling aid: do not measure the prefill")
-    ap.add_argument("--zero-context", action="store_true",
-                    help="profiling aid: allocate the context's pages without computing them (a decode step's "
-                         "time does not depend on the cached values); the line's 'data' says so")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
@@ -79,7 +76,7 @@ def main() -> int:
         """Prompts are sized so that every sequence is still decoding, and within the context
         length, when the timed steps end: the first sequences decode while the later ones are still
         being prefilled under the token budget."""
-        prefill_steps = 0 if args.zero_context else -(-batch * ctx // budget) + 1
+        prefill_steps = -(-batch * ctx // budget) + 1
         n = ctx - (k + w + prefill_steps) - 2
         if n < 1:
             raise SystemExit("context is too short for this many steps")
@@ -122,14 +119,6 @@ def main() -> int:
         prompt_len, prefill_steps = prompt_len_for(batch)
         params = SamplingParams(max_tokens=k + w + prefill_steps + 2, temperature=0.0, ignore_eos=True)
         seqs = [engine.add_request(prompt(prompt_len), params) for _ in range(batch)]
-        if args.zero_context:
-            from mini_engine_amd.engine.sequence import SequenceStatus
-
-            for s in seqs:  # admit by hand: pages for the whole prompt, all but its last token "computed"
-                engine.scheduler.waiting.remove(s)
-                assert engine.block_manager.try_allocate(s, prompt_len)
-                s.status, s.num_computed_tokens = SequenceStatus.RUNNING, prompt_len - 1
-                engine.scheduler.running.append(s)
         while any(s.num_output_tokens == 0 for s in seqs):
             engine.step()
         for _ in range(w - 1):
@@ -189,7 +178,7 @@ def main() -> int:
     pts = {f"decode_b{b}": round(m[0], 1) for b, m in measured.items()}
     # the same bound as `roofline`, for the other batch sizes: bytes a step must read / its time / the HBM peak
     pts_frac = {f"decode_b{b}": round(m[2] / HBM_PEAK_GBS, 4) for b, m in measured.items()}
-    if max_batch >= 64 and not args.zero_context:
+    if max_batch >= 64:
         throughput, prefix = reference_workloads()
         pts["throughput_64x256in_128out"] = round(throughput, 1)
         pts["shared_prefix_64x544in_64out"] = round(prefix, 1)
@@ -197,8 +186,7 @@ def main() -> int:
         "metric": f"decode tok/s at batch {args.batch} (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights"
-                + (" (context pages allocated, not computed)" if args.zero_context else ""),
+        "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights",
         "config": {"model": "Qwen3-0.6B shape", "layers": cfg.num_hidden_layers, "layers_of_config": 28,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,

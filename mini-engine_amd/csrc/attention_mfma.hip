@@ -1109,6 +1109,8 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_prefill_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
   if (nh <= 0 || nkv <= 0 || nh % nkv) return me_fail("me_attention_prefill_bf16: nh=%d nkv=%d", nh, nkv);
+  // the kernel takes the tile maximum on unscaled scores and scales afterwards: right for a positive scale only
+  if (!(scale > 0.f) || scale > 3.0e38f) return me_fail("me_attention_prefill_bf16: scale=%g must be positive and finite", scale);
   const int group = nh / nkv;
   if (group > 16) return me_fail("me_attention_prefill_bf16: group size %d exceeds 16", group);
   if ((long long)num_work * nkv > 0x7fffffffLL) return me_fail("me_attention_prefill_bf16: %d x %d blocks exceed the grid", num_work, nkv);

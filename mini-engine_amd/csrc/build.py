@@ -34,7 +34,9 @@ ROCM_LIB = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
 LINK_LIBS = [f"-L{ROCM_LIB}", f"-Wl,-rpath,{ROCM_LIB}", "-lhipblaslt"]
 
 
-HOST_FLAGS = ["-x", "c++", "-O2", "-std=c++17", "-fPIC", "-Wall"]
+ROCM_INCLUDE = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "include")
+# The host sources are plain C++; those that launch kernels see the HIP runtime's C interface only.
+HOST_FLAGS = ["-x", "c++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", ROCM_INCLUDE]
 
 
 def sources() -> list[str]:

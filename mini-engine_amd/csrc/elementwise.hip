@@ -30,6 +30,37 @@ extern "C" int me_embed(void* x, const void* table, const int* ids, int num_toke
   return me_check_launch("me_embed");
 }
 
+// The same lookup for a step whose token ids are still on the device: where fed_rows[t] >= 0 the id of token t
+// is fed_tokens[fed_rows[t]], what an earlier step's sampling kernel wrote there, not ids[t]. A decode step
+// can then be launched before the host has read the tokens of the step before it.
+template <typename T>
+__global__ void embed_fed_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ ids,
+                                 const int* __restrict__ fed_rows, const int* __restrict__ fed_tokens, int hidden,
+                                 int vocab) {
+  const int t = blockIdx.x;
+  const int from = fed_rows[t];
+  int id = from >= 0 ? fed_tokens[from] : ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* row = table + (size_t)id * hidden;
+  float* out = x + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_float(row[i]);
+}
+
+extern "C" int me_embed_fed(void* x, const void* table, const int* ids, const int* fed_rows, const int* fed_tokens,
+                            int num_tokens, int hidden, int vocab, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (hidden <= 0 || vocab <= 0) return me_fail("me_embed_fed: hidden=%d vocab=%d", hidden, vocab);
+  if (!fed_rows || !fed_tokens) return me_fail("me_embed_fed: no fed rows or tokens");
+  const int threads = hidden >= 256 ? 256 : 64;
+  if (dtype == ME_F32)
+    embed_fed_kernel<float><<<num_tokens, threads, 0, stream>>>((float*)x, (const float*)table, ids, fed_rows, fed_tokens,
+                                                                hidden, vocab);
+  else
+    embed_fed_kernel<bf16_t><<<num_tokens, threads, 0, stream>>>((float*)x, (const bf16_t*)table, ids, fed_rows, fed_tokens,
+                                                                 hidden, vocab);
+  return me_check_launch("me_embed_fed");
+}
+
 // ---------------------------------------------------------------------- residual add + RMSNorm
 // For output row r (input row src = rows ? rows[r] : r):
 //   s = x[src] + (delta ? delta[src] : 0);  if (write_x) x[src] = s;

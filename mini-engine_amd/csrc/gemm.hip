@@ -10,8 +10,9 @@
 #define F32_BN 64
 #define F32_BK 16
 
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
-                                                       float* __restrict__ C, int M, int N, int K) {
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(256) void gemm_plain_kernel(const TIn* __restrict__ A, const TIn* __restrict__ W,
+                                                         TOut* __restrict__ C, int M, int N, int K) {
   __shared__ float As[F32_BK][F32_BM + 4];
   __shared__ float Ws[F32_BK][F32_BN + 4];
   const int tid = threadIdx.x;
@@ -25,8 +26,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     for (int j = 0; j < 4; ++j) {
       const int k = k0 + lk + j;
       const int am = m0 + lrow, wn = n0 + lrow;
-      As[lk + j][lrow] = (am < M && k < K) ? A[(size_t)am * K + k] : 0.f;
-      Ws[lk + j][lrow] = (wn < N && k < K) ? W[(size_t)wn * K + k] : 0.f;
+      As[lk + j][lrow] = (am < M && k < K) ? to_float(A[(size_t)am * K + k]) : 0.f;
+      Ws[lk + j][lrow] = (wn < N && k < K) ? to_float(W[(size_t)wn * K + k]) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
-      if (n < N) C[(size_t)m * N + n] = acc[i][j];
+      if (n < N) C[(size_t)m * N + n] = from_float<TOut>(acc[i][j]);
     }
   }
 }
@@ -60,6 +61,27 @@ extern "C" int me_gemm_f32(const float* A, const float* W, float* C, int M, int 
   if (K <= 0) return me_fail("me_gemm_f32: K=%d", K);
   dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
   if (grid.y > 65535) return me_fail("me_gemm_f32: M=%d needs more than 65535 row tiles", M);
-  gemm_f32_kernel<<<grid, 256, 0, stream>>>(A, W, C, M, N, K);
+  gemm_plain_kernel<float, float><<<grid, 256, 0, stream>>>(A, W, C, M, N, K);
   return me_check_launch("me_gemm_f32");
+}
+
+// The same kernel for any storage type: bfloat16 operands are widened as they are loaded, the sum stays
+// float32 on the vector units, the result is stored as float32 or bfloat16. It takes every size, at a
+// fraction of the matrix cores' speed; bfloat16 products that neither the matrix-core kernels nor the GEMM
+// library take (widths that are no multiple of 8) go here.
+extern "C" int me_gemm_plain(const void* A, const void* W, void* C, int M, int N, int K, int in_dtype, int out_dtype,
+                             hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0) return me_fail("me_gemm_plain: K=%d", K);
+  dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
+  if (grid.y > 65535) return me_fail("me_gemm_plain: M=%d needs more than 65535 row tiles", M);
+  if (in_dtype == ME_F32 && out_dtype == ME_F32)
+    gemm_plain_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)A, (const float*)W, (float*)C, M, N, K);
+  else if (in_dtype == ME_BF16 && out_dtype == ME_F32)
+    gemm_plain_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (float*)C, M, N, K);
+  else if (in_dtype == ME_BF16 && out_dtype == ME_BF16)
+    gemm_plain_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (bf16_t*)C, M, N, K);
+  else
+    return me_fail("me_gemm_plain: float32 operands give float32 results");
+  return me_check_launch("me_gemm_plain");
 }

@@ -49,6 +49,8 @@ std::vector<std::vector<int32_t>> unflatten(const me::Core& c, const int32_t* hi
 
 }  // namespace
 
+me::Core* me::core_in_box(void* box) { return &((CoreBox*)box)->core; }
+
 extern "C" {
 
 int me_host_error_kind() { return g_kind; }
@@ -262,14 +264,15 @@ int me_core_step_check(void* box, int vocab_size, int scan_pages) {
 }
 
 // out: tokens, items, rows, total, then the offsets of token_ids, positions, token_item, want_rows, item_start,
-// item_ctx, state_slots, live_items, temperatures, sample_keys, then per group its width and its table's offset.
+// item_ctx, state_slots, live_items, temperatures, sample_keys, token_source, then per group its width and its
+// table's offset.
 static void write_layout(const me::StepLayout& l, int32_t* out) {
   const int head[] = {l.tokens, l.items, l.rows, l.total, l.token_ids, l.positions, l.token_item, l.want_rows, l.item_start,
-                      l.item_ctx, l.state_slots, l.live_items, l.temperatures, l.sample_keys};
-  std::copy(head, head + 14, out);
+                      l.item_ctx, l.state_slots, l.live_items, l.temperatures, l.sample_keys, l.token_source};
+  std::copy(head, head + 15, out);
   for (size_t g = 0; g < l.widths.size(); ++g) {
-    out[14 + 2 * g] = l.widths[g];
-    out[15 + 2 * g] = l.tables[g];
+    out[15 + 2 * g] = l.widths[g];
+    out[16 + 2 * g] = l.tables[g];
   }
 }
 

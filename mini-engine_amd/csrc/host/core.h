@@ -152,7 +152,7 @@ struct StepLayout {
   int tokens = 0, items = 0, rows = 0;
   std::vector<int> widths;
   int token_ids = 0, positions = 0, token_item = 0, want_rows = 0, item_start = 0, item_ctx = 0, state_slots = 0,
-      live_items = 0, temperatures = 0, sample_keys = 0;
+      live_items = 0, temperatures = 0, sample_keys = 0, token_source = 0;
   std::vector<int> tables;
   int total = 0;
   static StepLayout make(int tokens, int items, int rows, const std::vector<int>& widths);
@@ -228,5 +228,8 @@ class Core {
   std::vector<StepItem> step_;
   void reap(Request* r);
 };
+
+// The core inside the box that the C functions of api.cpp hand out.
+Core* core_in_box(void* box);
 
 }  // namespace me

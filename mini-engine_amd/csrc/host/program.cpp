@@ -1,0 +1,447 @@
+// Running a step program: the choice of kernel per operation and step size, and the launches.
+#include "program.h"
+
+#include <algorithm>
+#include <mutex>
+#include <set>
+#include <tuple>
+
+#include "../kernels.h"
+
+namespace me {
+
+namespace {
+
+constexpr int kF32 = 0, kBF16 = 1;
+constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
+constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
+constexpr int kTiledMinRows = 256;
+constexpr int kDecodeWaves = 1024;  // waves that a decode attention launch aims at (four per compute unit of 256)
+
+void ok(int code) {
+  if (code) throw Error(kBadState, me_last_error());
+}
+
+struct Arena {
+  char* base;
+  size_t size, used = 0;
+  void* take(size_t bytes) {
+    const size_t at = (used + 255) & ~(size_t)255;
+    if (at + bytes > size)
+      throw Error(kBadState, "the step needs more workspace than the program's arena holds (" + std::to_string(at + bytes) +
+                                 " of " + std::to_string(size) + " bytes)");
+    used = at + bytes;
+    return base + at;
+  }
+};
+
+struct Pending {
+  const void* delta = nullptr;
+  const float* parts = nullptr;
+  int num_parts = 0;
+  long long stride = 0;
+  bool any() const { return delta || parts; }
+};
+
+// Whether the small matrix-core kernel serves a product of m rows with a weight of `rows_of_w` rows. Up to 16
+// rows always. From 17 to 64 rows for products with many output columns, where a block per 16 columns fills
+// the chip (measured at 24 to 64 rows: 4,096 columns 9.6-12.0 us against 12.3-12.8 with the library, the
+// gated 2 x 3,072 columns 11.5-14.7 against 18.3-19.0 for the library and the SwiGLU kernel; 1,024 columns
+// lose against the library; not the vocabulary-sized head, whose thousands of blocks would each read all of x).
+bool small_serves(int m, int rows_of_w, int k, bool gated) {
+  if (k % 8) return false;
+  if (m <= kSmallFastRows) return true;
+  return m <= kSmallMaxRows && (gated || (rows_of_w >= 2048 && rows_of_w <= 16384));
+}
+
+// Into how many runs of k a product of 17 to 64 rows with few output columns is cut (1: not at all): a block
+// per 16 columns leaves most of the chip idle and makes each block read all of x, so k is cut until about
+// every compute unit has a block, each with at least 256 of k.
+int delta_splits(int rows, int n, int k) {
+  if (!(rows > kSmallFastRows && rows <= kSmallMaxRows) || n >= 2048 || k % 8) return 1;
+  return std::max(1, std::min({8, 256 / ((n + 15) / 16), k / 256}));
+}
+
+std::mutex g_refused_mutex;
+std::set<std::tuple<int, int, int>> g_refused;  // (N, K, output type) the GEMM library has no algorithm for
+
+// A plain bfloat16 product of many rows: the GEMM library, as the reference hands every projection to one;
+// sizes it has no algorithm for go to the kernels of this folder.
+void library_product(const void* x, const void* w, void* out, int m, int n, int k, int out_dtype, hipStream_t stream) {
+  const auto shape = std::make_tuple(n, k, out_dtype);
+  bool refused;
+  {
+    std::lock_guard<std::mutex> hold(g_refused_mutex);
+    refused = g_refused.count(shape) != 0;
+  }
+  if (!refused) {
+    if (me_gemm_bf16_library(x, w, out, m, n, k, out_dtype, stream) == 0) return;
+    std::lock_guard<std::mutex> hold(g_refused_mutex);
+    g_refused.insert(shape);
+  }
+  if (k % 8 == 0) {  // slices of 64 rows through the matrix-core kernel
+    const size_t out_elem = out_dtype == kF32 ? 4 : 2;
+    for (int lo = 0; lo < m; lo += kSmallMaxRows) {
+      const int rows = std::min(kSmallMaxRows, m - lo);
+      ok(me_gemm_bf16_small((const char*)x + (size_t)lo * k * 2, nullptr, nullptr, nullptr, 0.f, nullptr, w,
+                            (char*)out + (size_t)lo * n * out_elem, rows, n, k, 0, 0, out_dtype, 1, stream));
+    }
+    return;
+  }
+  ok(me_gemm_plain(x, w, out, m, n, k, kBF16, out_dtype, stream));
+}
+
+// (keys per split, number of splits) of a decode launch: enough waves to fill the chip, splits of at least 64
+// keys, boundaries at multiples of 64.
+void decode_splits(int items, int kv_units, int max_ctx, int& split_keys, int& num_splits) {
+  const int units = std::max(1, items * kv_units);
+  const int splits = std::max(1, std::min((kDecodeWaves + units - 1) / units, std::max(max_ctx, 64) / 64));
+  split_keys = (max_ctx + splits - 1) / splits;
+  split_keys = (split_keys + 63) / 64 * 64;
+  num_splits = (max_ctx + split_keys - 1) / split_keys;
+}
+
+struct SplitPlan {
+  int split_keys, num_splits, full_splits;
+  const int* live;
+};
+
+// The grid of a launch that a graph replays with fewer live items than it holds is laid out for the fewest it
+// will ever see; the kernel reads the count of live items and takes as many of the grid's splits as they need.
+SplitPlan split_plan(int items, int kv_units, int max_ctx, int least_live, const int* live_count) {
+  int keys, full;
+  decode_splits(items, kv_units, max_ctx, keys, full);
+  if (!live_count || least_live >= items) return {keys, full, full, nullptr};
+  int splits;
+  decode_splits(std::max(1, least_live), kv_units, max_ctx, keys, splits);
+  return {keys, splits, std::min(full, splits), live_count};
+}
+
+class Run {
+ public:
+  Run(const Program& prog, const std::vector<Value>& values, const StepView& s, Arena& arena, int32_t* fed_tokens,
+      hipStream_t stream)
+      : prog_(prog), s_(s), arena_(arena), fed_tokens_(fed_tokens), stream_(stream), dtype_(prog.dtype()),
+        elem_(prog.dtype() == kF32 ? 4 : 2), t_(s.lay.tokens), h_(prog.hidden()) {
+    x_ = (float*)arena_.take((size_t)t_ * h_ * 4);
+    spare_ = (float*)arena_.take((size_t)t_ * h_ * 4);
+    normed_ = arena_.take((size_t)t_ * h_ * elem_);
+    for (const Value& v : values) bufs_.push_back(arena_.take((size_t)t_ * v.cols * v.elem));
+  }
+
+  RunResult go() {
+    for (const Op& op : prog_.ops()) {
+      const size_t mark = arena_.used;
+      step(op);
+      if (op.kind != kOpHead && op.kind != kOpSample && op.kind != kOpLinearDelta) arena_.used = mark;
+      // (the logits, the drawn tokens and partial sums that wait for the next norm outlive their operation)
+      if (op.kind == kOpNormLinear || op.kind == kOpNorm) arena_.used = mark;
+    }
+    return result_;
+  }
+
+ private:
+  const int32_t* idx(int offset) const { return s_.dev + offset; }
+
+  void step(const Op& op) {
+    switch (op.kind) {
+      case kOpEmbed: {
+        const int table_dtype = dtype_;
+        if (s_.fed && fed_tokens_)
+          ok(me_embed_fed(x_, op.p[0], idx(s_.lay.token_ids), idx(s_.lay.token_source), fed_tokens_, t_, h_, prog_.vocab(),
+                          table_dtype, stream_));
+        else
+          ok(me_embed(x_, op.p[0], idx(s_.lay.token_ids), t_, h_, prog_.vocab(), table_dtype, stream_));
+        pending_ = Pending();
+        break;
+      }
+      case kOpNormLinear:
+        norm_linear(op);
+        break;
+      case kOpNorm:
+        add_norm((const float*)op.p[0], op.f[0], bufs_[op.out]);
+        break;
+      case kOpLinear:
+        product(bufs_[op.in], op.p[1], (int)op.i[0], (int)op.i[1], op.i[2] != 0, dtype_, bufs_[op.out]);
+        break;
+      case kOpLinearDelta:
+        linear_delta(op);
+        break;
+      case kOpDelta:
+        pending_ = Pending();
+        pending_.delta = bufs_[op.in];
+        break;
+      case kOpAttention:
+        attention(op);
+        break;
+      case kOpHead:
+        head(op);
+        break;
+      case kOpSample:
+        sample();
+        break;
+      default:
+        throw Error(kBadValue, "unknown operation in a step program");
+    }
+  }
+
+  // x += pending; out = rmsnorm(x) * w, as a kernel of its own.
+  void add_norm(const float* w, float eps, void* out) {
+    ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w, out, nullptr, t_, h_, eps, 1,
+                      dtype_, stream_));
+    pending_ = Pending();
+    release_parts();
+  }
+
+  void release_parts() {
+    if (parts_mark_ != (size_t)-1 && !pending_.parts) {
+      arena_.used = std::min(arena_.used, parts_mark_);
+      parts_mark_ = (size_t)-1;
+    }
+  }
+
+  void norm_linear(const Op& op) {
+    const float* w_norm = (const float*)op.p[0];
+    const int rows_of_w = (int)op.i[0], k = (int)op.i[1];
+    const bool gated = op.i[2] != 0;
+    if (k != h_) throw Error(kBadValue, "a product behind a norm reads the hidden size");
+    const int n = gated ? rows_of_w / 2 : rows_of_w;
+    // decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
+    // residual buffer, since other blocks of the kernel still read the first
+    if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts) {
+      ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
+                            bufs_[op.out], t_, n, k, 1, gated ? 1 : 0, dtype_, 1, stream_));
+      if (pending_.delta) std::swap(x_, spare_);
+      pending_ = Pending();
+      return;
+    }
+    add_norm(w_norm, op.f[0], normed_);
+    product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
+  }
+
+  // out = x . W^T (gated: silu(gate) * up with W = [gate rows; up rows]).
+  void product(const void* x, const void* w, int rows_of_w, int k, bool gated, int out_dtype, void* out) {
+    const int m = t_rows_;
+    const int n = gated ? rows_of_w / 2 : rows_of_w;
+    if (dtype_ == kF32) {  // a true 32-bit product on the vector units, additions in ascending k
+      if (!gated) {
+        ok(me_gemm_f32((const float*)x, (const float*)w, (float*)out, m, n, k, stream_));
+        return;
+      }
+      float* both = (float*)arena_.take((size_t)m * rows_of_w * 4);
+      ok(me_gemm_f32((const float*)x, (const float*)w, both, m, rows_of_w, k, stream_));
+      ok(me_swiglu(both, out, m, n, kF32, stream_));
+      return;
+    }
+    if (small_serves(m, rows_of_w, k, gated)) {
+      ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, out, m, n, k, 0, gated ? 1 : 0, out_dtype, 1, stream_));
+      return;
+    }
+    if (gated) {
+      if (m >= kTiledMinRows && k % 64 == 0 && out_dtype == kBF16) {  // ahead of the library product + SwiGLU kernel
+        ok(me_gemm_bf16_tiled(x, w, out, m, n, k, 1, out_dtype, 0, stream_));
+        return;
+      }
+      void* both = arena_.take((size_t)m * rows_of_w * 2);
+      library_product(x, w, both, m, rows_of_w, k, kBF16, stream_);
+      ok(me_swiglu(both, out, m, n, kBF16, stream_));
+      return;
+    }
+    library_product(x, w, out, m, n, k, out_dtype, stream_);
+  }
+
+  // A product whose result only ever is the pending delta of the residual stream.
+  void linear_delta(const Op& op) {
+    const int n = (int)op.i[0], k = (int)op.i[1];
+    if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
+    const void* x = bufs_[op.in];
+    pending_ = Pending();
+    if (dtype_ == kBF16 && !small_serves(t_, n, k, false)) {
+      const int splits = delta_splits(t_, n, k);
+      if (splits > 1) {  // partial sums over runs of k, each by blocks of its own; the next norm adds them up
+        parts_mark_ = arena_.used;
+        float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);
+        ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], parts, t_, n, k, 0, 0, kF32, splits, stream_));
+        pending_.parts = parts;
+        pending_.num_parts = splits;
+        pending_.stride = (long long)t_ * n;
+        return;
+      }
+    }
+    const size_t mark = arena_.used;
+    product(x, op.p[1], n, k, false, dtype_, bufs_[op.out]);
+    arena_.used = mark;
+    pending_.delta = bufs_[op.out];
+  }
+
+  void attention(const Op& op) {
+    const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], rd = (int)op.i[3], bs = (int)op.i[4];
+    const int window = (int)op.i[5], g = (int)op.i[7];
+    const bool owns = op.i[6] != 0;
+    const float eps = op.f[0], scale = op.f[1];
+    const float* q_w = (const float*)op.p[0];
+    const float* k_w = owns ? (const float*)op.p[1] : nullptr;
+    const float* rope = (const float*)op.p[2];
+    void *kc = (void*)op.p[3], *vc = (void*)op.p[4];
+    if (g < 0 || g >= (int)s_.lay.widths.size()) throw Error(kBadValue, "an attention layer names a cache group the step lacks");
+    const int32_t* table = idx(s_.lay.tables[g]);
+    const int width = s_.lay.widths[g], items = s_.lay.items, group = nh / nkv;
+    if (rope && op.i[8] < s_.max_ctx)
+      throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[8]) + " positions, the step may reach " +
+                                 std::to_string(s_.max_ctx));
+    void* out = bufs_[op.out];
+    const void* qkv = bufs_[op.in];
+    const bool mfma = dtype_ == kBF16 && me_attention_mfma_supported(d, bs) && group <= 16;
+    auto partials = [&](const SplitPlan& sp, float*& part_o, float*& part_ml) {
+      part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * d * 4);
+      part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
+    };
+    const int chunks = (group + 15) / 16;
+    if (s_.decode_only && (long long)width * bs < s_.max_ctx && mfma)
+      throw Error(kBadValue, "the block table cannot hold the step's longest context");
+    if (dtype_ == kBF16 && s_.decode_only && me_attention_decode_fused_supported(d, bs, rd, group)) {
+      // one new token per item: norm, rotary, page write and attention in one launch
+      const SplitPlan sp = split_plan(items, nkv * chunks, s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
+      float *part_o, *part_ml;
+      partials(sp, part_o, part_ml);
+      ok(me_attention_decode_fused_bf16(qkv, q_w, k_w, rope, rd, eps, owns ? 1 : 0, kc, vc, idx(s_.lay.item_ctx), table, width, out,
+                                        part_o, part_ml, items, nh, nkv, d, bs, window, scale, sp.split_keys, sp.num_splits,
+                                        s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves, stream_));
+      return;
+    }
+    void* q = arena_.take((size_t)t_ * nh * d * elem_);
+    int segments = 0, seg_items = 0;
+    if (owns && t_ >= 64) {  // many tokens: the values are written a page segment (a transposed tile) at a time
+      seg_items = items;
+      for (int i = 0; i < items; ++i) segments += (s_.starts[i] + s_.qlens[i] - 1) / 16 - s_.starts[i] / 16 + 1;
+    }
+    ok(me_qk_norm_rope_scatter(qkv, q_w, k_w, rope, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, kc, vc, t_, nh,
+                               nkv, d, rd, bs, eps, owns ? 1 : 0, dtype_, segments ? idx(s_.lay.item_start) : nullptr, seg_items,
+                               segments, stream_));
+    if (mfma && s_.decode_only) {
+      const SplitPlan sp = split_plan(items, nkv * chunks, s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
+      float *part_o, *part_ml;
+      partials(sp, part_o, part_ml);
+      ok(me_attention_decode_bf16(q, kc, vc, idx(s_.lay.item_ctx), table, width, out, part_o, part_ml, items, nh, nkv, d, bs, window,
+                                  scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
+                                  stream_));
+      return;
+    }
+    if (mfma) {
+      auto it = s_.plans.find({nh, nkv, d, window});
+      if (it == s_.plans.end()) throw Error(kBroken, "the step has no work list for a prefill attention layer");
+      const StepView::Plan& p = it->second;
+      float *part_o = nullptr, *part_ml = nullptr;
+      if (p.max_chunks > 1) {
+        part_o = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * d * 4);
+        part_ml = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * 2 * 4);
+      }
+      ok(me_attention_prefill_bf16(q, kc, vc, items, table, width, out, idx(p.work), idx(p.bundle_first), p.bundles, part_o, part_ml,
+                                   p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d, bs, window,
+                                   scale, p.columns, stream_));
+      return;
+    }
+    ok(me_attention_general(q, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, out, t_, nh, nkv, d, bs, window,
+                            scale, dtype_, stream_));
+  }
+
+  // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
+  void head(const Op& op) {
+    const int rows = s_.lay.rows, vocab = prog_.vocab();
+    result_.rows = rows;
+    if (rows == 0) {
+      pending_ = Pending();
+      return;
+    }
+    void* picked = arena_.take((size_t)rows * h_ * elem_);
+    ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, (const float*)op.p[0], picked,
+                      idx(s_.lay.want_rows), rows, h_, op.f[0], 0, dtype_, stream_));
+    pending_ = Pending();
+    float* logits = (float*)arena_.take((size_t)rows * vocab * 4);
+    if (dtype_ == kF32)
+      ok(me_gemm_f32((const float*)picked, (const float*)op.p[1], logits, rows, vocab, h_, stream_));
+    else if (rows <= kSmallFastRows && h_ % 8 == 0)
+      ok(me_gemm_bf16_small(picked, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], logits, rows, vocab, h_, 0, 0, kF32, 1, stream_));
+    else
+      library_product(picked, op.p[1], logits, rows, vocab, h_, kF32, stream_);
+    result_.logits = logits;
+  }
+
+  void sample() {
+    const int rows = s_.lay.rows;
+    if (rows == 0 || !result_.logits) return;
+    int32_t* drawn = fed_tokens_ ? fed_tokens_ : (int32_t*)arena_.take((size_t)rows * 4);
+    void* ws = arena_.take((size_t)rows * me_sample_chunks(prog_.vocab()) * 8);
+    ok(me_sample(result_.logits, rows, prog_.vocab(), (const float*)idx(s_.lay.temperatures),
+                 (const uint64_t*)idx(s_.lay.sample_keys), drawn, ws, stream_));
+    result_.drawn = drawn;
+  }
+
+  const Program& prog_;
+  const StepView& s_;
+  Arena& arena_;
+  int32_t* fed_tokens_;
+  hipStream_t stream_;
+  const int dtype_, elem_, t_, h_;
+  const int& t_rows_ = t_;
+  float *x_, *spare_;
+  void* normed_;
+  std::vector<void*> bufs_;
+  Pending pending_;
+  size_t parts_mark_ = (size_t)-1;
+  RunResult result_;
+};
+
+}  // namespace
+
+RunResult Program::run(const StepView& s, char* arena, size_t arena_bytes, int32_t* fed_tokens, hipStream_t stream) const {
+  Arena a{arena, arena_bytes};
+  Run run(*this, values_, s, a, fed_tokens, stream);
+  return run.go();
+}
+
+std::vector<std::vector<int>> Program::prefill_geometries() const {
+  std::vector<std::vector<int>> out;
+  if (dtype_ != kBF16) return out;
+  for (const Op& op : ops_) {
+    if (op.kind != kOpAttention) continue;
+    const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], bs = (int)op.i[4], window = (int)op.i[5];
+    if (!me_attention_mfma_supported(d, bs) || nh / nkv > 16) continue;
+    std::vector<int> key = {nh, nkv, d, window};
+    if (std::find(out.begin(), out.end(), key) == out.end()) out.push_back(key);
+  }
+  return out;
+}
+
+size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t max_ctx) const {
+  const size_t elem = dtype_ == kF32 ? 4 : 2;
+  const size_t pad = 256;
+  size_t fixed = 2 * ((size_t)tokens * hidden_ * 4 + pad) + (size_t)tokens * hidden_ * elem + pad;
+  for (const Value& v : values_) fixed += (size_t)tokens * v.cols * v.elem + pad;
+  size_t scratch = 0;
+  for (const Op& op : ops_) {
+    size_t need = 0;
+    if (op.kind == kOpNormLinear || op.kind == kOpLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
+    if (op.kind == kOpLinearDelta) need = (size_t)8 * std::min<int64_t>(tokens, kSmallMaxRows) * op.i[0] * 4 + pad;
+    if (op.kind == kOpAttention) {
+      const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
+      const int chunks = (nh / nkv + 15) / 16;
+      size_t most = 0;  // items x splits at its largest over the batch sizes a launch may hold
+      for (int64_t b = 1; b <= items; ++b) {
+        int keys, splits;
+        decode_splits((int)std::max<int64_t>(1, (b + 1) / 2), nkv * chunks, (int)max_ctx, keys, splits);
+        most = std::max(most, (size_t)b * splits);
+      }
+      const size_t decode = most * nh * (d + 2) * 4 + 2 * pad;
+      const size_t prefill = (size_t)(256ll << 20) + (size_t)(256ll << 20) * 2 / d + (size_t)tokens * nh * 8 + 2 * pad;
+      need = (size_t)tokens * nh * d * elem + pad + std::max(decode, tokens > items ? prefill : (size_t)0);
+    }
+    scratch = std::max(scratch, need);
+  }
+  const size_t tail = (size_t)rows * hidden_ * elem + (size_t)rows * vocab_ * 4 + (size_t)rows * 4 +
+                      (size_t)rows * me_sample_chunks(vocab_) * 8 + 4 * pad;
+  // partial sums of the last delta wait beside the head's buffers
+  return fixed + 2 * scratch + tail + (size_t)8 * kSmallMaxRows * hidden_ * 4 + (1 << 16);
+}
+
+}  // namespace me

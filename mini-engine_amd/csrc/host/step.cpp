@@ -4,6 +4,8 @@
 // Sections of the buffer, in order (T tokens, B items, R wanted rows, G groups of width W_g):
 //   token_ids[T] positions[T] token_item[T] want_rows[R] item_start[B+1] item_ctx[B] state_slots[B]
 //   live_items[1] temperatures[R] (float bits) sample_keys[R] (64 bits each, 8-byte aligned)
+//   token_source[T] (-1: the token's id is token_ids[t]; r >= 0: it is the r-th token the step before drew,
+//   which is still on the device)
 //   block_table_0[B, W_0] ... block_table_{G-1}[B, W_{G-1}]
 // Instead of a padded mask the kernels get, per token, its absolute position and the index of its
 // item, and per item and cache group a row of the block table.
@@ -35,6 +37,7 @@ StepLayout StepLayout::make(int tokens, int items, int rows, const std::vector<i
   section(l.temperatures, rows);
   at += at & 1;  // the keys are read as 64-bit values
   section(l.sample_keys, 2 * rows);
+  section(l.token_source, tokens);
   for (int w : widths) {
     l.tables.push_back(at);
     at += items * w;
@@ -109,6 +112,7 @@ StepLayout Core::layout(const std::vector<int>* widths, int pad_items) const {
 
 void Core::pack(int32_t* dst, const StepLayout& lay, int spare_page, int spare_slot) const {
   std::fill(dst, dst + lay.total, 0);
+  std::fill_n(dst + lay.token_source, lay.tokens, -1);
   const int live = (int)step_.size();
   int cursor = 0, row = 0;
   for (int i = 0; i < lay.items; ++i) {
@@ -175,6 +179,7 @@ void Core::refill(int32_t* dst, const StepLayout& lay, std::vector<RowMemo>& row
     dst[lay.token_ids + i] = is_live ? r->tokens[it->start] : 0;
     dst[lay.positions + i] = is_live ? it->start : 0;
     dst[lay.item_ctx + i] = is_live ? it->start + 1 : 1;
+    dst[lay.token_source + i] = -1;
     dst[lay.state_slots + i] = is_live && r->state_slot >= 0 ? r->state_slot : spare_slot;
     float temperature = 0.f;
     uint64_t key = 0;

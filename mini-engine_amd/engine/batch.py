@@ -50,6 +50,7 @@ class StepBatch:
         self.live_items = view("live_items", 1)  # how many of the items are requests; the rest is padding
         self.temperatures = view("temperatures", r).view(torch.float32)  # per wanted row; 0: take the argmax
         self.sample_keys = view("sample_keys", 2 * r).view(torch.int64)  # per wanted row: the key of its draw
+        self.token_source = view("token_source", t)  # -1, or the row of the fed tokens that holds the token's id
         self.least_live = b  # the fewest live items a (replayed) batch of this layout will ever hold
         self._tables = [buf[o : o + b * w].view(b, w) for o, w in zip(layout["tables"], self.widths)]
         # host-side description; static graph batches keep the capture-time values

@@ -18,7 +18,7 @@ _vp, _i32p, _i64p, _u8p = ctypes.c_void_p, ctypes.POINTER(ctypes.c_int32), ctype
 _declared = False
 
 LAYOUT_HEAD = ("tokens", "items", "rows", "total", "token_ids", "positions", "token_item", "want_rows", "item_start",
-               "item_ctx", "state_slots", "live_items", "temperatures", "sample_keys")
+               "item_ctx", "state_slots", "live_items", "temperatures", "sample_keys", "token_source")
 
 
 def _api():
@@ -102,15 +102,15 @@ def chain_digest(parent: bytes, token_ids) -> bytes:
 
 def step_layout(tokens: int, items: int, rows: int, widths: list[int]) -> dict[str, int | list[int]]:
     """Offsets (in int32 units) of the sections of a packed step buffer, as the native packer lays them out."""
-    out = np.zeros(14 + 2 * len(widths), dtype=np.int32)
+    out = np.zeros(15 + 2 * len(widths), dtype=np.int32)
     _ok(_api().me_step_layout(tokens, items, rows, _ptr(_ints(widths)), len(widths), _ptr(out)))
     return _layout_dict(out, len(widths))
 
 
 def _layout_dict(out: np.ndarray, groups: int) -> dict:
-    d = {k: int(v) for k, v in zip(LAYOUT_HEAD, out[:14])}
-    d["widths"] = [int(out[14 + 2 * g]) for g in range(groups)]
-    d["tables"] = [int(out[15 + 2 * g]) for g in range(groups)]
+    d = {k: int(v) for k, v in zip(LAYOUT_HEAD, out[:15])}
+    d["widths"] = [int(out[15 + 2 * g]) for g in range(groups)]
+    d["tables"] = [int(out[16 + 2 * g]) for g in range(groups)]
     return d
 
 
@@ -301,7 +301,7 @@ class HostCore:
         _ok(self._L.me_core_step_check(self._box, vocab_size, int(scan_pages)))
 
     def step_layout(self, widths: list[int] | None = None, pad_items: int = 0) -> dict:
-        out = np.zeros(14 + 2 * self.num_groups, dtype=np.int32)
+        out = np.zeros(15 + 2 * self.num_groups, dtype=np.int32)
         _ok(self._L.me_core_step_layout(self._box, _ptr(None if widths is None else _ints(widths)), pad_items, _ptr(out)))
         return _layout_dict(out, self.num_groups)
 

@@ -30,6 +30,8 @@ def raw_layout(t: int, b: int, r: int, widths: list[int]) -> dict:
     at += at % 2  # 64-bit keys start at an even offset
     lay["sample_keys"] = at
     at += 2 * r
+    lay["token_source"] = at
+    at += t
     lay["tables"] = []
     for w in widths:
         lay["tables"].append(at)
@@ -47,6 +49,7 @@ def pack_raw(items: list[RawItem], num_groups: int, widths: list[int] | None = N
         widths = [max([1] + [len(it.tables[g]) for it in items]) for g in range(num_groups)]
     lay = raw_layout(t, b, r, widths)
     arr = np.zeros(lay["total"], dtype=np.int32)
+    arr[lay["token_source"]:lay["token_source"] + t] = -1  # every token's id is in token_ids
     cursor = row = 0
     for i in range(b):
         it = items[i] if i < len(items) else RawItem([[] for _ in range(num_groups)], [0], 0, [0])
