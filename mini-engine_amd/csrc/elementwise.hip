@@ -104,6 +104,40 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
   }
 }
 
+// The residual add alone, for a norm that is not of this shape and runs as a part of its own:
+// x += delta (+ the partial sums, in the order of the runs).
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,
+                                    int num_parts, size_t part_stride, size_t count) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+    float s = x[i];
+    if (delta) s += to_float(delta[i]);
+    if (parts) {
+      float d = parts[i];
+      for (int p = 1; p < num_parts; ++p) d += parts[p * part_stride + i];
+      s += d;
+    }
+    x[i] = s;
+  }
+}
+
+extern "C" int me_residual_add(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
+                               int num_rows, int dim, int dtype, hipStream_t stream) {
+  if (num_rows <= 0 || dim <= 0) return 0;
+  if (!delta && !parts) return 0;
+  if (parts && num_parts < 1) return me_fail("me_residual_add: partial sums without parts");
+  const size_t count = (size_t)num_rows * dim;
+  const size_t want = (count + 255) / 256;
+  const int blocks = (int)(want < 4096 ? want : 4096);
+  if (dtype == ME_F32)
+    residual_add_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, (const float*)delta, parts, num_parts,
+                                                           (size_t)part_stride, count);
+  else
+    residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>((float*)x, (const bf16_t*)delta, parts, num_parts,
+                                                            (size_t)part_stride, count);
+  return me_check_launch("me_residual_add");
+}
+
 // The same for more than 16 bfloat16 rows: a wave per row, the row in registers (CHUNKS x 8 elements per lane), 16-byte
 // loads and stores, no LDS and no barrier. dim is a multiple of 8 and at most 512 * CHUNKS.
 template <typename T, int CHUNKS>

@@ -64,6 +64,8 @@ long long pack(std::vector<Piece> pieces, int bins, std::vector<std::vector<Piec
 // units: from 4,096 tokens of whole prompts on, or a 2,048-token portion behind 2,048 tokens, 8-24%
 // faster; three prompts of 1,024 tokens, a third slower); not when the wide blocks would be a third
 // emptier than the narrow ones (many items of few tokens).
+static double g_wide_min_blocks = 1.0, g_wide_min_key_tiles = 20.0;  // per compute unit
+
 bool wide_blocks_pay(const int* starts, const int* qlens, int items, int tpb, int window, int nkv, int slots) {
   const int half = std::max(1, tpb / 2);
   long long wide_fill = 0, narrow_fill = 0;
@@ -80,7 +82,7 @@ bool wide_blocks_pay(const int* starts, const int* qlens, int items, int tpb, in
       ++blocks;
       key_tiles += last / 64 - first / 64 + 1;
     }
-  return blocks * nkv >= 1.0 * slots || key_tiles * nkv >= 20.0 * slots;
+  return blocks * nkv >= g_wide_min_blocks * slots || key_tiles * nkv >= g_wide_min_key_tiles * slots;
 }
 
 // A tile of `tpb` query tokens of an item meets the keys from its window's first (rounded down to a
@@ -194,6 +196,17 @@ int me_prefill_work_list(const int32_t* starts, const int32_t* qlens, int items,
   std::copy(list.bundle_first.begin(), list.bundle_first.end(), bundle_first);
   std::copy(list.token_chunks.begin(), list.token_chunks.end(), token_chunks);
   return 0;
+}
+
+// The two limits of wide_blocks_pay (blocks and key tiles per compute unit), for measurements and tests that
+// want one block width whatever the step: sets both, gives the old ones back through `old` (2 doubles).
+void me_prefill_wide_limits(double min_blocks, double min_key_tiles, double* old) {
+  if (old) {
+    old[0] = me::g_wide_min_blocks;
+    old[1] = me::g_wide_min_key_tiles;
+  }
+  me::g_wide_min_blocks = min_blocks;
+  me::g_wide_min_key_tiles = min_key_tiles;
 }
 
 int me_prefill_wide_blocks_pay(const int32_t* starts, const int32_t* qlens, int items, int tpb, int window, int nkv, int slots) {

@@ -132,10 +132,12 @@ class Run {
   RunResult go() {
     for (const Op& op : prog_.ops()) {
       const size_t mark = arena_.used;
+      released_to_ = (size_t)-1;
       step(op);
-      if (op.kind != kOpHead && op.kind != kOpSample && op.kind != kOpLinearDelta) arena_.used = mark;
-      // (the logits, the drawn tokens and partial sums that wait for the next norm outlive their operation)
-      if (op.kind == kOpNormLinear || op.kind == kOpNorm) arena_.used = mark;
+      // the logits, the drawn tokens and partial sums that wait for the next norm outlive their operation;
+      // an operation that used up waiting partial sums gives their memory back too
+      if (op.kind != kOpHead && op.kind != kOpSample && op.kind != kOpLinearDelta)
+        arena_.used = released_to_ != (size_t)-1 ? released_to_ : mark;
     }
     return result_;
   }
@@ -195,7 +197,7 @@ class Run {
 
   void release_parts() {
     if (parts_mark_ != (size_t)-1 && !pending_.parts) {
-      arena_.used = std::min(arena_.used, parts_mark_);
+      arena_.used = released_to_ = parts_mark_;
       parts_mark_ = (size_t)-1;
     }
   }
@@ -388,7 +390,7 @@ class Run {
   void* normed_;
   std::vector<void*> bufs_;
   Pending pending_;
-  size_t parts_mark_ = (size_t)-1;
+  size_t parts_mark_ = (size_t)-1, released_to_ = (size_t)-1;
   RunResult result_;
 };
 

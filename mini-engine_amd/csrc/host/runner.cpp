@@ -32,7 +32,6 @@ struct Runner {
   int parity = 0;
   int32_t* dev_index = nullptr;
   size_t dev_index_ints = 0;
-  int32_t* fed_tokens = nullptr;
   int spare_page = 0, spare_slot = 0;
   int compute_units = 0;
   std::vector<std::vector<int>> geometries;
@@ -94,6 +93,7 @@ void report(const me::RunResult& res, int64_t* out) {
   out[0] = (int64_t)(intptr_t)res.logits;
   out[1] = res.rows;
   out[2] = (int64_t)(intptr_t)res.drawn;
+  out[3] = 0;
 }
 
 }  // namespace
@@ -142,14 +142,15 @@ int64_t me_runner_index_need(void* runner, int tokens, int items, int rows, cons
                return (int64_t)l.total + (int64_t)r->geometries.size() * (entries * 9 + tokens) + 64;)
 }
 
+// The memory of eager steps; may be given anew (larger) between steps, once the device has finished the last.
 int me_runner_memory(void* runner, void* arena, int64_t arena_bytes, int32_t* staging0, int32_t* staging1, int64_t staging_ints,
-                     int32_t* dev_index, int64_t dev_index_ints, int32_t* fed_tokens, int spare_page, int spare_slot) {
+                     int32_t* dev_index, int64_t dev_index_ints, int spare_page, int spare_slot) {
   ME_RUN_GUARD(Runner* r = (Runner*)runner;
                if (!arena || arena_bytes < 1 || !staging0 || !staging1 || !dev_index)
                  throw me::Error(me::kBadValue, "the runner needs an arena, two staging buffers and an index buffer");
                r->arena = (char*)arena; r->arena_bytes = (size_t)arena_bytes; r->staging[0] = staging0; r->staging[1] = staging1;
                r->staging_ints = (size_t)staging_ints; r->dev_index = dev_index; r->dev_index_ints = (size_t)dev_index_ints;
-               r->fed_tokens = fed_tokens; r->spare_page = spare_page; r->spare_slot = spare_slot;
+               r->spare_page = spare_page; r->spare_slot = spare_slot; r->in_flight[0] = r->in_flight[1] = false;
                int dev = 0; hip_ok(hipGetDevice(&dev), "hipGetDevice");
                hip_ok(hipDeviceGetAttribute(&r->compute_units, hipDeviceAttributeMultiprocessorCount, dev), "compute unit count");
                for (int i = 0; i < 2; ++i)
@@ -158,7 +159,8 @@ int me_runner_memory(void* runner, void* arena, int64_t arena_bytes, int32_t* st
 }
 
 // Run the step that the core holds, eagerly: out[0] logits (device, float32 [rows, vocab]), out[1] rows,
-// out[2] the tokens drawn for the rows (device int32), if the program draws.
+// out[2] the tokens drawn for the rows (device int32), if the program draws, out[3] the query columns of the
+// prefill attention's blocks (0: the step ran no such kernel).
 int me_runner_step(void* runner, void* core_box, hipStream_t stream, int64_t* out) {
   ME_RUN_GUARD(
       Runner* r = (Runner*)runner; me::Core& c = *me::core_in_box(core_box);
@@ -199,23 +201,30 @@ int me_runner_step(void* runner, void* core_box, hipStream_t stream, int64_t* ou
       hip_ok(hipEventRecord(r->copied[slot], stream), "hipEventRecord"); r->in_flight[slot] = true;
       s.dev = r->dev_index;
       report(r->prog.run(s, r->arena, r->arena_bytes, nullptr, stream), out);
+      if (!s.plans.empty()) out[3] = s.plans.begin()->second.columns;
       return 0;)
 }
 
 // Run a decode step whose indices already are on the device, in a buffer of `bucket` one-token items laid
-// out with `widths` (what a graph is captured on and replayed from). `fed`: token ids may come from the
-// tokens the step before drew; the draws of this step go to the same place.
-int me_runner_static(void* runner, const int32_t* dev_index, int bucket, const int32_t* widths, int num_groups, int max_ctx,
-                     int least_live, int fed, hipStream_t stream, int64_t* out) {
+// out with `widths` (what a graph is captured on and replayed from), with workspaces from an arena of the
+// caller's (the one a graph was captured on stays the graph's). `drawn`: where the tokens drawn for the
+// rows go (null: into the arena); with `fed`, token ids come from there too, where the buffer's
+// token_source section says so: the tokens the step before drew.
+int me_runner_static(void* runner, void* arena, int64_t arena_bytes, const int32_t* dev_index, int bucket,
+                     const int32_t* widths, int num_groups, int max_ctx, int least_live, int32_t* drawn, int fed,
+                     hipStream_t stream, int64_t* out) {
   ME_RUN_GUARD(
       Runner* r = (Runner*)runner;
-      if (!r->arena) throw me::Error(me::kBadState, "the runner has no memory yet");
+      if (!arena || arena_bytes < 1 || !dev_index) throw me::Error(me::kBadValue, "a static step needs an arena and an index buffer");
+      if (bucket < 1 || max_ctx < 1) throw me::Error(me::kBadValue, "a static step needs items and a context length");
+      if (fed && !drawn) throw me::Error(me::kBadValue, "fed token ids need the buffer the step before drew into");
       me::StepView s;
       s.lay = me::StepLayout::make(bucket, bucket, bucket, std::vector<int>(widths, widths + num_groups));
       std::vector<int> starts(bucket, 0), qlens(bucket, 1);
-      s.starts = starts.data(); s.qlens = qlens.data(); s.max_ctx = max_ctx; s.decode_only = true; s.least_live = least_live;
+      s.starts = starts.data(); s.qlens = qlens.data(); s.max_ctx = max_ctx; s.decode_only = true;
+      s.least_live = std::max(1, std::min(least_live, bucket));
       s.dev = dev_index; s.fed = fed != 0;
-      report(r->prog.run(s, r->arena, r->arena_bytes, r->fed_tokens, stream), out);
+      report(r->prog.run(s, (char*)arena, (size_t)arena_bytes, drawn, stream), out);
       return 0;)
 }
 

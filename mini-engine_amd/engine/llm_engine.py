@@ -19,7 +19,6 @@ from ..config.engine_config import EngineConfig
 from ..config.registry import get_architecture, plan_from_folder
 from ..config.specs import ModelPlan
 from ..parts.decoder import Decoder
-from ..sampling.sampler import Sampler
 from ..weights.loader import FolderSource
 from ..weights.random_init import RandomSource
 from .runner import TORCH_DTYPES, ModelRunner
@@ -63,7 +62,7 @@ class LLMEngine:
         self.scheduler = Scheduler(
             SchedulerConfig(config.max_num_seqs, config.max_num_batched_tokens, config.max_model_len),
             self.block_manager, eos)
-        self.sampler = Sampler()
+        self.sampler = self.runner.sampler
         self.stats = EngineStats()
         self.time_phases = False  # synchronise after each phase of a step and add its time to the stats
 
@@ -126,7 +125,7 @@ class LLMEngine:
         logits = self.runner.run_planned()
         if timed:
             clock.lap("forward")
-        drawn = self.sampler.draw(logits, self.runner.batch, rows, bool(warm))
+        drawn = self.runner.draw(rows, bool(warm))
         if timed:
             clock.lap("sample")
         finished = self.scheduler.settle_rows(drawn)

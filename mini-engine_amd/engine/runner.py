@@ -7,6 +7,10 @@ single decoded tokens, cut anywhere (reference: ``src/mini_engine/engine.py:158-
 which every item is one decoded token can be replayed from a HIP graph captured per batch-size
 bucket (reference: ``src/mini_engine/cuda_graphs.py``): the graph reads its indices from one static
 buffer whose pinned source the core refills in place before each replay.
+
+A model whose parts all wrote their operations into a native step program runs a step as one call
+into C++ (check, pack, upload, every kernel, the draw of the next tokens); any other model runs
+:meth:`Decoder.forward`, one call per kernel, and draws with the sampler.
 """
 
 from __future__ import annotations
@@ -17,8 +21,10 @@ from ..cache.block_manager import BlockManager
 from ..cache.storage import CacheStorage, plan_layout
 from ..config.engine_config import EngineConfig
 from ..parts.decoder import Decoder
+from ..sampling.sampler import Sampler
 from .batch import StepBatch, StepItem, batch_from_core
 from .core import HostCore, step_layout
+from .program import StepMemory, StepProgram, run_static, run_step
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
@@ -32,7 +38,7 @@ def batch_buckets(max_batch: int) -> list[int]:
 
 
 class ModelRunner:
-    def __init__(self, decoder: Decoder, config: EngineConfig, eos_token_ids=()):
+    def __init__(self, decoder: Decoder, config: EngineConfig, eos_token_ids=(), native: bool = True):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible: this engine runs on the GPU only")
         self.decoder, self.config = decoder, config
@@ -48,10 +54,22 @@ class ModelRunner:
         self.core = HostCore(config.block_size, [(g.window, g.num_blocks or config.num_blocks) for g in self.layout.groups],
                              config.enable_prefix_caching, self.num_state_slots, self.layout.has_state, config.max_num_seqs,
                              config.max_num_batched_tokens, config.max_model_len, eos_token_ids, config.seed)
-        self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, StepBatch, torch.Tensor, torch.Tensor]] = {}
+        self.program: StepProgram | None = None
+        self.memory: StepMemory | None = None
+        if native and not self.layout.has_state:
+            program = StepProgram(self.dtype, decoder.plan.hidden_size, decoder.plan.vocab_size, config.max_model_len)
+            if decoder.emit(program):
+                self.program = program
+                self.memory = StepMemory(program, self.device, [self.max_blocks_per_seq] * self.num_groups,
+                                         self.storage.spare_block, self.storage.spare_slot)
+        self.sampler = Sampler()
+        self._graphs: dict[int, tuple] = {}
         self._graph_pool = None
+        self._static_arena: torch.Tensor | None = None
         self._copy_done: dict[int, torch.cuda.Event] = {}
-        self.batch: StepBatch | None = None  # the batch of the last step (its sampling inputs are read from it)
+        self.batch: StepBatch | None = None  # the batch of the last step on the per-kernel path
+        self._logits: torch.Tensor | None = None
+        self._drawn: torch.Tensor | None = None  # what the native program drew for the last step's rows
         self.graph_replays = 0
         self.eager_steps = 0
 
@@ -64,8 +82,7 @@ class ModelRunner:
     def step(self, items: list[StepItem]) -> torch.Tensor:
         """Logits float32 [R, V]: for every item in order, for every place in its ``want``.
 
-        After a replayed step the result is a view of the graph's output buffer: read it before the
-        next step."""
+        The result lies in memory that the next step uses again: read it before the next step."""
         core = self.core
         core.step_clear()
         try:
@@ -86,18 +103,44 @@ class ModelRunner:
         tokens, items, rows, longest, ctx, decode_only, last_only, _ = (int(v) for v in core.step_summary())
         replay = bool(self.config.cuda_graphs and not self.layout.has_state and decode_only and last_only
                       and 0 < items <= self.config.max_num_seqs)
-        # a replayed step checks the pages of its block tables while they are written into the graph's buffer
-        core.step_check(self.decoder.plan.vocab_size, scan_pages=not replay)
+        self._drawn = None
+        if replay:
+            # a replayed step checks the pages of its block tables while they are written into the graph's buffer
+            core.step_check(self.decoder.plan.vocab_size, scan_pages=False)
+            return self._replay(items)
+        self.eager_steps += 1
+        if self.program is not None:  # one call: check, pack, upload, every kernel, the draw
+            c = self.config
+            self.memory.ensure(max(tokens, c.max_num_batched_tokens), max(items, c.max_num_seqs), max(rows, c.max_num_seqs),
+                               max(ctx, c.max_model_len))
+            self._logits, self._drawn, _ = run_step(self.program, self.memory, core)
+            if self._logits is None:
+                self._logits = torch.empty((0, self.decoder.plan.vocab_size), dtype=torch.float32, device=self.device)
+            return self._logits
+        core.step_check(self.decoder.plan.vocab_size, scan_pages=True)
         if self.layout.has_state:
             _, starts, _, _, slots = core.step_items()
             self.storage.zero_state([s for s, p0 in zip(slots, starts) if p0 == 0 and s >= 0])
-        if replay:
-            return self._replay(items)
-        self.eager_steps += 1
         self.batch = batch_from_core(core, self.device, self.storage.spare_block, self.storage.spare_slot)
-        return self.decoder.forward(self.batch)
+        self._logits = self.decoder.forward(self.batch)
+        return self._logits
+
+    def draw(self, rows: int, tempered: bool):
+        """One token id per wanted row of the last step (int32, on the host): what the native program
+        drew beside the logits, or the sampler's draw from them."""
+        if rows == 0:
+            return self.sampler.draw(None, None, 0, False)
+        if self._drawn is not None:
+            return self._drawn[:rows].cpu().numpy()
+        return self.sampler.draw(self._logits, self.batch, rows, tempered)
 
     # ---------------------------------------------------------------------------------- graphs
+    def _forward_static(self, batch: StepBatch, bucket: int):
+        """The launches of one decode step on a graph's static buffers: (logits, drawn or None)."""
+        if self.program is None:
+            return self.decoder.forward(batch), None
+        return run_static(self.program, self._static_arena, batch.buf, bucket, batch.widths, batch.max_ctx, batch.least_live)
+
     def _capture(self, bucket: int):
         widths = [self.max_blocks_per_seq] * self.num_groups
         layout = step_layout(bucket, bucket, bucket, widths)
@@ -109,18 +152,22 @@ class ModelRunner:
         batch.max_ctx = self.config.max_model_len
         smaller = [b for b in batch_buckets(self.config.max_num_seqs) if b < bucket]
         batch.least_live = smaller[-1] + 1 if smaller else 1  # fewer items replay a smaller bucket's graph
+        if self.program is not None and self._static_arena is None:
+            most = self.config.max_num_seqs  # every bucket's graph works in the same memory: replays are serial
+            self._static_arena = torch.empty(self.program.arena_need(most, most, most, self.config.max_model_len),
+                                             dtype=torch.uint8, device=self.device)
         stream = torch.cuda.Stream()
         stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream):
-            self.decoder.forward(batch)  # warm-up outside capture: loads code objects, sets up the GEMM library
+            self._forward_static(batch, bucket)  # warm-up outside capture: loads code objects, sets up the GEMM library
         torch.cuda.current_stream().wait_stream(stream)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, pool=self._graph_pool):
-            logits = self.decoder.forward(batch)
+            logits, drawn = self._forward_static(batch, bucket)
         self._graph_pool = graph.pool()
         torch.cuda.synchronize()
-        self._graphs[bucket] = (graph, batch, host, logits)
+        self._graphs[bucket] = (graph, batch, host, logits, drawn)
         return self._graphs[bucket]
 
     @torch.inference_mode()
@@ -132,7 +179,7 @@ class ModelRunner:
 
     def _replay(self, n: int) -> torch.Tensor:
         bucket = next(b for b in batch_buckets(self.config.max_num_seqs) if b >= n)
-        graph, batch, host, logits = self._graphs.get(bucket) or self._capture(bucket)
+        graph, batch, host, logits, drawn = self._graphs.get(bucket) or self._capture(bucket)
         done = self._copy_done.get(bucket)
         if done is not None:
             done.synchronize()  # the previous upload from this pinned buffer has been read
@@ -144,4 +191,6 @@ class ModelRunner:
         graph.replay()
         self.graph_replays += 1
         self.batch = batch
-        return logits[:n]
+        self._logits = logits[:n]
+        self._drawn = None if drawn is None else drawn[:n]
+        return self._logits

@@ -131,6 +131,25 @@ def add_rmsnorm(
     return out
 
 
+def residual_add(x: torch.Tensor, delta: "torch.Tensor | PartialSums") -> torch.Tensor:
+    """``x += delta`` in place for the float32 residual stream [T, D] and a delta in the compute dtype
+    (or partial sums): the add alone, for a norm that runs as a part of its own."""
+    _want(x, "x", torch.float32, (None, None))
+    t, d = x.shape
+    parts = None
+    if isinstance(delta, PartialSums):
+        parts, delta = delta.parts, None
+        _want(parts, "partial sums", torch.float32, (None, t, d))
+    else:
+        if delta.dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"delta: float32 or bfloat16 expected, got {delta.dtype}")
+        _want(delta, "delta", delta.dtype, (t, d))
+    check(lib().me_residual_add(_p(x), _p(delta), _p(parts), _i(0 if parts is None else parts.shape[0]),
+                                ctypes.c_longlong(0 if parts is None else t * d), _i(t), _i(d),
+                                _i(_code(torch.float32 if delta is None else delta.dtype)), _stream()))
+    return x
+
+
 def rmsnorm(inp: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
     """RMSNorm over the last dim of ``inp`` [..., D]; weight float32 [D]."""
     _want(inp, "inp")
@@ -631,9 +650,6 @@ def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write
     return out
 
 
-_PARTIAL_BYTES_MAX = 256 << 20  # most memory the partial results of cut tiles may take
-
-
 class PrefillPlan:
     """The work list of one step's prefill attention, on the device: which tile of query tokens meets
     which range of keys, and which block runs which entries. It depends on the step's items and on the
@@ -647,96 +663,34 @@ class PrefillPlan:
         self.columns = lib().me_attention_prefill_columns(0) if columns is None else columns
 
 
-PIECE_OVERHEAD = 2  # what starting another piece of work costs a block, in key tiles (3 us against 1.5 us)
-
-
-def _cut(lengths: list[int], cap: int) -> list[tuple[int, int, int, int]]:
-    """Pieces (length, entry, chunk or -1, first key tile) of entries cut into ranges of at most ``cap``
-    key tiles: full ranges first, the remainder last (small remainders fill the gaps beside long pieces)."""
-    pieces = []
-    for i, n in enumerate(lengths):
-        if n <= cap:
-            pieces.append((n, i, -1, 0))
-            continue
-        for j, t0 in enumerate(range(0, n, cap)):
-            pieces.append((min(cap, n - t0), i, j, t0))
-    return pieces
-
-
-def _pack(pieces, bins: int):
-    """Longest piece first into the least loaded bin: (makespan, the bins' pieces)."""
-    import heapq
-
-    heap = [(0, b) for b in range(bins)]
-    loads: list[list] = [[] for _ in range(bins)]
-    for piece in sorted(pieces, key=lambda q: -q[0]):
-        load, b = heapq.heappop(heap)
-        loads[b].append(piece)
-        heapq.heappush(heap, (load + piece[0] + PIECE_OVERHEAD, b))
-    return max(load for load, _ in heap), loads
-
-
 def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int,
                       partial_row_bytes: int = 0):
     """Host side of :class:`PrefillPlan`: (entries int32 [n, 8], first entry of each bundle int32 [b],
-    chunks per token int32 [T], max chunks).
+    chunks per token int32 [T], max chunks), as ``csrc/host/prefill_plan.cpp`` builds it (the native
+    step uses the same builder).
 
     A tile of ``tpb`` query tokens of an item meets the keys from its window's first (rounded down to a
-    multiple of 64) to its last token's position: ``n`` key tiles of 64. A bundle of entries is run by one
-    block per kv head. With more tiles than compute units per kv head the bundles are the tiles,
-    longest first (the hardware starts blocks in that order and evens them out). With at most that many
-    (a prompt of up to a few thousand tokens, whose causal tiles differ in length by a factor of their
-    number; a short portion over a long context) the tiles are cut into ranges of at most ``cap`` key
-    tiles, whose partial results a second kernel adds up, and the pieces are packed into one bundle per
-    compute unit, longest piece first into the emptiest bundle; ``cap`` is the candidate with the
-    shortest longest bundle. (Packing costs a few tenths of a millisecond on the host; steps that mix
-    decoded tokens with a portion have more tiles than that and skip it.) An entry is (item, first token, tokens, first position, first key, last key, chunk
-    or -1, 1 if its bundle ends with it)."""
-    rows = []  # item, first token, tokens, first position, first key, last key, key tiles
-    offset = 0
-    for i, (s0, n) in enumerate(zip(starts, qlens)):
-        for t0 in range(0, n, tpb):
-            count = min(tpb, n - t0)
-            p_first = s0 + t0
-            p_last = p_first + count - 1
-            k0 = (max(p_first - window + 1, 0) // 64) * 64 if window > 0 else 0
-            rows.append((i, offset + t0, count, p_first, k0, p_last, (p_last - k0) // 64 + 1))
-        offset += n
-    lengths = [r[6] for r in rows]
-    bins = max(1, slots // max(1, nkv))
-    longest, total = max(lengths), sum(lengths)
-    if len(rows) > bins:
-        bundles = [[piece] for piece in sorted(_cut(lengths, longest), key=lambda q: -q[0])]
-    else:
-        chunk_limit = 1 << 30
-        if partial_row_bytes:
-            chunk_limit = max(1, _PARTIAL_BYTES_MAX // (partial_row_bytes * offset))
-        caps = {longest, -(-total // bins), -(-total // (2 * bins)), -(-longest // 2), -(-longest // 3)}
-        best = None
-        for cap in sorted(c for c in caps if c >= 1 and -(-longest // c) <= chunk_limit):
-            pieces = _cut(lengths, cap)
-            span, loads = _pack(pieces, bins)
-            score = (span + 0.01 * len(pieces), cap)
-            if best is None or score < best[0]:
-                best = (score, loads)
-        bundles = sorted((b for b in best[1] if b), key=lambda b: -sum(q[0] for q in b))
-    token_chunks = np.ones(offset, dtype=np.int32)
-    chunks_of = {}
-    for bundle in bundles:
-        for _, i, chunk, _ in bundle:
-            chunks_of[i] = max(chunks_of.get(i, 1), chunk + 1)
-    work, bundle_first = [], []
-    for bundle in bundles:
-        bundle_first.append(len(work))
-        for n, i, chunk, t0 in bundle:
-            item, tb, count, p_first, k0, p_last, _ = rows[i]
-            work.append((item, tb, count, p_first, k0 + 64 * t0, min(p_last, k0 + 64 * (t0 + n) - 1), chunk, 0))
-        work[-1] = work[-1][:7] + (1,)
-    for i, c in chunks_of.items():
-        if c > 1:
-            token_chunks[rows[i][1]:rows[i][1] + rows[i][2]] = c
-    return (np.array(work, dtype=np.int32), np.array(bundle_first, dtype=np.int32), token_chunks,
-            max(chunks_of.values()))
+    multiple of 64) to its last token's position. A bundle of entries is run by one block per kv head;
+    tiles of a step with few of them are cut into key ranges whose partial results a second kernel adds
+    up. An entry is (item, first token, tokens, first position, first key, last key, chunk or -1, 1 if
+    its bundle ends with it)."""
+    s = np.ascontiguousarray(starts, dtype=np.int32)
+    q = np.ascontiguousarray(qlens, dtype=np.int32)
+    total = int(q.sum())
+    counts = np.zeros(3, dtype=np.int32)
+    cap_entries = cap_bundles = 0
+    for _ in range(2):  # the first call says how much room the lists need
+        work = np.empty((cap_entries, 8), dtype=np.int32)
+        first = np.empty(cap_bundles, dtype=np.int32)
+        token_chunks = np.empty(total, dtype=np.int32)
+        rc = lib().me_prefill_work_list(_vp(s.ctypes.data), _vp(q.ctypes.data), _i(len(q)), _i(tpb), _i(window), _i(nkv),
+                                        _i(slots), ctypes.c_longlong(partial_row_bytes), _vp(work.ctypes.data), _i(cap_entries),
+                                        _vp(first.ctypes.data), _i(cap_bundles), _vp(token_chunks.ctypes.data), _i(total),
+                                        _vp(counts.ctypes.data))
+        if rc == 0:
+            return work, first, token_chunks, int(counts[2])
+        cap_entries, cap_bundles = int(counts[0]), int(counts[1])
+    raise RuntimeError("me_prefill_work_list: the lists do not fit the room it asked for")
 
 
 _PLANS: dict = {}  # the last plans made, by what they were made from: steps of a serving loop repeat
@@ -754,28 +708,24 @@ def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int,
     return plan
 
 
-# Blocks of twice as many query columns read each key and value tile once for twice the work, but a step
-# has half as many of them. They are taken when every compute unit still gets a whole one, or when the step
-# has so many key tiles to walk that tiles are cut into key ranges anyway (measured on 256 compute units:
-# from 4,096 tokens of whole prompts on, or a 2,048-token portion behind 2,048 tokens, 8-24% faster;
-# three prompts of 1,024 tokens, a third slower).
-PREFILL_WIDE_MIN_BLOCKS = 1.0
-PREFILL_WIDE_MIN_KEY_TILES = 20.0  # per compute unit
-
-
 def wide_blocks_pay(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int) -> bool:
-    # not when the wide blocks would be a third emptier than the narrow ones (many items of few tokens)
-    half = max(1, tpb // 2)
-    if 3 * sum(-(-n // tpb) * tpb for n in qlens) > 4 * sum(-(-n // half) * half for n in qlens):
-        return False
-    blocks = key_tiles = 0
-    for start, n in zip(starts, qlens):
-        for t0 in range(0, n, tpb):
-            last = start + min(t0 + tpb, n) - 1
-            first = max(0, start + t0 - window + 1) if window > 0 else 0
-            blocks += 1
-            key_tiles += last // 64 - first // 64 + 1
-    return blocks * nkv >= PREFILL_WIDE_MIN_BLOCKS * slots or key_tiles * nkv >= PREFILL_WIDE_MIN_KEY_TILES * slots
+    """Whether a step takes prefill attention blocks of twice as many query columns: they read each key and
+    value tile once for twice the work, but a step has half as many of them (the rule and its limits live
+    in ``csrc/host/prefill_plan.cpp``, which the native step uses too)."""
+    s = np.ascontiguousarray(starts, dtype=np.int32)
+    q = np.ascontiguousarray(qlens, dtype=np.int32)
+    return bool(lib().me_prefill_wide_blocks_pay(_vp(s.ctypes.data), _vp(q.ctypes.data), _i(len(q)), _i(tpb), _i(window),
+                                                 _i(nkv), _i(slots)))
+
+
+def set_prefill_wide_limits(min_blocks: float, min_key_tiles: float) -> tuple[float, float]:
+    """Set the two limits of :func:`wide_blocks_pay` (blocks and key tiles per compute unit from which wide
+    blocks are taken) and return the old ones: for measurements and tests that want one block width
+    whatever the step. Plans already made keep their width."""
+    old = (ctypes.c_double * 2)()
+    lib().me_prefill_wide_limits(ctypes.c_double(min_blocks), ctypes.c_double(min_key_tiles), old)
+    _PLANS.clear()
+    return old[0], old[1]
 
 
 def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,

@@ -102,6 +102,20 @@ class Attention(Mixer):
         out = self.attend(q, batch, table, b)
         return K.linear(out, self.w_o, as_delta=True)
 
+    def emit(self, program, h, cache: KVBinding | None = None) -> None:
+        s, b = self.spec, cache
+        if b is None:
+            raise RuntimeError("attention mixer was given no cache")
+        owns = s.cache_from is None
+        qkv = program.linear(h, self.w_qkv)
+        out = program.attention(
+            qkv, q_norm=self.q_norm_w, k_norm=self.k_norm_w if owns else None,
+            rope=None if self.position is None else self.position.tables(program.max_positions),
+            k_cache=b.k_cache, v_cache=b.v_cache, heads=self.nh, kv_heads=self.nkv, head_dim=self.d,
+            block_size=b.block_size, window=int(s.window), writes=owns, group=b.group,
+            eps=0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps), scale=float(s.scale))
+        program.linear_delta(out, self.w_o)
+
     def attend(self, q: torch.Tensor, batch, table: torch.Tensor, b: KVBinding) -> torch.Tensor:
         """bfloat16 with sizes the matrix-core kernels take: the split-context kernel when every item
         brings one token, else the tiled prefill kernel. Everything else (float32, other head or page

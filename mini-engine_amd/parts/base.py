@@ -80,8 +80,15 @@ class Part:
 
 
 class Norm(Part):
-    weight: torch.Tensor
-    eps: float
+    def as_fused(self) -> tuple[torch.Tensor, float] | None:
+        """``(weight float32 [dim], eps)`` when the norm is ``x * rsqrt(mean(x^2) + eps) * weight``: the block
+        then lets the residual add and the norm ride on a neighbouring kernel. None for any other
+        norm: the block adds the residual with a kernel of its own and calls the part."""
+        return None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """The norm of the float32 residual stream ``[T, dim]``, in the compute dtype."""
+        raise NotImplementedError
 
 
 class PositionEncoding(Part):

@@ -54,13 +54,35 @@ class PreNormBlock:
         return self._run(self.ffn, self.ffn_norm, x, a, spare, batch, ())
 
     def _run(self, part, norm, x, pending, spare, batch, extra):
-        h = K.NormedInput(x, pending, norm.weight, norm.eps, self.dtype, spare)
+        fused = norm.as_fused()
+        if fused is None:  # any other norm: the add as a kernel of its own, then the part
+            if pending is not None:
+                K.residual_add(x, pending)
+            return x, spare, part.forward(norm.forward(x), batch, *extra)
+        h = K.NormedInput(x, pending, fused[0], fused[1], self.dtype, spare)
         out = part.forward(h if getattr(part, "takes_normed_input", False) else h.materialize(), batch, *extra)
         if h.residual is None:  # the part never looked at its input: the add still has to happen
             h.materialize()
         if h.residual is not x:
             x, spare = h.residual, x
         return x, spare, out
+
+
+    # ---- the native step program
+    def can_emit(self) -> bool:
+        """Whether every part of the block can write its operations into a step program."""
+        return (all(callable(getattr(p, "emit", None)) for p in (self.mixer, self.ffn))
+                and all(n.as_fused() is not None for n in (self.mixer_norm, self.ffn_norm)))
+
+    def emit(self, program, cache=None) -> None:
+        for part, norm, extra in ((self.mixer, self.mixer_norm, (cache,)), (self.ffn, self.ffn_norm, ())):
+            with program.scope():
+                h = program.normed(norm)
+                out = part.emit(program, h, *extra)
+                if not h.used:  # the part never looked at its input: the add still has to happen
+                    h.value()
+                if out is not None:
+                    program.delta(out)
 
 
 BLOCK_ARRANGEMENTS = {"pre_norm": PreNormBlock}

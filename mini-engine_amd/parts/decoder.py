@@ -71,12 +71,13 @@ class Decoder:
                 seen.add(t.data_ptr())
                 total += t.numel() * t.element_size()
         add(self.head)
-        add(self.final_norm.weight)
+        parts = [self.final_norm]
         for i in set(self.plan.order):
-            for obj in (self.blocks[i].mixer, self.blocks[i].ffn, self.blocks[i].mixer_norm, self.blocks[i].ffn_norm):
-                for v in vars(obj).values():
-                    if isinstance(v, torch.Tensor):
-                        add(v)
+            parts += [self.blocks[i].mixer, self.blocks[i].ffn, self.blocks[i].mixer_norm, self.blocks[i].ffn_norm]
+        for obj in parts:
+            for v in vars(obj).values():
+                if isinstance(v, torch.Tensor):
+                    add(v)
         return total
 
     # ---- step
@@ -92,9 +93,29 @@ class Decoder:
             x, spare, pending = self.blocks[i].forward(x, pending, batch, self.bindings[r], spare)
         return self.logits(x, pending, batch.want_rows)
 
+    def emit(self, program) -> bool:
+        """Write the model's forward pass and the draw of the next tokens into a native step program;
+        False (and nothing written) when a part cannot: a part without ``emit``, a norm that is not
+        RMS-shaped. The cache bindings have to be in place."""
+        if self.embed_table is None:
+            raise RuntimeError("weights are not loaded")
+        if not all(self.blocks[i].can_emit() for i in set(self.plan.order)) or self.final_norm.as_fused() is None:
+            return False
+        program.embed(self.embed_table)
+        for r, i in enumerate(self.plan.order):
+            self.blocks[i].emit(program, self.bindings[r])
+        program.head(self.final_norm, self.head)
+        program.sample()
+        return True
+
     def logits(self, x: torch.Tensor, pending: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
         if rows.numel() == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
-        h = K.add_rmsnorm(x, pending, self.final_norm.weight, self.final_norm.eps, self.dtype, rows=rows,
-                          write_x=False)
+        fused = self.final_norm.as_fused()
+        if fused is not None:
+            h = K.add_rmsnorm(x, pending, fused[0], fused[1], self.dtype, rows=rows, write_x=False)
+        else:
+            if pending is not None:
+                K.residual_add(x, pending)
+            h = self.final_norm.forward(x.index_select(0, rows.long()))
         return K.linear(h, self.head, torch.float32)

@@ -36,5 +36,9 @@ class GatedMlp(FeedForward):
         act = K.linear(h, self.w_gate_up, gated=True)
         return K.linear(act, self.w_down, as_delta=True)
 
+    def emit(self, program, h) -> None:
+        act = program.linear(h, self.w_gate_up, gated=True)
+        program.linear_delta(act, self.w_down)
+
 
 FEED_FORWARDS.register("gated_mlp", GatedMlp)

@@ -23,6 +23,12 @@ class RMSNorm(Norm):
     def load(self, tensors, name: str) -> None:
         self.weight = tensors[name]
 
+    def as_fused(self):
+        return self.weight, self.eps
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return K.add_rmsnorm(x, None, self.weight, self.eps, self.dtype, write_x=False)
+
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
         """Norm of activations [..., dim] in the compute dtype (no residual involved)."""
         return K.rmsnorm(x, self.weight, self.eps)

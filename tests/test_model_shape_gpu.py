@@ -59,7 +59,7 @@ def test_benchmark_layer_sizes_against_plain(model, graphs):
     assert all(len(p.free_pool) == p.num_blocks for p in session.bm.pools)
 
 
-def test_long_prompt_runs_wide_attention_blocks_and_agrees_with_narrow_ones(model, monkeypatch):
+def test_long_prompt_runs_wide_attention_blocks_and_agrees_with_narrow_ones(model):
     """A 4,200-token prompt gives every compute unit a block of 256 query columns, so the step takes
     the wide prefill attention blocks; its logits agree with those of the narrow blocks (which the
     test above holds against the plain implementation), and so does a later portion of 100 tokens
@@ -71,24 +71,22 @@ def test_long_prompt_runs_wide_attention_blocks_and_agrees_with_narrow_ones(mode
     tokens = random_prompt(4300, 512, seed=77)
     steps = [{"step": 0, "entries": [{"id": "p", "tokens": tokens[:4200], "want": list(range(4190, 4200))}], "end": []},
              {"step": 1, "entries": [{"id": "p", "tokens": tokens[4200:], "want": list(range(90, 100))}], "end": ["p"]}]
-    chosen = []
-    make = K._make_prefill_plan
-
-    def spy(*args, **kwargs):
-        plan = make(*args, **kwargs)
-        chosen.append(plan.columns)
-        return plan
-
-    monkeypatch.setattr(K, "_make_prefill_plan", spy)
     outs = {}
-    for name, (blocks, tiles) in {"chosen": (K.PREFILL_WIDE_MIN_BLOCKS, K.PREFILL_WIDE_MIN_KEY_TILES), "narrow": (1e9, 1e9)}.items():
-        monkeypatch.setattr(K, "PREFILL_WIDE_MIN_BLOCKS", blocks)
-        monkeypatch.setattr(K, "PREFILL_WIDE_MIN_KEY_TILES", tiles)
-        K._PLANS.clear()
-        chosen.clear()
-        session = TraceSession(build_session(folder, "bfloat16", 4352, block_size=16, max_live=2, cuda_graphs=False))
-        outs[name] = th.replay_in_process(session, steps)
-        assert chosen == ([256, 128] if name == "chosen" else [128, 128]), (name, chosen)
+    chosen_limits = K.set_prefill_wide_limits(1e9, 1e9)
+    try:
+        for name, limits in {"narrow": (1e9, 1e9), "chosen": chosen_limits}.items():
+            K.set_prefill_wide_limits(*limits)
+            session = TraceSession(build_session(folder, "bfloat16", 4352, block_size=16, max_live=2, cuda_graphs=False))
+            program = session.engine.runner.program
+            assert program is not None
+            outs[name], columns = [], []
+            for step in steps:
+                outs[name].append(torch.from_numpy(session.run_step(step).copy()))
+                columns.append(program.last_prefill_columns)
+            assert not session.live
+            assert columns == ([256, 128] if name == "chosen" else [128, 128]), (name, columns)
+    finally:
+        K.set_prefill_wide_limits(*chosen_limits)
     for step in (0, 1):
         a, b = outs["chosen"][step], outs["narrow"][step]
         assert len({int(t) for t in a.argmax(-1)}) > 1
