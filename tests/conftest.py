@@ -34,10 +34,15 @@ def tiny_configs():
     c = Qwen3Config(vocab_size=320, hidden_size=128, intermediate_size=256, num_hidden_layers=2,
                     num_attention_heads=4, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6,
                     rope_theta=50000.0, max_position_embeddings=2048, tie_word_embeddings=True)
-    return {"A": a, "B": b, "C": c}
+    # the head size, the group size and the page size of the benchmark's model, so that portions, tails and
+    # pages that are used again pass through the kernels that serve it
+    d = Qwen3Config(vocab_size=448, hidden_size=256, intermediate_size=384, num_hidden_layers=2,
+                    num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+                    rope_theta=1e6, max_position_embeddings=4096, tie_word_embeddings=False)
+    return {"A": a, "B": b, "C": c, "D": d}
 
 
-BLOCK_SIZES = {"A": 16, "B": 8, "C": 16}
+BLOCK_SIZES = {"A": 16, "B": 8, "C": 16, "D": 16}
 
 
 def write_tiny(folder: str, cfg, seed: int = 0, std: float = 0.02, dtype=torch.bfloat16) -> str:

@@ -176,7 +176,7 @@ def test_bfloat16_generation_stays_close(peaked):
     tokens agree, and each engine token is one the plain logits rank near the top."""
     from mini_engine_amd import SamplingParams
 
-    for name in ("A", "B", "C"):  # C: heads of 64, the matrix-core attention kernels
+    for name in ("A", "B", "C", "D"):  # C, D: heads of 64 and 128, the matrix-core attention kernels
         folder, pcfg, w = peaked[name]
         eng = engine(folder, name, dtype="bfloat16", block_size=16)
         prompts = prompts_for(name)
@@ -186,7 +186,7 @@ def test_bfloat16_generation_stays_close(peaked):
         for p, g in zip(prompts, got):
             logits = plain.forward_logits(w, pcfg, p + g)[len(p) - 1 : -1]
             chosen = logits.gather(1, torch.tensor(g)[:, None])[:, 0]
-            assert ((logits.max(-1).values - chosen) < 0.05 * logits.abs().max()).all()
+            assert ((logits.max(-1).values - chosen) <= 0.02 * logits.abs().max(-1).values).all()
 
 
 def test_tiny_b_workload_with_temperature_and_shared_prefix(peaked):

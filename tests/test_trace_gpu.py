@@ -1,5 +1,6 @@
 """Replay of the same requests under every way of cutting them, in float32 and bfloat16, on the
-tiny configurations (C reaches the matrix-core attention kernels in bfloat16), compared with the plain implementation position by position:
+tiny configurations (C and D reach the matrix-core attention kernels in bfloat16, D with the head, group
+and page sizes of the benchmark's model), compared with the plain implementation position by position:
 whole; most in one step and the last 32 tokens one by one; portions of changing size down to two
 tokens; mixed with other requests in a pool so small that pages are used again."""
 
@@ -49,7 +50,7 @@ def plain_for(folders, name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_replay_matches_plain(tiny_folders, name, dtype, mode):
     reqs = requests_for(name)
@@ -71,10 +72,12 @@ def test_replay_matches_plain(tiny_folders, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_modes_agree_with_each_other_beyond_rounding(tiny_folders, dtype):
-    """The logits at a position do not depend on the cut: compare the modes directly (tighter than
-    through the plain implementation in bfloat16, where both share the storage rounding)."""
-    name = "B"
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_modes_agree_with_each_other_beyond_rounding(tiny_folders, name, dtype):
+    """The logits at a position do not depend on the cut: compare the modes directly, row by row
+    (float32: the same sums in the same order, so nearly the same bits; bfloat16: the kernels of
+    prompts and of decoded tokens round at different places, measured 1.1-1.8% of a row's largest
+    logit)."""
     reqs = requests_for(name)
     session = session_for(tiny_folders, name, dtype, 320)
     results = []
@@ -84,8 +87,9 @@ def test_modes_agree_with_each_other_beyond_rounding(tiny_folders, dtype):
     tol = 2e-5 if dtype == "float32" else 0.02
     for other in results[1:]:
         for rid in reqs:
-            err = (other[rid] - results[0][rid]).abs().max().item()
-            assert err < tol * max(1.0, results[0][rid].abs().max().item()), (rid, err)
+            err = (other[rid] - results[0][rid]).abs().max(dim=-1).values
+            scale = results[0][rid].abs().max(dim=-1).values
+            assert (err <= tol * scale).all(), (name, rid, (err / scale).max().item())
 
 
 def test_first_tokens_of_a_sequence(tiny_folders):

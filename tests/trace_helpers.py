@@ -113,14 +113,19 @@ def plain_logits(folder: str, requests: dict[str, list[int]]) -> dict[str, torch
 
 def assert_logits_close(got: torch.Tensor, want: torch.Tensor, dtype: str, what: str = "") -> None:
     """float32: the reference's own parity tolerance (tests/test_parity.py:76), tightened.
-    bfloat16: 2.5% of the logits' scale (reference tests/test_gpu.py:42 takes 2e-2 on attention)."""
+    bfloat16, row by row: no element further off than 2% of that row's largest logit, and the row's
+    root-mean-square error at most 1.5% of the row's root mean square (measured on the tiny
+    configurations: 0.9-1.3% and 0.8-1.1%; the reference's tests/test_gpu.py:42 takes 2e-2 on
+    attention alone)."""
     assert got.shape == want.shape, (what, got.shape, want.shape)
     err = (got - want).abs()
     if dtype == "float32":
-        bad = err > 5e-5 + 1e-4 * want.abs()
+        bad = (err > 5e-5 + 1e-4 * want.abs()).any(dim=-1)
     else:
-        bad = err > 0.025 * max(1.0, want.abs().max().item())
+        bad = (err.max(dim=-1).values > 0.02 * want.abs().max(dim=-1).values) | (
+            err.pow(2).mean(dim=-1).sqrt() > 0.015 * want.pow(2).mean(dim=-1).sqrt())
     if bad.any():
-        pos = int(bad.any(dim=-1).nonzero()[0])
+        pos = int(bad.nonzero()[0])
         raise AssertionError(f"{what}: first wrong position {pos} of {got.shape[0]}, max abs error "
-                             f"{err.max().item():.3e} (at that position {err[pos].max().item():.3e})")
+                             f"{err.max().item():.3e} (at that position {err[pos].max().item():.3e}, "
+                             f"the row's largest logit {want[pos].abs().max().item():.3e})")
