@@ -1,6 +1,6 @@
 """A plain, slow Qwen3 dense decoder: whole sequences, no cache, no batching, float32 on the CPU.
 
-Written from the formulas of the reference (``/root/reference/src/mini_engine``), one function per
+Written from the formulas of the reference (``src/mini_engine`` there), one function per
 part, each citing the lines it restates. It shares no code with the package under test: it reads
 ``config.json`` with ``json`` and the weights with the ``safetensors`` library, and uses only
 elementary torch operations (matmul, exp, sum, ...), so that each library routine that computes the

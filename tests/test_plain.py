@@ -1,8 +1,8 @@
 """Pins the plain implementation (tests/plain_qwen3.py) by what fixes each formula beside the
 reference's text: special cases that reduce to a library routine, invariants, and the one mask
 vector the reference's own tests hold. Each check is chosen so that a plausible mistake fails it.
-The reference holds no numeric model vectors (its parity tests run an installed model), so whole
-model parity with it is "parity unpinned" beyond these checks."""
+The reference holds no numeric model vectors (its parity tests run an installed model's code, which
+is no source here), so whole model parity with it is "parity unpinned" beyond these checks."""
 
 from __future__ import annotations
 
@@ -82,6 +82,65 @@ def test_rope_scores_depend_on_distance_only():
 
     torch.testing.assert_close(score(9, 4), score(105, 100), rtol=1e-4, atol=1e-5)
     assert abs(score(9, 4) - score(9, 5)) > 1e-3  # and does depend on the distance
+
+
+# ------------------------------------------------------------------------- the attention block
+def _block_inputs(seed: int, eps: float):
+    g = torch.Generator().manual_seed(seed)
+    cfg = plain.PlainConfig(vocab_size=11, hidden_size=24, intermediate_size=8, num_layers=1, num_heads=4, num_kv_heads=2,
+                            head_dim=16, rms_norm_eps=eps, rope_theta=10000.0, tie_word_embeddings=True)
+    w = {"a.q_proj.weight": torch.randn(64, 24, generator=g), "a.k_proj.weight": torch.randn(32, 24, generator=g),
+         "a.v_proj.weight": torch.randn(32, 24, generator=g), "a.o_proj.weight": torch.randn(24, 64, generator=g),
+         # weights that differ inside every rotated pair (j, j + d/2): where the norm sits then shows
+         "a.q_norm.weight": 0.5 + torch.rand(16, generator=g), "a.k_norm.weight": 0.5 + torch.rand(16, generator=g)}
+    return cfg, w, torch.randn(9, 24, generator=g)
+
+
+def test_attention_block_depends_on_distances_only_so_qk_norm_sits_before_rope():
+    """With the q/k norm before the rotation, scores are a function of position differences, so a
+    shift of all positions changes nothing. A norm weight applied after the rotation scales the two
+    elements of a rotated pair differently and the scores come to depend on the positions themselves:
+    the same check on such a variant fails, which shows that it can."""
+    cfg, w, x = _block_inputs(3, 1e-6)
+    here = plain.attention_block(x, w, "a", cfg, torch.arange(9))
+    shifted = plain.attention_block(x, w, "a", cfg, torch.arange(9) + 777)
+    torch.testing.assert_close(shifted, here, rtol=1e-3, atol=1e-3)
+
+    def norm_after_rope(positions):
+        q = (x @ w["a.q_proj.weight"].T).view(9, 4, 16)
+        k = (x @ w["a.k_proj.weight"].T).view(9, 2, 16)
+        v = (x @ w["a.v_proj.weight"].T).view(9, 2, 16)
+        cos, sin = plain.rope_tables(positions, 16, cfg.rope_theta)
+        q = plain.rms_norm(plain.apply_rope(q, cos, sin), w["a.q_norm.weight"], 1e-6)
+        k = plain.rms_norm(plain.apply_rope(k, cos, sin), w["a.k_norm.weight"], 1e-6)
+        return plain.grouped_causal_attention(q, k, v, 16**-0.5).reshape(9, -1) @ w["a.o_proj.weight"].T
+
+    assert (norm_after_rope(torch.arange(9)) - norm_after_rope(torch.arange(9) + 777)).abs().max() > 0.05
+    assert (here - norm_after_rope(torch.arange(9))).abs().max() > 0.05  # and the two orders are different functions
+
+
+def test_attention_block_equals_library_routines_put_together():
+    """The whole block from library routines: ``F.rms_norm`` per head with the one [d] weight (and an
+    eps large enough to matter, the configuration's only one), the rotation as a complex product,
+    ``F.scaled_dot_product_attention`` with its default scale (1/sqrt(d)) and ``is_causal``. A scale
+    from another size, a norm weight per head, a norm on v or an eps of its own would fail it."""
+    cfg, w, x = _block_inputs(4, 0.3)
+    t, nh, nkv, d = 9, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+    got = plain.attention_block(x, w, "a", cfg, torch.arange(t))
+    q = F.rms_norm((x @ w["a.q_proj.weight"].T).view(t, nh, d), (d,), w["a.q_norm.weight"], 0.3)
+    k = F.rms_norm((x @ w["a.k_proj.weight"].T).view(t, nkv, d), (d,), w["a.k_norm.weight"], 0.3)
+    v = (x @ w["a.v_proj.weight"].T).view(t, nkv, d)
+    ang = torch.arange(t)[:, None].double() * torch.tensor([cfg.rope_theta ** (-2.0 * j / d) for j in range(d // 2)],
+                                                           dtype=torch.float64)
+    turn = torch.polar(torch.ones_like(ang), ang)[:, None, :]
+
+    def rotate(z):
+        zc = torch.complex(z[..., : d // 2].double(), z[..., d // 2:].double()) * turn
+        return torch.cat((zc.real, zc.imag), dim=-1).float()
+
+    out = F.scaled_dot_product_attention(rotate(q).transpose(0, 1), rotate(k).repeat_interleave(nh // nkv, dim=1).transpose(0, 1),
+                                         v.repeat_interleave(nh // nkv, dim=1).transpose(0, 1), is_causal=True).transpose(0, 1)
+    torch.testing.assert_close(got, out.reshape(t, -1) @ w["a.o_proj.weight"].T, rtol=1e-4, atol=1e-4)
 
 
 # ----------------------------------------------------------------------------------- attention
