@@ -111,6 +111,8 @@ class ModelPlan:
     tie_word_embeddings: bool
     max_position_embeddings: int
     eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+    embedding_multiplier: float | None = None  # the looked-up rows are multiplied by it (None: as they are)
+    logit_scale: float | None = None  # the logits are multiplied by it (None: as they are)
 
     def __post_init__(self) -> None:
         n = len(self.layers)

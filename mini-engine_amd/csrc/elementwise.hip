@@ -6,27 +6,27 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------- embedding
-// x[t, :] = table[ids[t], :] as float32. One block per token.
+// x[t, :] = table[ids[t], :] * scale as float32. One block per token.
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ ids,
-                             int hidden, int vocab) {
+                             int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // ids are validated on the host; never fault
   const T* row = table + (size_t)id * hidden;
   float* out = x + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_float(row[i]) * scale;
 }
 
-extern "C" int me_embed(void* x, const void* table, const int* ids, int num_tokens, int hidden, int vocab,
+extern "C" int me_embed(void* x, const void* table, const int* ids, int num_tokens, int hidden, int vocab, float scale,
                         int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (hidden <= 0 || vocab <= 0) return me_fail("me_embed: hidden=%d vocab=%d", hidden, vocab);
   const int threads = hidden >= 256 ? 256 : 64;
   if (dtype == ME_F32)
-    embed_kernel<float><<<num_tokens, threads, 0, stream>>>((float*)x, (const float*)table, ids, hidden, vocab);
+    embed_kernel<float><<<num_tokens, threads, 0, stream>>>((float*)x, (const float*)table, ids, hidden, vocab, scale);
   else
-    embed_kernel<bf16_t><<<num_tokens, threads, 0, stream>>>((float*)x, (const bf16_t*)table, ids, hidden, vocab);
+    embed_kernel<bf16_t><<<num_tokens, threads, 0, stream>>>((float*)x, (const bf16_t*)table, ids, hidden, vocab, scale);
   return me_check_launch("me_embed");
 }
 
@@ -36,28 +36,28 @@ extern "C" int me_embed(void* x, const void* table, const int* ids, int num_toke
 template <typename T>
 __global__ void embed_fed_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ ids,
                                  const int* __restrict__ fed_rows, const int* __restrict__ fed_tokens, int hidden,
-                                 int vocab) {
+                                 int vocab, float scale) {
   const int t = blockIdx.x;
   const int from = fed_rows[t];
   int id = from >= 0 ? fed_tokens[from] : ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* row = table + (size_t)id * hidden;
   float* out = x + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_float(row[i]) * scale;
 }
 
 extern "C" int me_embed_fed(void* x, const void* table, const int* ids, const int* fed_rows, const int* fed_tokens,
-                            int num_tokens, int hidden, int vocab, int dtype, hipStream_t stream) {
+                            int num_tokens, int hidden, int vocab, float scale, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (hidden <= 0 || vocab <= 0) return me_fail("me_embed_fed: hidden=%d vocab=%d", hidden, vocab);
   if (!fed_rows || !fed_tokens) return me_fail("me_embed_fed: no fed rows or tokens");
   const int threads = hidden >= 256 ? 256 : 64;
   if (dtype == ME_F32)
     embed_fed_kernel<float><<<num_tokens, threads, 0, stream>>>((float*)x, (const float*)table, ids, fed_rows, fed_tokens,
-                                                                hidden, vocab);
+                                                                hidden, vocab, scale);
   else
     embed_fed_kernel<bf16_t><<<num_tokens, threads, 0, stream>>>((float*)x, (const bf16_t*)table, ids, fed_rows, fed_tokens,
-                                                                 hidden, vocab);
+                                                                 hidden, vocab, scale);
   return me_check_launch("me_embed_fed");
 }
 
@@ -102,6 +102,18 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
     const float s = (adds && !write_x) ? sum_at(i) : xr[i];
     hr[i] = from_float<T>(s * inv * w[i]);
   }
+}
+
+// x *= scale over `count` float32 elements (a model's scale on its logits).
+__global__ void scale_kernel(float* __restrict__ x, float scale, size_t count) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) x[i] *= scale;
+}
+
+extern "C" int me_scale_f32(float* x, float scale, long long count, hipStream_t stream) {
+  if (count <= 0) return 0;
+  const size_t want = ((size_t)count + 255) / 256;
+  scale_kernel<<<(int)(want < 4096 ? want : 4096), 256, 0, stream>>>(x, scale, (size_t)count);
+  return me_check_launch("me_scale_f32");
 }
 
 // The residual add alone, for a norm that is not of this shape and runs as a part of its own:

@@ -151,9 +151,9 @@ class Run {
         const int table_dtype = dtype_;
         if (s_.fed && fed_tokens_)
           ok(me_embed_fed(x_, op.p[0], idx(s_.lay.token_ids), idx(s_.lay.token_source), fed_tokens_, t_, h_, prog_.vocab(),
-                          table_dtype, stream_));
+                          op.f[0], table_dtype, stream_));
         else
-          ok(me_embed(x_, op.p[0], idx(s_.lay.token_ids), t_, h_, prog_.vocab(), table_dtype, stream_));
+          ok(me_embed(x_, op.p[0], idx(s_.lay.token_ids), t_, h_, prog_.vocab(), op.f[0], table_dtype, stream_));
         pending_ = Pending();
         break;
       }
@@ -366,6 +366,7 @@ class Run {
       ok(me_gemm_bf16_small(picked, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], logits, rows, vocab, h_, 0, 0, kF32, 1, stream_));
     else
       library_product(picked, op.p[1], logits, rows, vocab, h_, kF32, stream_);
+    if (op.f[1] != 1.f) ok(me_scale_f32(logits, op.f[1], (long long)rows * vocab, stream_));
     result_.logits = logits;
   }
 

@@ -21,7 +21,7 @@
 namespace me {
 
 enum OpKind {
-  kOpEmbed = 0,       // p0 table; -> x
+  kOpEmbed = 0,       // p0 table, f0 the multiplier on the looked-up rows; -> x
   kOpNormLinear = 1,  // p0 norm weight, f0 eps, p1 W [rows, K], i0 rows of W, i1 K, i2 gated; pending + x -> out
   kOpNorm = 2,        // p0 norm weight, f0 eps; pending + x -> out [tokens, hidden]
   kOpLinear = 3,      // in, p1 W, i0 rows of W, i1 K, i2 gated -> out
@@ -30,7 +30,8 @@ enum OpKind {
   kOpAttention = 6,   // in qkv, p0 q-norm weight, p1 k-norm weight, p2 rotary table, p3 key pages, p4 value pages;
                       // i0 heads, i1 kv heads, i2 head size, i3 rotary size, i4 page size, i5 window, i6 writes pages,
                       // i7 cache group, i8 positions the table covers; f0 eps, f1 scale -> out [tokens, heads * head size]
-  kOpHead = 7,        // p0 final norm weight, f0 eps, p1 head W [vocab, hidden] -> logits of the wanted rows
+  kOpHead = 7,        // p0 final norm weight, f0 eps, p1 head W [vocab, hidden], f1 the scale on the logits -> logits of the
+                      // wanted rows
   kOpSample = 8,      // logits -> one token per wanted row
 };
 

@@ -8,9 +8,11 @@
 
 extern "C" {
 const char* me_last_error();
-int me_embed(void* x, const void* table, const int* ids, int num_tokens, int hidden, int vocab, int dtype, hipStream_t stream);
+int me_embed(void* x, const void* table, const int* ids, int num_tokens, int hidden, int vocab, float scale, int dtype,
+             hipStream_t stream);
 int me_embed_fed(void* x, const void* table, const int* ids, const int* fed_rows, const int* fed_tokens, int num_tokens,
-                 int hidden, int vocab, int dtype, hipStream_t stream);
+                 int hidden, int vocab, float scale, int dtype, hipStream_t stream);
+int me_scale_f32(float* x, float scale, long long count, hipStream_t stream);
 int me_add_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, const float* w,
                    void* h, const int* rows, int num_rows, int dim, float eps, int write_x, int dtype, hipStream_t stream);
 int me_rmsnorm(const void* in, const float* w, void* out, int num_rows, int dim, float eps, int dtype, hipStream_t stream);

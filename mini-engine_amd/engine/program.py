@@ -149,9 +149,10 @@ class StepProgram:
         fv = (ctypes.c_float * 2)(*[float(v) for v in floats])
         self.num_ops = _ok(self._L.me_runner_op(self.handle, kind, in_, out, p, iv, fv))
 
-    def embed(self, table: torch.Tensor) -> None:
+    def embed(self, table: torch.Tensor, multiplier: float = 1.0) -> None:
+        """The residual stream starts as the tokens' rows of ``table``, times ``multiplier``."""
         self._want(table, self.dtype, (self.vocab, self.hidden), "embedding table")
-        self.op(EMBED, ptrs=[table])
+        self.op(EMBED, ptrs=[table], floats=[multiplier])
 
     def normed(self, norm) -> Normed:
         """The add-and-norm before a part, for a norm that is RMS-shaped (``norm.as_fused()`` gives its
@@ -217,10 +218,11 @@ class StepProgram:
                 floats=[eps, scale])
         return out
 
-    def head(self, norm, weight: torch.Tensor) -> None:
+    def head(self, norm, weight: torch.Tensor, logit_scale: float = 1.0) -> None:
+        """Final norm of the wanted rows, the head product, the logits times ``logit_scale``."""
         norm_weight, eps = norm.as_fused()
         self._want(weight, self.dtype, (self.vocab, self.hidden), "head")
-        self.op(HEAD, ptrs=[norm_weight, weight], floats=[eps])
+        self.op(HEAD, ptrs=[norm_weight, weight], floats=[eps, logit_scale])
         self.pending_consumed()
 
     def sample(self) -> None:

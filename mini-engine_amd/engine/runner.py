@@ -63,6 +63,7 @@ class ModelRunner:
                 self.memory = StepMemory(program, self.device, [self.max_blocks_per_seq] * self.num_groups,
                                          self.storage.spare_block, self.storage.spare_slot)
         self.sampler = Sampler()
+        self.graph_safe = decoder.graph_safe()  # every part can be captured: decode steps may replay graphs
         self._graphs: dict[int, tuple] = {}
         self._graph_pool = None
         self._static_arena: torch.Tensor | None = None
@@ -101,12 +102,13 @@ class ModelRunner:
         """Run the step that the core holds (planned by the scheduler or listed by :meth:`step`)."""
         core = self.core
         tokens, items, rows, longest, ctx, decode_only, last_only, _ = (int(v) for v in core.step_summary())
-        replay = bool(self.config.cuda_graphs and not self.layout.has_state and decode_only and last_only
+        replay = bool(self.config.cuda_graphs and self.graph_safe and decode_only and last_only
                       and 0 < items <= self.config.max_num_seqs)
         self._drawn = None
         if replay:
             # a replayed step checks the pages of its block tables while they are written into the graph's buffer
             core.step_check(self.decoder.plan.vocab_size, scan_pages=False)
+            self._zero_fresh_state()
             return self._replay(items)
         self.eager_steps += 1
         if self.program is not None:  # one call: check, pack, upload, every kernel, the draw
@@ -118,12 +120,16 @@ class ModelRunner:
                 self._logits = torch.empty((0, self.decoder.plan.vocab_size), dtype=torch.float32, device=self.device)
             return self._logits
         core.step_check(self.decoder.plan.vocab_size, scan_pages=True)
-        if self.layout.has_state:
-            _, starts, _, _, slots = core.step_items()
-            self.storage.zero_state([s for s, p0 in zip(slots, starts) if p0 == 0 and s >= 0])
+        self._zero_fresh_state()
         self.batch = batch_from_core(core, self.device, self.storage.spare_block, self.storage.spare_slot)
         self._logits = self.decoder.forward(self.batch)
         return self._logits
+
+    def _zero_fresh_state(self) -> None:
+        """An item that starts at position 0 starts from a zero state, whoever held its slot before."""
+        if self.layout.has_state:
+            _, starts, _, _, slots = self.core.step_items()
+            self.storage.zero_state([s for s, p0 in zip(slots, starts) if p0 == 0 and s >= 0])
 
     def draw(self, rows: int, tempered: bool):
         """One token id per wanted row of the last step (int32, on the host): what the native program

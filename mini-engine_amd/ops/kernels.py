@@ -68,16 +68,23 @@ def _want(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: t
 # ------------------------------------------------------------------------------------ row-wise ops
 
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """``out[t] = float32(table[ids[t]])``; ids int32 [T], table [V, H]."""
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None, multiplier: float = 1.0) -> torch.Tensor:
+    """``out[t] = float32(table[ids[t]]) * multiplier``; ids int32 [T], table [V, H]."""
     _want(ids, "ids", torch.int32)
     _want(table, "table", None, (None, None))
     t, (v, h) = ids.numel(), table.shape
     if out is None:
         out = torch.empty((t, h), dtype=torch.float32, device=table.device)
     _want(out, "out", torch.float32, (t, h))
-    check(lib().me_embed(_p(out), _p(table), _p(ids), _i(t), _i(h), _i(v), _i(_code(table.dtype)), _stream()))
+    check(lib().me_embed(_p(out), _p(table), _p(ids), _i(t), _i(h), _i(v), _f(multiplier), _i(_code(table.dtype)), _stream()))
     return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x *= factor`` in place, float32 of any shape."""
+    _want(x, "x", torch.float32)
+    check(lib().me_scale_f32(_p(x), _f(factor), ctypes.c_longlong(x.numel()), _stream()))
+    return x
 
 
 class PartialSums:

@@ -23,6 +23,8 @@ MAX_HEAD_DIM = 256
 
 
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         s = spec

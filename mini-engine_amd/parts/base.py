@@ -17,6 +17,10 @@ A mixer or feed-forward class may set ``takes_normed_input = True``; its ``forwa
 to ``ops.kernels.linear`` as the input of its first matrix product, which fuses both into that
 product for decode-sized batches (``h.materialize()`` gives the tensor where it is needed).
 
+A part class that sets ``graph_safe = True`` promises that its ``forward`` can be captured into a graph for
+decode steps (see :class:`Part`); rows that pad a replayed batch carry the spare page and the spare state
+slot, which belong to no request.
+
 ``h`` is the normed input [T, hidden] in the compute dtype, ``batch`` a ``StepBatch`` (token
 positions, item boundaries, block tables per cache group, state slots), ``cache`` the binding
 (``KVBinding`` / ``StateBinding`` / None) of this run of the layer: a layer that the order names
@@ -69,6 +73,13 @@ class StateBinding:
 
 
 class Part:
+    # Whether the part's ``forward`` may run inside a graph capture of a decode step (every item one token)
+    # and be replayed with other indices: it reads positions, state slots and block tables from the batch's
+    # device tensors only (never from ``batch.starts`` / ``qlens`` / ``slots_host``, which a replay does not
+    # update), does not wait for the device and allocates nothing but torch tensors. Parts defined outside
+    # the package say so themselves; a model with a part that does not is stepped without graphs.
+    graph_safe = False
+
     def __init__(self, spec: Any, dtype: torch.dtype, device: torch.device):
         self.spec, self.dtype, self.device = spec, dtype, device
 

@@ -86,7 +86,7 @@ class Decoder:
         ``batch.want_rows``."""
         if self.embed_table is None:
             raise RuntimeError("weights are not loaded")
-        x = K.embed(batch.token_ids, self.embed_table)
+        x = K.embed(batch.token_ids, self.embed_table, multiplier=self.plan.embedding_multiplier or 1.0)
         spare = torch.empty_like(x)  # the residual stream alternates between two buffers
         pending = None
         for r, i in enumerate(self.plan.order):
@@ -101,10 +101,10 @@ class Decoder:
             raise RuntimeError("weights are not loaded")
         if not all(self.blocks[i].can_emit() for i in set(self.plan.order)) or self.final_norm.as_fused() is None:
             return False
-        program.embed(self.embed_table)
+        program.embed(self.embed_table, self.plan.embedding_multiplier or 1.0)
         for r, i in enumerate(self.plan.order):
             self.blocks[i].emit(program, self.bindings[r])
-        program.head(self.final_norm, self.head)
+        program.head(self.final_norm, self.head, self.plan.logit_scale or 1.0)
         program.sample()
         return True
 
@@ -118,4 +118,16 @@ class Decoder:
             if pending is not None:
                 K.residual_add(x, pending)
             h = self.final_norm.forward(x.index_select(0, rows.long()))
-        return K.linear(h, self.head, torch.float32)
+        logits = K.linear(h, self.head, torch.float32)
+        if self.plan.logit_scale not in (None, 1.0):
+            K.scale_(logits, self.plan.logit_scale)
+        return logits
+
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be captured into a graph: every part says so
+        (``graph_safe`` of :class:`~mini_engine_amd.parts.base.Part`)."""
+        parts = [self.final_norm]
+        for i in set(self.plan.order):
+            b = self.blocks[i]
+            parts += [b.mixer, b.ffn, b.mixer_norm, b.ffn_norm]
+        return all(getattr(p, "graph_safe", False) for p in parts)

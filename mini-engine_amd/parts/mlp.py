@@ -12,6 +12,8 @@ from .base import FEED_FORWARDS, FeedForward
 
 
 class GatedMlp(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.activation != "silu":

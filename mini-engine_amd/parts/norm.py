@@ -11,6 +11,8 @@ from .base import NORMS, Norm
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         self.eps = float(spec.eps)
