@@ -19,7 +19,6 @@ import argparse
 import json
 import os
 import sys
-import tempfile
 
 import numpy as np
 
@@ -105,31 +104,6 @@ class TraceSession:
         return out
 
 
-def random_model_folder(spec: str, seed: int, dtype: str) -> str:
-    """Write a model folder with seeded random weights for ``ARCHITECTURE:key=value,...`` (the keys of
-    that architecture's config.json) into a temporary folder and return its path."""
-    import torch
-
-    from .. import models as _models  # noqa: F401
-    from ..config.registry import get_architecture
-    from ..parts.decoder import Decoder
-    from ..weights import write_model_folder
-
-    name, _, rest = spec.partition(":")
-    values: dict = {}
-    for pair in filter(None, rest.split(",")):
-        key, _, value = pair.partition("=")
-        values[key.strip()] = json.loads(value) if value.strip() not in ("True", "False") else value.strip() == "True"
-    values.setdefault("architectures", [name])
-    entry = get_architecture(name)
-    arch_config = entry.config_from_dict(values)
-    folder = tempfile.mkdtemp(prefix="trace_model_")
-    wants = Decoder(entry.plan_from_config(arch_config), torch.float32, "cpu").weight_wants()
-    write_model_folder(folder, arch_config.to_config_json(), wants, seed=seed,
-                       dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
-    return folder
-
-
 def main(argv: list[str] | None = None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
     src = ap.add_mutually_exclusive_group(required=True)
@@ -150,6 +124,8 @@ def main(argv: list[str] | None = None) -> int:
         ap.error("one of --max-tokens and --num-blocks is needed")
     os.makedirs(args.out, exist_ok=True)
     print("[trace_run] loading kernels and model", file=sys.stderr, flush=True)
+    from ..weights.random_init import random_model_folder
+
     model_dir = args.model or random_model_folder(args.random_shape, args.seed, args.dtype)
     session = TraceSession(build_session(model_dir, args.dtype, args.max_tokens or 0, args.block_size, args.max_live,
                                          num_blocks=args.num_blocks))

@@ -80,6 +80,22 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = Non
     return out
 
 
+def probe_read(buf: torch.Tensor, out: torch.Tensor) -> None:
+    """Launch the kernel that streams ``buf`` (a multiple of 16 bytes) once; ``out`` is one int32 word
+    it may write. For measuring the memory rate a kernel reaches on this GPU."""
+    nbytes = buf.numel() * buf.element_size()
+    _want(out, "out", torch.int32)
+    check(lib().me_probe_read(_p(buf), ctypes.c_longlong(nbytes), _p(out), _stream()))
+
+
+def probe_mfma(blocks: int, iterations: int, out: torch.Tensor) -> float:
+    """Launch the kernel that issues bfloat16 16x16x32 matrix-core products from registers; returns
+    the floating-point operations of the launch. ``out`` is one float32 word it may write."""
+    _want(out, "out", torch.float32)
+    check(lib().me_probe_mfma(_i(blocks), _i(iterations), _p(out), _stream()))
+    return blocks * 4 * 4 * iterations * 2.0 * 16 * 16 * 32
+
+
 def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
     """``x *= factor`` in place, float32 of any shape."""
     _want(x, "x", torch.float32)

@@ -1,5 +1,5 @@
 from .loader import FolderSource, TensorWant, WeightError, check_names_and_shapes, load_tensors
-from .random_init import RandomSource, write_model_folder
+from .random_init import RandomSource, parse_shape, random_model_folder, write_model_folder
 from .safetensors_io import read_folder_header, read_header, write_file
 
 __all__ = [
@@ -9,6 +9,8 @@ __all__ = [
     "WeightError",
     "check_names_and_shapes",
     "load_tensors",
+    "parse_shape",
+    "random_model_folder",
     "read_folder_header",
     "read_header",
     "write_file",

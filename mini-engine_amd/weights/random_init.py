@@ -63,3 +63,43 @@ def write_model_folder(
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(config_json, f, indent=1)
     write_file(os.path.join(folder, "model.safetensors"), tensors, {"format": "pt", "seed": str(seed)})
+
+
+def parse_shape(spec: str) -> tuple[str, dict]:
+    """``ARCHITECTURE:key=value,...`` -> (architecture name, config.json keys); values are JSON
+    (``true``/``false`` also capitalised)."""
+    name, _, rest = spec.partition(":")
+    values: dict = {}
+    for pair in filter(None, rest.split(",")):
+        key, eq, value = pair.partition("=")
+        if not eq or not key.strip():
+            raise ValueError(f"{pair!r}: key=value expected")
+        text = value.strip()
+        values[key.strip()] = json.loads(text.lower() if text in ("True", "False") else text)
+    if not name.strip():
+        raise ValueError("a shape starts with the architecture's name")
+    values.setdefault("architectures", [name.strip()])
+    return name.strip(), values
+
+
+def random_model_folder(spec: str, seed: int, dtype: str, std: float = 0.02) -> str:
+    """Write a model folder with seeded random weights for ``ARCHITECTURE:key=value,...`` (the keys of
+    that architecture's config.json) into a temporary folder, which is removed when the process ends,
+    and return its path."""
+    import atexit
+    import shutil
+    import tempfile
+
+    from .. import models as _models  # noqa: F401  (registers the architectures)
+    from ..config.registry import get_architecture
+    from ..parts.decoder import Decoder
+
+    name, values = parse_shape(spec)
+    entry = get_architecture(name)
+    arch_config = entry.config_from_dict(values)
+    folder = tempfile.mkdtemp(prefix="random_model_")
+    atexit.register(shutil.rmtree, folder, True)
+    wants = Decoder(entry.plan_from_config(arch_config), torch.float32, "cpu").weight_wants()
+    write_model_folder(folder, arch_config.to_config_json(), wants, seed=seed,
+                       dtype=torch.float32 if dtype == "float32" else torch.bfloat16, std=std)
+    return folder

@@ -295,3 +295,26 @@ def test_command_line(peaked):
     lines = [l for l in proc.stdout.splitlines() if l.startswith("A: ")]
     assert lines[0] == "A: " + " ".join(map(str, plain.greedy_generate(w, pcfg, [5, 6, 7, 8, 9], 6)))
     assert "tokens in" in proc.stdout and "served from prefix cache" in proc.stdout
+
+
+def test_command_line_with_a_random_shape_and_random_prompts():
+    """``--random ARCH:keys --seed`` stands for a model folder and ``--random-prompts NxLEN`` for prompts:
+    the same seed gives the same text twice, another seed another, and the shared half of the prompts
+    is served from the prefix cache."""
+    shape = ("Qwen3ForCausalLM:vocab_size=211,hidden_size=48,intermediate_size=80,num_hidden_layers=2,num_attention_heads=3,"
+             "num_key_value_heads=1,head_dim=16,rms_norm_eps=1e-6,rope_theta=10000.0,max_position_embeddings=256,"
+             "tie_word_embeddings=true")
+
+    def run(seed):
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "examples", "generate.py"), "--random", shape, "--seed", str(seed),
+                               "--random-prompts", "4x40", "--max-tokens", "5", "--dtype", "float32", "--block-size", "8"],
+                              capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        return proc.stdout
+
+    first = run(3)
+    answers = [l for l in first.splitlines() if l.startswith("A: ")]
+    assert len(answers) == 4 and all(len(a.split()) == 6 for a in answers)
+    assert "served from prefix cache 48" in first  # 20 shared ids: two full pages of 8, three times
+    assert [l for l in run(3).splitlines() if l.startswith("A: ")] == answers
+    assert [l for l in run(4).splitlines() if l.startswith("A: ")] != answers

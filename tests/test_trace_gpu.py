@@ -153,3 +153,36 @@ def test_trace_run_program(tiny_folders, tmp_path):
                                            f"program {dtype} step {s['step']} {e['id']}")
                     r += 1
                 fed[e["id"]] += len(e["tokens"])
+
+
+def test_trace_run_program_with_a_shape_and_a_seed(tmp_path):
+    """``--random-shape ARCH:keys --seed`` stands for ``--model``, ``--block-size`` and ``--num-blocks``
+    size the pool: Tiny B (pages of 8) replayed from the command line, mixed, in a pool of 40 pages."""
+    from mini_engine_amd.weights import random_model_folder
+
+    cfg = tiny_configs()["B"]
+    keys = cfg.to_config_json()
+    shape = "Qwen3ForCausalLM:" + ",".join(
+        f"{k}={json.dumps(keys[k])}" for k in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers",
+                                               "num_attention_heads", "num_key_value_heads", "head_dim", "rms_norm_eps",
+                                               "rope_theta", "max_position_embeddings", "tie_word_embeddings"))
+    reqs = {k: v for k, v in list(requests_for("B").items())[:5]}
+    steps = th.mixed(reqs, 320, seed=2)
+    want = th.plain_logits(random_model_folder(shape, 13, "float32"), reqs)
+    out_dir = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--random-shape", shape, "--seed", "13", "--dtype", "float32",
+         "--out", str(out_dir), "--block-size", "8", "--num-blocks", "40"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    fed = {rid: 0 for rid in reqs}
+    for s in steps:
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        got = torch.from_numpy(np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(wanted, cfg.vocab_size))
+        r = 0
+        for e in s["entries"]:
+            n = len(e["tokens"])
+            th.assert_logits_close(got[r : r + n], want[e["id"]][fed[e["id"]] : fed[e["id"]] + n], "float32",
+                                   f"step {s['step']} {e['id']}")
+            r += n
+            fed[e["id"]] += n
