@@ -1,6 +1,8 @@
 // Running a step program: the choice of kernel per operation and step size, and the launches.
 #include "program.h"
 
+#include <hip/hip_runtime_api.h>
+
 #include <algorithm>
 #include <mutex>
 #include <set>
@@ -17,6 +19,8 @@ constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
 constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
 constexpr int kTiledMinRows = 256;
 constexpr int kDecodeWaves = 1024;  // waves that a decode attention launch aims at (four per compute unit of 256)
+constexpr int64_t kStreamMinElements = 8ll << 20;  // weights from 16 MiB on: streaming them is the product's time
+constexpr int64_t kStreamMaxBytes = 1ll << 31;     // what the weight-streaming kernel addresses
 
 void ok(int code) {
   if (code) throw Error(kBadState, me_last_error());
@@ -52,6 +56,30 @@ bool small_serves(int m, int rows_of_w, int k, bool gated) {
   if (k % 8) return false;
   if (m <= kSmallFastRows) return true;
   return m <= kSmallMaxRows && (gated || (rows_of_w >= 2048 && rows_of_w <= 16384));
+}
+
+// Whether a product of up to 64 rows is bound by streaming its weight: the layers of wide models. Their
+// deltas go to the weight-streaming kernel with k cut into runs (measured at 4,096 and 5,120 columns, k of 4,096
+// to 25,600: 8.7-29 us and 21-80 us against 9.4-65 and 27-245 with the small kernel, 10-38 and 20-156 with
+// the library); their other products go to the same kernel up to 16 rows (qkv and gate/up 14.7-43 and 24-117 us
+// against 15-51 and 26-139 with the small kernel) and to the library from 17 to 64 rows (qkv 15-33 us against
+// 21-56 with the streaming kernel, whose time grows with the rows). The norm before such a product is a kernel
+// of its own: the partial sums it adds up are read once, not by every block of a product.
+bool weight_bound(int m, int rows_of_w, int k) {
+  const int64_t elements = (int64_t)rows_of_w * k;
+  return m <= kSmallMaxRows && k % 8 == 0 && elements >= kStreamMinElements && elements * 2 < kStreamMaxBytes;
+}
+
+int compute_units() {
+  static int units = 0;
+  if (!units) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      units = n;
+    else
+      units = 256;
+  }
+  return units;
 }
 
 // Into how many runs of k a product of 17 to 64 rows with few output columns is cut (1: not at all): a block
@@ -210,7 +238,7 @@ class Run {
     const int n = gated ? rows_of_w / 2 : rows_of_w;
     // decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
     // residual buffer, since other blocks of the kernel still read the first
-    if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts) {
+    if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts && !weight_bound(t_, rows_of_w, k)) {
       ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
                             bufs_[op.out], t_, n, k, 1, gated ? 1 : 0, dtype_, 1, stream_));
       if (pending_.delta) std::swap(x_, spare_);
@@ -235,7 +263,13 @@ class Run {
       ok(me_swiglu(both, out, m, n, kF32, stream_));
       return;
     }
-    if (small_serves(m, rows_of_w, k, gated)) {
+    const bool heavy = weight_bound(m, rows_of_w, k);
+    if (heavy && m <= kSmallFastRows && (out_dtype == kBF16 || !gated)) {  // up to 16 rows it is ahead of the library too
+      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated ? 1 : 0, out_dtype, 1, compute_units(), stream_));
+      return;
+    }
+    const bool to_library = heavy && m > kSmallFastRows;
+    if (!to_library && small_serves(m, rows_of_w, k, gated)) {
       ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, out, m, n, k, 0, gated ? 1 : 0, out_dtype, 1, stream_));
       return;
     }
@@ -258,6 +292,21 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
+    if (dtype_ == kBF16 && weight_bound(t_, n, k)) {
+      const int splits = me_gemm_bf16_stream_splits(n, k, compute_units());
+      if (splits > 1) {
+        parts_mark_ = arena_.used;
+        float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);
+        ok(me_gemm_bf16_stream(x, op.p[1], parts, t_, n, k, 0, kF32, splits, compute_units(), stream_));
+        pending_.parts = parts;
+        pending_.num_parts = splits;
+        pending_.stride = (long long)t_ * n;
+        return;
+      }
+      ok(me_gemm_bf16_stream(x, op.p[1], bufs_[op.out], t_, n, k, 0, kBF16, 1, compute_units(), stream_));
+      pending_.delta = bufs_[op.out];
+      return;
+    }
     if (dtype_ == kBF16 && !small_serves(t_, n, k, false)) {
       const int splits = delta_splits(t_, n, k);
       if (splits > 1) {  // partial sums over runs of k, each by blocks of its own; the next norm adds them up
@@ -425,7 +474,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
   for (const Op& op : ops_) {
     size_t need = 0;
     if (op.kind == kOpNormLinear || op.kind == kOpLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
-    if (op.kind == kOpLinearDelta) need = (size_t)8 * std::min<int64_t>(tokens, kSmallMaxRows) * op.i[0] * 4 + pad;
+    if (op.kind == kOpLinearDelta) need = (size_t)16 * std::min<int64_t>(tokens, kSmallMaxRows) * op.i[0] * 4 + pad;
     if (op.kind == kOpAttention) {
       const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
       const int chunks = (nh / nkv + 15) / 16;
@@ -444,7 +493,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
   const size_t tail = (size_t)rows * hidden_ * elem + (size_t)rows * vocab_ * 4 + (size_t)rows * 4 +
                       (size_t)rows * me_sample_chunks(vocab_) * 8 + 4 * pad;
   // partial sums of the last delta wait beside the head's buffers
-  return fixed + 2 * scratch + tail + (size_t)8 * kSmallMaxRows * hidden_ * 4 + (1 << 16);
+  return fixed + 2 * scratch + tail + (size_t)16 * kSmallMaxRows * hidden_ * 4 + (1 << 16);
 }
 
 }  // namespace me

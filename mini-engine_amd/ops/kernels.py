@@ -354,13 +354,51 @@ class NormedInput:
         return self._tensor
 
     def fusable(self, weight: torch.Tensor) -> bool:
+        """Whether add, norm and the product with ``weight`` go into one kernel: decode-sized steps whose
+        delta is a tensor (partial sums are read once, by the add-and-norm kernel, not by every block of a
+        product) and whose weight is not so large that the weight-streaming kernel serves it."""
         return (self.dtype is torch.bfloat16 and self._tensor is None and self.x.shape[0] <= SMALL_FAST_ROWS
                 and self.x.shape[1] % 8 == 0 and (self.delta is None or self.spare is not None)
-                and weight.dtype is torch.bfloat16)
+                and not isinstance(self.delta, PartialSums) and weight.dtype is torch.bfloat16
+                and weight.numel() < STREAM_MIN_ELEMENTS)
 
 
 SMALL_MAX_ROWS = 64  # what the kernel accepts
 SMALL_FAST_ROWS = 16  # up to here it beats the GEMM library on every shape, with the norm as its prologue too
+
+
+def compute_units(device=None) -> int:
+    return torch.cuda.get_device_properties(device or torch.cuda.current_device()).multi_processor_count
+
+
+def stream_splits(n: int, k: int, device=None) -> int:
+    """Into how many runs of k :func:`gemm_bf16_stream` cuts a product whose result may stay partial sums."""
+    return int(lib().me_gemm_bf16_stream_splits(_i(n), _i(k), _i(compute_units(device))))
+
+
+def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
+                     out: torch.Tensor | None = None, k_splits: int = 1) -> torch.Tensor:
+    """bfloat16 ``x @ weight.T`` for at most 64 rows and weights large enough that streaming them is the
+    kernel's time: x is staged in LDS once per block of columns, the weight goes straight to the matrix
+    cores. ``swiglu`` and ``k_splits`` as in :func:`gemm_bf16_small` (``k_splits`` as :func:`stream_splits`
+    gives it, or 1)."""
+    _want(x, "x", torch.bfloat16, (None, None))
+    m, k = x.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0]
+    if swiglu:
+        if n % 2:
+            raise ValueError(f"a gate/up weight needs an even number of rows, got {n}")
+        n //= 2
+    if m > SMALL_MAX_ROWS:
+        raise ValueError(f"gemm_bf16_stream takes at most {SMALL_MAX_ROWS} rows, got {m}")
+    shape = (k_splits, m, n) if k_splits > 1 else (m, n)
+    if out is None:
+        out = torch.empty(shape, dtype=out_dtype, device=weight.device)
+    _want(out, "out", out_dtype, shape)
+    check(lib().me_gemm_bf16_stream(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(1 if swiglu else 0),
+                                    _i(_code(out_dtype)), _i(k_splits), _i(compute_units(x.device)), _stream()))
+    return out
 
 
 def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
@@ -463,6 +501,18 @@ def small_ok(x, weight: torch.Tensor, gated: bool = False) -> bool:
     return x.shape[0] <= SMALL_MAX_ROWS and (gated or 2048 <= weight.shape[0] <= 16384)
 
 
+STREAM_MIN_ELEMENTS = 8 << 20  # weights from 16 MiB on: streaming them is the product's time
+STREAM_MAX_BYTES = 1 << 31  # what the weight-streaming kernel addresses
+
+
+def weight_bound(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether a product of up to 64 rows is bound by streaming its weight (the layers of wide models): their
+    deltas go to the weight-streaming kernel with k cut into runs, their other products of 17 to 64 rows to
+    the library (the same rule as ``csrc/host/program.cpp``, where the measurements are)."""
+    return (x.shape[0] <= SMALL_MAX_ROWS and x.shape[1] % 8 == 0 and STREAM_MIN_ELEMENTS <= weight.numel()
+            and weight.numel() * 2 < STREAM_MAX_BYTES and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
 def delta_splits(rows: int, n: int, k: int) -> int:
     """Into how many runs of k a product of 17 to 64 rows with few output columns is cut (1: not at all):
     a block per 16 columns leaves most of the chip idle and makes each block read all of x, so k is
@@ -495,7 +545,15 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
             raise TypeError("the float32 path keeps float32 results")
         y = gemm_f32(x, weight)
         return swiglu(y) if gated else y
-    if small_ok(x, weight, gated):
+    heavy = weight_bound(x, weight)
+    if heavy and as_delta and not gated:
+        splits = stream_splits(weight.shape[0], x.shape[1], x.device)
+        if splits > 1:
+            return PartialSums(gemm_bf16_stream(x, weight, torch.float32, k_splits=splits))
+        return gemm_bf16_stream(x, weight, out_dtype)
+    if heavy and x.shape[0] <= SMALL_FAST_ROWS and (out_dtype is torch.bfloat16 or not gated):
+        return gemm_bf16_stream(x, weight, out_dtype, gated)
+    if small_ok(x, weight, gated) and not heavy:
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if as_delta and not gated and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0:
         splits = delta_splits(x.shape[0], weight.shape[0], x.shape[1])

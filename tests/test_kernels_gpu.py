@@ -235,6 +235,50 @@ def test_gemm_bf16_small_with_very_many_columns(m, n, k):
         assert (got - want).abs().max().item() <= tol_abs, (out_dtype, (got - want).abs().max().item(), scale)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 16, 128), (7, 100, 72), (16, 1040, 1000), (17, 4099, 1536), (33, 200, 2056), (48, 68, 8200),
+                                   (64, 9000, 648), (64, 40, 136)])
+@pytest.mark.parametrize("gated", [True, False])
+def test_gemm_bf16_stream(m, n, k, gated):
+    """The weight-streaming product at every row-tile count, with column counts that are no multiple of a
+    block's (every arrangement of a block's waves: many, some and few columns), k that is no multiple of a
+    step, both output types, the gated form, and partial sums over runs of k whose sum is the product."""
+    g = torch.Generator().manual_seed(m * 977 + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
+    w[n - 1] *= 4  # the last column stands out: a tile that stops short of it, or runs past it, shows
+    y = x.float() @ w.float().T
+    want = plain.silu(y[:, :n]) * y[:, n:] if gated else y
+    scale = max(1.0, want.abs().max().item())
+    got = K().gemm_bf16_stream(dev(x), dev(w), torch.bfloat16, gated).float().cpu()
+    assert (got - want).abs().max().item() <= 2**-7 * scale
+    if gated:
+        return
+    got = K().gemm_bf16_stream(dev(x), dev(w), torch.float32).cpu()
+    assert (got - want).abs().max().item() <= 1e-4 * scale
+    steps = -(-k // 128)
+    for splits in sorted({K().stream_splits(n, k), 2, 3, min(steps, 64)} - {1}):
+        if steps < splits or -(-steps // -(-steps // splits)) != splits:
+            continue  # runs are whole steps, none of them empty
+        parts = K().gemm_bf16_stream(dev(x), dev(w), torch.float32, k_splits=splits).cpu()
+        assert parts.shape == (splits, m, n)
+        assert (parts.sum(0) - want).abs().max().item() <= 1e-4 * scale
+        assert parts[-1].abs().max() > 0
+
+
+def test_gemm_bf16_stream_refuses_what_it_cannot_do():
+    x, w = dev(torch.zeros(65, 64).bfloat16()), dev(torch.zeros(32, 64).bfloat16())
+    with pytest.raises(ValueError):
+        K().gemm_bf16_stream(x, w)
+    x = dev(torch.zeros(4, 68).bfloat16())
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        K().gemm_bf16_stream(x, dev(torch.zeros(32, 68).bfloat16()))
+    x = dev(torch.zeros(4, 256).bfloat16())
+    with pytest.raises(RuntimeError, match="runs of whole steps"):
+        K().gemm_bf16_stream(x, dev(torch.zeros(32, 256).bfloat16()), torch.float32, k_splits=3)
+    with pytest.raises(RuntimeError, match="plain float32"):
+        K().gemm_bf16_stream(x, dev(torch.zeros(32, 256).bfloat16()), torch.bfloat16, k_splits=2)
+
+
 def test_normed_input_falls_back_to_the_separate_kernels():
     """More than 64 rows or float32: the add-and-norm kernel runs, in place, and the product follows."""
     for dtype, m in ((torch.bfloat16, 100), (torch.float32, 5)):
