@@ -11,6 +11,7 @@
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <initializer_list>
 #include <mutex>
 #include <unordered_map>
 
@@ -23,7 +24,10 @@ struct LibraryPlan {
   size_t workspace = 0;
 };
 
-constexpr size_t WORKSPACE_BYTES = 32u << 20;  // the most a product may ask for; allocated once
+constexpr size_t WORKSPACE_BYTES = 256u << 20;  // the most a product may ask for (the library's split-k kernels for
+                                                // products of thousands of rows want tens of MB); allocated once
+constexpr int MAX_CANDIDATES = 8;               // algorithms asked of the heuristic: the first whose workspace fits is taken
+constexpr size_t MAX_PLANS = 2048;              // per output type; a serving loop's steps bring ever new row counts
 
 std::mutex g_mutex;
 hipblasLtHandle_t g_handle = nullptr;
@@ -45,23 +49,34 @@ int make_plan(LibraryPlan& p, int M, int N, int K, int out_dtype) {
     return me_fail("me_gemm_bf16_library: no preference object");
   size_t most = WORKSPACE_BYTES;
   hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &most, sizeof(most));
-  hipblasLtMatmulHeuristicResult_t result;
+  hipblasLtMatmulHeuristicResult_t results[MAX_CANDIDATES];
   int found = 0;
-  const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, 1, &result, &found);
+  const hipblasStatus_t st =
+      hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, MAX_CANDIDATES, results, &found);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (st != HIPBLAS_STATUS_SUCCESS || found < 1)
     return me_fail("me_gemm_bf16_library: the library has no algorithm for a %d x %d x %d product (status %d)", M, N, K, (int)st);
-  if (result.workspaceSize > WORKSPACE_BYTES)
-    return me_fail("me_gemm_bf16_library: the algorithm wants %zu bytes of workspace", result.workspaceSize);
-  p.algo = result.algo;
-  p.workspace = result.workspaceSize;
-  return 0;
+  for (int i = 0; i < found; ++i)
+    if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= WORKSPACE_BYTES) {
+      p.algo = results[i].algo;
+      p.workspace = results[i].workspaceSize;
+      return 0;
+    }
+  return me_fail("me_gemm_bf16_library: every algorithm for a %d x %d x %d product wants more than %zu bytes of workspace", M, N,
+                 K, WORKSPACE_BYTES);
+}
+
+void destroy_plan(LibraryPlan& p) {
+  if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+  for (hipblasLtMatrixLayout_t l : {p.a, p.b, p.c})
+    if (l) hipblasLtMatrixLayoutDestroy(l);
+  p = LibraryPlan();
 }
 
 }  // namespace
 
 // X [M, K] and W [N, K] bfloat16, C [M, N] bfloat16 or float32 (out_dtype), all contiguous. The first call
-// creates the library's handle and a workspace of 32 MB that lives as long as the process; the first call
+// creates the library's handle and a workspace of 256 MB that lives as long as the process; the first call
 // for a shape must not come while a graph is being captured (it may load code), later ones may.
 extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype,
                                     hipStream_t stream) {
@@ -88,8 +103,15 @@ extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M
     const uint64_t key = ((uint64_t)(uint32_t)M << 42) ^ ((uint64_t)(uint32_t)N << 21) ^ (uint64_t)(uint32_t)K;
     auto it = plans.find(key);
     if (it == plans.end()) {
+      if (plans.size() >= MAX_PLANS) {  // start over: the shapes in use come back within a few steps
+        for (auto& kv : plans) destroy_plan(kv.second);
+        plans.clear();
+      }
       LibraryPlan fresh;
-      if (make_plan(fresh, M, N, K, out_dtype)) return 1;
+      if (make_plan(fresh, M, N, K, out_dtype)) {
+        destroy_plan(fresh);
+        return 1;
+      }
       it = plans.emplace(key, fresh).first;
     }
     plan = it->second;

@@ -107,7 +107,11 @@ void library_product(const void* x, const void* w, void* out, int m, int n, int 
     std::lock_guard<std::mutex> hold(g_refused_mutex);
     g_refused.insert(shape);
   }
-  if (k % 8 == 0) {  // slices of 64 rows through the matrix-core kernel
+  if (k % 64 == 0 && m > kSmallMaxRows && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {  // the tiled matrix-core kernel of this folder
+    ok(me_gemm_bf16_tiled(x, w, out, m, n, k, 0, out_dtype, 0, stream));
+    return;
+  }
+  if (k % 8 == 0) {  // slices of 64 rows through the small matrix-core kernel
     const size_t out_elem = out_dtype == kF32 ? 4 : 2;
     for (int lo = 0; lo < m; lo += kSmallMaxRows) {
       const int rows = std::min(kSmallMaxRows, m - lo);

@@ -163,6 +163,27 @@ def test_small_gemm_partial_sums_and_their_add_rmsnorm(m, n, k, splits):
     torch.testing.assert_close(h2.float().cpu(), plain.rms_norm(s[pick.long()], wn, 1e-5), **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,dim,num_parts", [(3, 5120, 7), (40, 5120, 7), (64, 8192, 16), (8, 1000, 5), (20, 16384, 2), (2, 20000, 3),
+                                                (5, 1002, 4), (1, 16, 9)])
+def test_add_rmsnorm_with_partial_sums_at_every_row_length(dtype, rows, dim, num_parts):
+    """Partial sums stand where a delta stands, for few rows and many, rows longer than the wave-per-row
+    kernel takes, lengths that are no multiple of 4 and lengths beyond the vectorised kernel's."""
+    g = torch.Generator().manual_seed(rows * dim + num_parts)
+    x, w = torch.randn(rows, dim, generator=g) * 3, 1 + 0.1 * torch.randn(dim, generator=g)
+    parts = torch.randn(num_parts, rows, dim, generator=g)
+    xd = dev(x.clone())
+    h = K().add_rmsnorm(xd, K().PartialSums(dev(parts)), dev(w), 1e-5, dtype)
+    s = x + parts.sum(0)
+    torch.testing.assert_close(xd.cpu(), s, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(h.float().cpu(), plain.rms_norm(s, w, 1e-5), **tol(dtype))
+    pick = torch.tensor([rows - 1, 0], dtype=torch.int32)
+    xd2 = dev(x.clone())
+    h2 = K().add_rmsnorm(xd2, K().PartialSums(dev(parts)), dev(w), 1e-5, dtype, rows=dev(pick), write_x=False)
+    assert torch.equal(xd2.cpu(), x)
+    torch.testing.assert_close(h2.float().cpu(), plain.rms_norm(s[pick.long()], w, 1e-5), **tol(dtype))
+
+
 def test_linear_hands_back_partial_sums_only_when_asked():
     x = dev(torch.randn(40, 2048).bfloat16())
     w = dev((torch.randn(1024, 2048) * 0.02).bfloat16())
