@@ -267,11 +267,24 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float* __restrict
       }
       if (pr) {  // a delta that still is a sum of partial products: added in the order of the runs
         float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < num_parts; ++p) {
-          const float4 pa = *reinterpret_cast<const float4*>(pr + p * part_stride + e);
-          const float4 pb = *reinterpret_cast<const float4*>(pr + p * part_stride + e + 4);
+        auto add = [&](const float4& pa, const float4& pb) {
           d[0] += pa.x, d[1] += pa.y, d[2] += pa.z, d[3] += pa.w, d[4] += pb.x, d[5] += pb.y, d[6] += pb.z, d[7] += pb.w;
+        };
+        const float* at = pr + e;
+        int p = 0;
+        for (; p + 4 <= num_parts; p += 4) {  // the loads of four runs in flight at once, their sums in the runs' order
+          float4 pa[4], pb[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            pa[q] = *reinterpret_cast<const float4*>(at + (size_t)(p + q) * part_stride);
+            pb[q] = *reinterpret_cast<const float4*>(at + (size_t)(p + q) * part_stride + 4);
+          }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) add(pa[q], pb[q]);
         }
+        for (; p < num_parts; ++p)
+          add(*reinterpret_cast<const float4*>(at + (size_t)p * part_stride),
+              *reinterpret_cast<const float4*>(at + (size_t)p * part_stride + 4));
 #pragma unroll
         for (int j = 0; j < 8; ++j) s[c][j] += d[j];
       }

@@ -47,16 +47,15 @@ struct Pending {
   bool any() const { return delta || parts; }
 };
 
-// Whether the small matrix-core kernel serves a product of m rows with a weight of `rows_of_w` rows. Up to 16
-// rows always. From 17 to 64 rows for products with many output columns, where a block per 16 columns fills
-// the chip (measured at 24 to 64 rows: 4,096 columns 9.6-12.0 us against 12.3-12.8 with the library, the
-// gated 2 x 3,072 columns 11.5-14.7 against 18.3-19.0 for the library and the SwiGLU kernel; 1,024 columns
-// lose against the library; not the vocabulary-sized head, whose thousands of blocks would each read all of x).
-bool small_serves(int m, int rows_of_w, int k, bool gated) {
-  if (k % 8) return false;
-  if (m <= kSmallFastRows) return true;
-  return m <= kSmallMaxRows && (gated || (rows_of_w >= 2048 && rows_of_w <= 16384));
-}
+// Which kernel serves a bfloat16 product of m rows (measured on the layer sizes of a 0.6B, an 8B and a 32B model):
+//   up to 16 rows, weights below 16 MiB: the small matrix-core kernel, the residual add and the norm as its prologue
+//     (a launch less; at these sizes a launch is most of a kernel's time);
+//   17 to 64 rows, weights below 16 MiB: the weight-streaming kernel (qkv 5.0-6.7 us, gate/up with SwiGLU 6.6-9.3
+//     against 5.8-7.7 and 7.5-10.3 with the small kernel, 8.2-8.6 and 14.4-14.7 with the library and a SwiGLU kernel);
+//   a delta of the residual stream from 17 rows on, or of a large weight: the weight-streaming kernel with k cut
+//     into runs whose partial sums the next add-and-norm adds up (1,024 columns: 3.9-5.3 us against 7.9-16 and 7.6-9.8);
+//   everything else: the GEMM library, as the reference hands every projection to one.
+bool small_serves(int m, int k) { return k % 8 == 0 && m <= kSmallFastRows; }
 
 // Whether a product of up to 64 rows is bound by streaming its weight: the layers of wide models. Their
 // deltas go to the weight-streaming kernel with k cut into runs (measured at 4,096 and 5,120 columns, k of 4,096
@@ -70,6 +69,11 @@ bool weight_bound(int m, int rows_of_w, int k) {
   return m <= kSmallMaxRows && k % 8 == 0 && elements >= kStreamMinElements && elements * 2 < kStreamMaxBytes;
 }
 
+// What the weight-streaming kernel takes at all.
+bool streams(int m, int rows_of_w, int k) {
+  return m <= kSmallMaxRows && k % 8 == 0 && (int64_t)rows_of_w * k * 2 < kStreamMaxBytes;
+}
+
 int compute_units() {
   static int units = 0;
   if (!units) {
@@ -80,14 +84,6 @@ int compute_units() {
       units = 256;
   }
   return units;
-}
-
-// Into how many runs of k a product of 17 to 64 rows with few output columns is cut (1: not at all): a block
-// per 16 columns leaves most of the chip idle and makes each block read all of x, so k is cut until about
-// every compute unit has a block, each with at least 256 of k.
-int delta_splits(int rows, int n, int k) {
-  if (!(rows > kSmallFastRows && rows <= kSmallMaxRows) || n >= 2048 || k % 8) return 1;
-  return std::max(1, std::min({8, 256 / ((n + 15) / 16), k / 256}));
 }
 
 std::mutex g_refused_mutex;
@@ -272,8 +268,11 @@ class Run {
       ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated ? 1 : 0, out_dtype, 1, compute_units(), stream_));
       return;
     }
-    const bool to_library = heavy && m > kSmallFastRows;
-    if (!to_library && small_serves(m, rows_of_w, k, gated)) {
+    if (!heavy && m > kSmallFastRows && streams(m, rows_of_w, k) && (out_dtype == kBF16 || !gated)) {
+      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated ? 1 : 0, out_dtype, 1, compute_units(), stream_));
+      return;
+    }
+    if (!heavy && small_serves(m, k)) {
       ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, out, m, n, k, 0, gated ? 1 : 0, out_dtype, 1, stream_));
       return;
     }
@@ -296,7 +295,7 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
-    if (dtype_ == kBF16 && weight_bound(t_, n, k)) {
+    if (dtype_ == kBF16 && (weight_bound(t_, n, k) || (t_ > kSmallFastRows && streams(t_, n, k)))) {
       const int splits = me_gemm_bf16_stream_splits(n, k, compute_units());
       if (splits > 1) {
         parts_mark_ = arena_.used;
@@ -310,18 +309,6 @@ class Run {
       ok(me_gemm_bf16_stream(x, op.p[1], bufs_[op.out], t_, n, k, 0, kBF16, 1, compute_units(), stream_));
       pending_.delta = bufs_[op.out];
       return;
-    }
-    if (dtype_ == kBF16 && !small_serves(t_, n, k, false)) {
-      const int splits = delta_splits(t_, n, k);
-      if (splits > 1) {  // partial sums over runs of k, each by blocks of its own; the next norm adds them up
-        parts_mark_ = arena_.used;
-        float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);
-        ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], parts, t_, n, k, 0, 0, kF32, splits, stream_));
-        pending_.parts = parts;
-        pending_.num_parts = splits;
-        pending_.stride = (long long)t_ * n;
-        return;
-      }
     }
     const size_t mark = arena_.used;
     product(x, op.p[1], n, k, false, dtype_, bufs_[op.out]);
@@ -415,6 +402,8 @@ class Run {
     float* logits = (float*)arena_.take((size_t)rows * vocab * 4);
     if (dtype_ == kF32)
       ok(me_gemm_f32((const float*)picked, (const float*)op.p[1], logits, rows, vocab, h_, stream_));
+    else if (rows > 2 && rows <= kSmallFastRows && weight_bound(rows, vocab, h_))  // 58-61 us against 63-71 at 8 to 16 rows
+      ok(me_gemm_bf16_stream(picked, op.p[1], logits, rows, vocab, h_, 0, kF32, 1, compute_units(), stream_));
     else if (rows <= kSmallFastRows && h_ % 8 == 0)
       ok(me_gemm_bf16_small(picked, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], logits, rows, vocab, h_, 0, 0, kF32, 1, stream_));
     else

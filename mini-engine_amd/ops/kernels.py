@@ -488,17 +488,9 @@ def tiled_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def small_ok(x, weight: torch.Tensor, gated: bool = False) -> bool:
-    """Whether the small matrix-core kernel serves this product. Up to 16 rows always. From 17 to 64 rows
-    for products with many output columns, where a block per 16 columns fills the chip: measured at 24 to
-    64 rows, 4,096 columns 9.6-12.0 us against 12.3-12.8 with the library, the gated 2 x 3,072 columns
-    11.5-14.7 against 18.3-19.0 for the library and the SwiGLU kernel; 1,024 columns (64 blocks that each
-    read all of x) lose against the library."""
-    if x.shape[1] % 8 or x.data_ptr() % 16 or weight.data_ptr() % 16:
-        return False
-    if x.shape[0] <= SMALL_FAST_ROWS:
-        return True
-    # (not the vocabulary-sized head: thousands of blocks would each read all of x)
-    return x.shape[0] <= SMALL_MAX_ROWS and (gated or 2048 <= weight.shape[0] <= 16384)
+    """Whether the small matrix-core kernel serves this product: up to 16 rows (with more rows the
+    weight-streaming kernel, which fetches x once per block of columns, is ahead)."""
+    return x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and x.shape[0] <= SMALL_FAST_ROWS
 
 
 STREAM_MIN_ELEMENTS = 8 << 20  # weights from 16 MiB on: streaming them is the product's time
@@ -513,13 +505,10 @@ def weight_bound(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and weight.numel() * 2 < STREAM_MAX_BYTES and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def delta_splits(rows: int, n: int, k: int) -> int:
-    """Into how many runs of k a product of 17 to 64 rows with few output columns is cut (1: not at all):
-    a block per 16 columns leaves most of the chip idle and makes each block read all of x, so k is
-    cut until about every compute unit has a block, each with at least 256 of k."""
-    if not SMALL_FAST_ROWS < rows <= SMALL_MAX_ROWS or n >= 2048 or k % 8:
-        return 1
-    return max(1, min(8, 256 // -(-n // 16), k // 256))
+def streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """What the weight-streaming kernel takes at all."""
+    return (x.shape[0] <= SMALL_MAX_ROWS and x.shape[1] % 8 == 0 and weight.numel() * 2 < STREAM_MAX_BYTES
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
 def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False,
@@ -530,11 +519,12 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     (what a mixer or a feed-forward returns): it may then come back as :class:`PartialSums`, which
     :func:`add_rmsnorm` adds up on the way.
 
-    float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16: the
-    fused matrix-core kernel for up to 16 rows; the tiled matrix-core kernel with the SwiGLU as its
-    epilogue for gated products of 256 rows or more; else the GEMM library (for the plain projections
-    of a prompt it is as fast as the tiled kernel or faster, measured). Rows are processed in slices of
-    64 when a float32 result is wanted from bfloat16 inputs (logits) and the library cannot give one."""
+    float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16, by rows and
+    weight size as ``csrc/host/program.cpp`` chooses (where the measurements are): up to 16 rows the small
+    matrix-core kernel, or the weight-streaming one for weights of 16 MiB and more; 17 to 64 rows the
+    weight-streaming kernel (the library for weights of 16 MiB and more); a delta of the residual stream
+    from 17 rows on, or of a large weight, as partial sums over runs of k; the tiled matrix-core kernel with
+    the SwiGLU as its epilogue for gated products of 256 rows or more; else the GEMM library."""
     if isinstance(x, NormedInput):
         if x.fusable(weight):
             return gemm_bf16_small(x, weight, out_dtype or x.dtype, gated)
@@ -545,20 +535,16 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
             raise TypeError("the float32 path keeps float32 results")
         y = gemm_f32(x, weight)
         return swiglu(y) if gated else y
-    heavy = weight_bound(x, weight)
-    if heavy and as_delta and not gated:
+    heavy, few = weight_bound(x, weight), x.shape[0] <= SMALL_FAST_ROWS
+    if as_delta and not gated and (heavy or (not few and streams(x, weight))):
         splits = stream_splits(weight.shape[0], x.shape[1], x.device)
         if splits > 1:
             return PartialSums(gemm_bf16_stream(x, weight, torch.float32, k_splits=splits))
         return gemm_bf16_stream(x, weight, out_dtype)
-    if heavy and x.shape[0] <= SMALL_FAST_ROWS and (out_dtype is torch.bfloat16 or not gated):
+    if (heavy if few else streams(x, weight) and not heavy) and (out_dtype is torch.bfloat16 or not gated):
         return gemm_bf16_stream(x, weight, out_dtype, gated)
     if small_ok(x, weight, gated) and not heavy:
         return gemm_bf16_small(x, weight, out_dtype, gated)
-    if as_delta and not gated and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0:
-        splits = delta_splits(x.shape[0], weight.shape[0], x.shape[1])
-        if splits > 1:
-            return PartialSums(gemm_bf16_small(x, weight, torch.float32, k_splits=splits))
     if gated:
         if tiled_ok(x, weight) and out_dtype is torch.bfloat16:
             return gemm_bf16_tiled(x, weight, out_dtype, True)  # measured ahead of the library product + SwiGLU kernel
