@@ -28,6 +28,8 @@ class Attention(Mixer):
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         s = spec
+        if not (float(s.scale) > 0.0 and float(s.scale) < float("inf")):
+            raise ValueError(f"the score scale must be positive and finite, got {s.scale}: the kernels scale before they mask")
         if s.num_heads % s.num_kv_heads:
             raise ValueError(f"{s.num_heads} query heads are not a multiple of {s.num_kv_heads} key/value heads")
         if s.head_dim % 16 or not 16 <= s.head_dim <= MAX_HEAD_DIM:

@@ -59,10 +59,10 @@ def read_header(path: str) -> dict[str, TensorEntry]:
         tag = info["dtype"]
         if tag not in _DTYPES:
             raise ValueError(f"{path}: tensor {name!r} has unsupported dtype {tag}")
-        b, e = info["data_offsets"]
+        b, e = (int(v) for v in info["data_offsets"])
         shape = tuple(int(s) for s in info["shape"])
         want = int(np.prod(shape, dtype=np.int64)) * np.dtype(_DTYPES[tag][0]).itemsize
-        if e - b != want or base + e > size:
+        if min(shape, default=0) < 0 or b < 0 or e < b or e - b != want or base + e > size:
             raise ValueError(f"{path}: tensor {name!r} has inconsistent offsets {b}..{e} for shape {shape}")
         entries[name] = TensorEntry(name, tag, shape, path, base + b, base + e)
     return entries

@@ -140,6 +140,10 @@ def test_attention_part_refuses_unsupported_head_sizes():
     with pytest.raises(ValueError, match="multiple"):
         MIXERS.build(AttentionSpec(hidden_size=64, num_heads=3, num_kv_heads=2, head_dim=16, scale=1.0),
                      torch.float32, torch.device("cuda"))
+    for scale in (0.0, -0.25, float("inf"), float("nan")):  # the kernels scale before or after masking: only a positive scale agrees
+        with pytest.raises(ValueError, match="scale"):
+            MIXERS.build(AttentionSpec(hidden_size=64, num_heads=2, num_kv_heads=1, head_dim=16, scale=scale),
+                         torch.float32, torch.device("cuda"))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

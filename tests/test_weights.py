@@ -40,6 +40,20 @@ def test_truncated_file_is_refused(tmp_path):
         read_header(str(p))
 
 
+def test_offsets_that_point_before_the_data_or_run_backwards_are_refused(tmp_path):
+    """A header whose offsets are negative (they would point into the header itself) or whose shape has a
+    negative size passes a length check alone; both are refused like any other inconsistent offsets."""
+    import json
+    import struct
+
+    for offsets, shape in (([-16, 0], [4]), ([16, 0], [-4]), ([0, 16], [-2, -2])):
+        header = json.dumps({"a": {"dtype": "F32", "shape": shape, "data_offsets": offsets}}).encode()
+        p = tmp_path / "bad.safetensors"
+        p.write_bytes(struct.pack("<Q", len(header)) + header + bytes(16))
+        with pytest.raises(ValueError, match="inconsistent offsets"):
+            read_header(str(p))
+
+
 def _decoder(cfg):
     return Decoder(plan_from_config(cfg), torch.float32, "cpu")
 
