@@ -161,10 +161,10 @@ class DecodeBench:
         engine, k, w = self.engine, steps, warmup
         prefill_steps = -(-batch * (prompt_len or self.ctx) // self.budget) + 1
         if prompt_len is None:
-            prompt_len = self.ctx - (k + w + prefill_steps) - 2
+            prompt_len = self.ctx - (k + w + prefill_steps) - 4
             if prompt_len < 1:
                 raise SystemExit("context is too short for this many steps")
-        params = SamplingParams(max_tokens=k + w + prefill_steps + 2, temperature=0.0, ignore_eos=True)
+        params = SamplingParams(max_tokens=k + w + prefill_steps + 4, temperature=0.0, ignore_eos=True)
         seqs = [engine.add_request(self.prompt(prompt_len), params) for _ in range(batch)]
         while any(s.num_output_tokens == 0 for s in seqs):
             engine.step()
@@ -173,6 +173,10 @@ class DecodeBench:
         synchronize()
         tokens_before = sum(len(s) for s in seqs)
         engine.time_phases = phases
+        if phases:
+            engine.step()  # settles a step that was launched ahead, untimed
+            synchronize()
+            tokens_before = sum(len(s) for s in seqs)
         before = dict(engine.stats.phase_seconds)
         t0 = time.perf_counter()
         for _ in range(k):

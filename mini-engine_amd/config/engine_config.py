@@ -23,6 +23,7 @@ class EngineConfig:
     dtype: str = "float32"
     seed: int = 0
     cuda_graphs: bool = True
+    decode_ahead: bool = True  # launch the next decode step before the host has read this step's tokens
 
     def __post_init__(self) -> None:
         if self.dtype not in DTYPES:

@@ -228,7 +228,7 @@ int me_core_queues(void* box, int64_t* waiting, int cap_waiting, int64_t* runnin
 // out: preemptions, tokens served by the prefix cache, evictions, unfinished (0/1)
 int me_core_counters(void* box, int64_t* out) {
   ME_GUARD(me::Core& c = core_of(box); out[0] = c.preemptions; out[1] = c.cached_tokens; out[2] = c.evictions();
-           out[3] = c.unfinished(); return 0;)
+           out[3] = c.unfinished(); out[4] = c.generated; return 0;)
 }
 
 // ---------------------------------------------------------------------------------------- step
@@ -314,6 +314,14 @@ int me_core_settle_rows(void* box, const int32_t* drawn, int count, int64_t* fin
              next.push_back(drawn[at++]); }
            if (at != count) throw me::Error(me::kBadValue, "more tokens were drawn than the step has wanted rows");
            std::vector<int64_t> done; const int n = c.settle(next.data(), (int)next.size(), done);
+           for (int i = 0; i < n && i < cap; ++i) finished[i] = done[i]; return n;)
+}
+
+// One step ahead (Core::plan_ahead, Core::settle_in_flight).
+int me_core_plan_ahead(void* box) { ME_GUARD(return core_of(box).plan_ahead();) }
+
+int me_core_settle_in_flight(void* box, const int32_t* drawn, int count, int64_t* finished, int cap) {
+  ME_GUARD(std::vector<int64_t> done; const int n = core_of(box).settle_in_flight(drawn, count, done);
            for (int i = 0; i < n && i < cap; ++i) finished[i] = done[i]; return n;)
 }
 

@@ -115,6 +115,10 @@ struct Request {
   float temperature = 0.f;
   bool ignore_eos = false;
   bool held = true;  // a Python object still names this request
+  // While a step is in flight whose draw for this request the host has not read yet: the last of `tokens` is a
+  // stand-in for that draw, which a step planned ahead feeds from row `fed_row` of the draws on the device.
+  bool pending = false;
+  int fed_row = -1;
 
   int size() const { return (int)tokens.size(); }
   int uncomputed() const { return size() - num_computed; }
@@ -199,12 +203,16 @@ class Core {
 
   // scheduler
   void enqueue(Request* r);
-  bool unfinished() const { return !waiting_.empty() || !running_.empty(); }
+  bool unfinished() const { return !waiting_.empty() || !running_.empty() || !in_flight_.empty(); }
   int plan();  // fills step() from the queues; returns the number of items
   int settle(const int32_t* next_tokens, int count, std::vector<int64_t>& finished);
+  // One step ahead: see scheduler.cpp.
+  int plan_ahead();
+  int settle_in_flight(const int32_t* drawn, int count, std::vector<int64_t>& finished);
+  bool has_in_flight() const { return !in_flight_.empty(); }
   const std::deque<Request*>& waiting() const { return waiting_; }
   const std::vector<Request*>& running() const { return running_; }
-  long preemptions = 0, cached_tokens = 0;
+  long preemptions = 0, cached_tokens = 0, generated = 0;  // generated: tokens appended to requests by draws
 
   // the step under construction / last planned
   std::vector<StepItem>& step() { return step_; }
@@ -226,7 +234,9 @@ class Core {
   std::deque<Request*> waiting_;
   std::vector<Request*> running_;
   std::vector<StepItem> step_;
+  std::vector<StepItem> in_flight_;  // the step launched before step_ whose draws are not settled yet
   void reap(Request* r);
+  void finish(Request* r, std::vector<int64_t>& finished);
 };
 
 // The core inside the box that the C functions of api.cpp hand out.

@@ -41,6 +41,8 @@ void Core::reap(Request* r) {
   if (std::find(waiting_.begin(), waiting_.end(), r) != waiting_.end()) return;
   for (const StepItem& it : step_)
     if (it.request == r) return;
+  for (const StepItem& it : in_flight_)
+    if (it.request == r) return;
   drop(r);
   requests_.erase(r->handle);
 }
@@ -78,6 +80,7 @@ void Core::evict(Request* r) {
 }
 
 int Core::plan() {
+  if (!in_flight_.empty()) throw Error(kBadState, "a step is in flight: settle it before the next one is planned from the queues");
   step_.clear();
   int budget = config_.max_num_batched_tokens;
   bool memory_was_tight = false;
@@ -134,26 +137,98 @@ bool Core::done(const Request* r, int32_t token) const {
   return r->num_output() >= r->max_tokens;
 }
 
+void Core::finish(Request* r, std::vector<int64_t>& finished) {
+  r->phase = kFinished;
+  drop(r);
+  running_.erase(std::find(running_.begin(), running_.end(), r));
+  finished.push_back(r->handle);
+}
+
 // After the model ran the planned step: next_tokens[i] is the token sampled for item i, or negative
-// for a portion that did not reach its request's last token (reference scheduler.py:107-123).
+// for a portion that did not reach its request's last token (reference scheduler.py:107-123). An item
+// of a step planned ahead whose request ended with the draw before it is passed over: its token was
+// computed for nothing.
 int Core::settle(const int32_t* next_tokens, int count, std::vector<int64_t>& finished) {
   if (count != (int)step_.size()) throw Error(kBadValue, "one token (or none) per scheduled sequence is needed");
+  if (!in_flight_.empty()) throw Error(kBadState, "the step before this one is still in flight: settle it first");
   finished.clear();
   std::vector<StepItem> items;
   items.swap(step_);
   for (int i = 0; i < count; ++i) {
     Request* r = items[i].request;
+    if (r->phase == kFinished) continue;
     r->num_computed += items[i].count;
     note_computed(r);
     drop_passed(r);
     if (next_tokens[i] < 0) continue;
     r->tokens.push_back(next_tokens[i]);
-    if (done(r, next_tokens[i])) {
-      r->phase = kFinished;
-      drop(r);
-      running_.erase(std::find(running_.begin(), running_.end(), r));
-      finished.push_back(r->handle);
+    ++generated;
+    if (done(r, next_tokens[i])) finish(r, finished);
+  }
+  for (const StepItem& it : items) reap(it.request);
+  return (int)finished.size();
+}
+
+// One step ahead. The planned step has been launched and its draws are still on the device. When it decodes
+// one token for every running request and no waiting request could be admitted, the step after it is known
+// but for the token ids: every request that cannot end by its count of tokens decodes the token it is about
+// to draw. plan_ahead() makes the launched step the one in flight (its requests advance as settle() would
+// advance them, with a stand-in for the unknown token) and plans that next step, whose token ids the device
+// takes from the draws of the step in flight (`fed_row`). Returns its number of items, or 0 when nothing was
+// changed: the caller then settles and plans as usual. The pages every request needs are taken first, so
+// nothing is evicted on the way. A request that ends with the draw in flight (an end token) has run one token
+// too many in the step planned ahead; settle() passes it over.
+int Core::plan_ahead() {
+  if (!in_flight_.empty()) throw Error(kBadState, "a step is in flight already");
+  if (step_.empty() || step_.size() != running_.size()) return 0;
+  if (!waiting_.empty() && (int)running_.size() < config_.max_num_seqs) return 0;
+  std::vector<int> goes_on;
+  for (size_t i = 0; i < step_.size(); ++i) {
+    const StepItem& it = step_[i];
+    const Request* r = it.request;
+    if (it.count != 1 || it.want.size() != 1 || it.want[0] != 0 || it.start + 1 != r->size() || r->pending ||
+        r->phase != kRunning)
+      return 0;
+    if (r->num_output() + 1 < r->max_tokens && r->size() + 1 <= config_.max_model_len) goes_on.push_back((int)i);
+  }
+  if (goes_on.empty()) return 0;
+  for (int i : goes_on)
+    if (!grow(step_[i].request, step_[i].request->size() + 1)) return 0;
+  in_flight_.swap(step_);
+  for (StepItem& it : in_flight_) {
+    Request* r = it.request;
+    r->num_computed += 1;
+    note_computed(r);
+    drop_passed(r);
+  }
+  for (int i : goes_on) {
+    Request* r = in_flight_[i].request;
+    r->tokens.push_back(0);
+    r->pending = true;
+    r->fed_row = i;
+    step_.push_back(StepItem{r, r->size() - 1, 1, {0}});
+  }
+  return (int)step_.size();
+}
+
+// The draws of the step in flight, one per item in the order of its rows: stand-ins become tokens, requests
+// end as in settle(). The step planned ahead stays planned.
+int Core::settle_in_flight(const int32_t* drawn, int count, std::vector<int64_t>& finished) {
+  if (count != (int)in_flight_.size()) throw Error(kBadValue, "one token per item of the step in flight is needed");
+  finished.clear();
+  std::vector<StepItem> items;
+  items.swap(in_flight_);
+  for (int i = 0; i < count; ++i) {
+    Request* r = items[i].request;
+    if (r->pending) {
+      r->tokens.back() = drawn[i];
+      r->pending = false;
+      r->fed_row = -1;
+    } else {
+      r->tokens.push_back(drawn[i]);
     }
+    ++generated;
+    if (done(r, drawn[i])) finish(r, finished);
   }
   for (const StepItem& it : items) reap(it.request);
   return (int)finished.size();

@@ -133,6 +133,7 @@ void Core::pack(int32_t* dst, const StepLayout& lay, int spare_page, int spare_s
       dst[lay.token_ids + cursor + j] = r->tokens[it.start + j];
       dst[lay.positions + cursor + j] = it.start + j;
       dst[lay.token_item + cursor + j] = i;
+      if (r->pending && it.start + j + 1 == r->size()) dst[lay.token_source + cursor + j] = r->fed_row;
     }
     for (int w : it.want) {
       // a wanted place that is the request's last token is where the next token is drawn from
@@ -179,7 +180,7 @@ void Core::refill(int32_t* dst, const StepLayout& lay, std::vector<RowMemo>& row
     dst[lay.token_ids + i] = is_live ? r->tokens[it->start] : 0;
     dst[lay.positions + i] = is_live ? it->start : 0;
     dst[lay.item_ctx + i] = is_live ? it->start + 1 : 1;
-    dst[lay.token_source + i] = -1;
+    dst[lay.token_source + i] = is_live && r->pending && it->start + 1 == r->size() ? r->fed_row : -1;
     dst[lay.state_slots + i] = is_live && r->state_slot >= 0 ? r->state_slot : spare_slot;
     float temperature = 0.f;
     uint64_t key = 0;

@@ -65,6 +65,8 @@ def _api():
         L.me_core_forget_rows.argtypes = [_vp, ctypes.c_int]
         L.me_core_pack_padding.argtypes = [_vp, _vp, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         L.me_core_settle_rows.argtypes = [_vp, _vp, ctypes.c_int, _vp, ctypes.c_int]
+        L.me_core_plan_ahead.argtypes = [_vp]
+        L.me_core_settle_in_flight.argtypes = [_vp, _vp, ctypes.c_int, _vp, ctypes.c_int]
         _declared = True
     return L
 
@@ -263,6 +265,19 @@ class HostCore:
         n = _ok(self._L.me_core_settle_rows(self._box, _ptr(drawn), len(drawn), _ptr(done), len(done)))
         return done[:n].tolist()
 
+    def plan_ahead(self) -> int:
+        """The planned step has been launched: when the step after it is known but for the token ids (every
+        running request decodes one more token, nobody waits for admission), make the launched step the one
+        in flight and plan that next step, whose ids the device takes from the draws in flight. Number of
+        items of the new step, or 0 when nothing was changed."""
+        return _ok(self._L.me_core_plan_ahead(self._box))
+
+    def settle_in_flight(self, drawn: np.ndarray) -> list[int]:
+        """The draws of the step in flight (int32, one per item in row order); the step planned ahead stays."""
+        done = np.zeros(max(1, len(drawn)), dtype=np.int64)
+        n = _ok(self._L.me_core_settle_in_flight(self._box, _ptr(drawn), len(drawn), _ptr(done), len(done)))
+        return done[:n].tolist()
+
     def queues(self) -> tuple[list[int], list[int]]:
         counts = np.zeros(2, dtype=np.int32)
         _ok(self._L.me_core_queues(self._box, None, 0, None, 0, _ptr(counts)))
@@ -271,7 +286,7 @@ class HostCore:
         return w[:counts[0]].tolist(), r[:counts[1]].tolist()
 
     def counters(self) -> np.ndarray:
-        """preemptions, tokens served by the prefix cache, evictions, unfinished"""
+        """preemptions, tokens served by the prefix cache, evictions, unfinished, tokens generated"""
         _ok(self._L.me_core_counters(self._box, _ptr(self._info)))
         return self._info
 

@@ -65,6 +65,7 @@ class LLMEngine:
         self.sampler = self.runner.sampler
         self.stats = EngineStats()
         self.time_phases = False  # synchronise after each phase of a step and add its time to the stats
+        self._launched: _Launched | None = None  # the step that was launched ahead and is not settled yet
 
     @property
     def kv_caches(self):
@@ -109,34 +110,83 @@ class LLMEngine:
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
         """Run all prompts to completion as one continuously batched workload; output ids per prompt."""
         requests = [self.add_request(p, params) for p in prompts]
-        while self.scheduler.has_unfinished():
+        while self.scheduler.has_unfinished() or self._launched is not None:
             self.step()
         return [r.output_token_ids for r in requests]
 
+    def _launch(self) -> "_Launched":
+        """Launch the step the core holds; its draws are read later."""
+        tokens, items, rows, *_, warm = (int(v) for v in self.core.step_summary())
+        self.runner.run_planned()
+        return _Launched(tokens, items, rows, bool(warm), self.runner.last_replay)
+
     def step(self) -> list[Sequence]:
-        """One step of the loop; returns the requests that finished in it."""
-        timed = self.time_phases
-        clock = _PhaseClock(self.stats.phase_seconds) if timed else None
+        """One step of the loop; returns the requests that finished in it.
+
+        With ``decode_ahead`` a decode step that was replayed from a graph is followed at once by the
+        step after it, whose token ids the device takes from this step's draws, before the host reads
+        those draws: scheduling, the refill of the next graph's indices and its launch overlap the
+        device's work. A request that ends with an end token has then run one token too many, which is
+        dropped."""
+        if self.time_phases:
+            return self._step_timed()
+        step = self._launched
+        if step is None:
+            if self.core.plan() == 0:
+                raise RuntimeError("scheduler produced an empty batch with work pending")
+            step = self._launch()
+        ahead = None
+        if self.config.decode_ahead and step.replay is not None and self.core.plan_ahead() > 0:
+            ahead = self._launch()
+        drawn = self.runner.draw(step.rows, step.tempered, step.replay)
+        before = int(self.core.counters()[4])
+        finished = self.scheduler.settle_in_flight(drawn) if ahead is not None else self.scheduler.settle_rows(drawn)
+        self._launched = ahead
+        s = self.stats
+        s.steps += 1
+        s.step_batch_sizes.append(step.items)
+        s.computed_tokens += step.tokens
+        s.generated_tokens += int(self.core.counters()[4]) - before
+        return finished
+
+    def _step_timed(self) -> list[Sequence]:
+        """A step with the device awaited after each phase, its time added to the stats (no step ahead)."""
+        if self._launched is not None:  # a step launched ahead before the timing was switched on: settled untimed
+            step, self._launched = self._launched, None
+            finished = self.scheduler.settle_rows(self.runner.draw(step.rows, step.tempered, step.replay))
+            self.stats.steps += 1
+            self.stats.step_batch_sizes.append(step.items)
+            self.stats.computed_tokens += step.tokens
+            self.stats.generated_tokens += step.rows
+            return finished
+        clock = _PhaseClock(self.stats.phase_seconds)
         if self.core.plan() == 0:
             raise RuntimeError("scheduler produced an empty batch with work pending")
         tokens, items, rows, *_, warm = (int(v) for v in self.core.step_summary())
-        if timed:
-            clock.lap("schedule")
-        logits = self.runner.run_planned()
-        if timed:
-            clock.lap("forward")
+        clock.lap("schedule")
+        self.runner.run_planned()
+        clock.lap("forward")
         drawn = self.runner.draw(rows, bool(warm))
-        if timed:
-            clock.lap("sample")
+        clock.lap("sample")
         finished = self.scheduler.settle_rows(drawn)
         s = self.stats
         s.steps += 1
         s.step_batch_sizes.append(items)
         s.computed_tokens += tokens
         s.generated_tokens += rows
-        if timed:
-            clock.lap("postprocess")
+        clock.lap("postprocess")
         return finished
+
+
+@dataclass
+class _Launched:
+    """A step that runs on the device and whose draws have not been read."""
+
+    tokens: int
+    items: int
+    rows: int
+    tempered: bool
+    replay: int | None  # the pinned buffer its draws are copied to, when it was replayed from a graph
 
 
 class _PhaseClock:

@@ -71,6 +71,14 @@ class ModelRunner:
         self.batch: StepBatch | None = None  # the batch of the last step on the per-kernel path
         self._logits: torch.Tensor | None = None
         self._drawn: torch.Tensor | None = None  # what the native program drew for the last step's rows
+        # Replayed steps of a native program draw into one buffer on the device, from which the next replay may
+        # take its token ids; every replay is followed by a copy of its draws into pinned memory (two buffers in
+        # turn: a step planned ahead is launched before the draws of the step before it are read).
+        self._fed = torch.zeros(max(config.max_num_seqs, 1), dtype=torch.int32, device=self.device)
+        self._fed_host = [torch.zeros(max(config.max_num_seqs, 1), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._fed_done = [torch.cuda.Event(), torch.cuda.Event()]
+        self._fed_turn = 0
+        self.last_replay: int | None = None  # which pinned buffer holds the draws of the last step, if it was replayed
         self.graph_replays = 0
         self.eager_steps = 0
 
@@ -105,6 +113,7 @@ class ModelRunner:
         replay = bool(self.config.cuda_graphs and self.graph_safe and decode_only and last_only
                       and 0 < items <= self.config.max_num_seqs)
         self._drawn = None
+        self.last_replay = None
         if replay:
             # a replayed step checks the pages of its block tables while they are written into the graph's buffer
             core.step_check(self.decoder.plan.vocab_size, scan_pages=False)
@@ -131,11 +140,17 @@ class ModelRunner:
             _, starts, _, _, slots = self.core.step_items()
             self.storage.zero_state([s for s, p0 in zip(slots, starts) if p0 == 0 and s >= 0])
 
-    def draw(self, rows: int, tempered: bool):
-        """One token id per wanted row of the last step (int32, on the host): what the native program
-        drew beside the logits, or the sampler's draw from them."""
+    def draw(self, rows: int, tempered: bool, replay: int | None = None):
+        """One token id per wanted row of a step (int32, on the host): what the native program drew
+        beside the logits, or the sampler's draw from them. ``replay`` names the pinned buffer of a
+        replayed step (``last_replay`` right after it was launched); without it the last step is meant."""
         if rows == 0:
             return self.sampler.draw(None, None, 0, False)
+        if replay is None:
+            replay = self.last_replay
+        if replay is not None:
+            self._fed_done[replay].synchronize()
+            return self._fed_host[replay][:rows].numpy().copy()
         if self._drawn is not None:
             return self._drawn[:rows].cpu().numpy()
         return self.sampler.draw(self._logits, self.batch, rows, tempered)
@@ -145,7 +160,8 @@ class ModelRunner:
         """The launches of one decode step on a graph's static buffers: (logits, drawn or None)."""
         if self.program is None:
             return self.decoder.forward(batch), None
-        return run_static(self.program, self._static_arena, batch.buf, bucket, batch.widths, batch.max_ctx, batch.least_live)
+        return run_static(self.program, self._static_arena, batch.buf, bucket, batch.widths, batch.max_ctx, batch.least_live,
+                          drawn=self._fed, fed=True)
 
     def _capture(self, bucket: int):
         widths = [self.max_blocks_per_seq] * self.num_groups
@@ -162,6 +178,7 @@ class ModelRunner:
             most = self.config.max_num_seqs  # every bucket's graph works in the same memory: replays are serial
             self._static_arena = torch.empty(self.program.arena_need(most, most, most, self.config.max_model_len),
                                              dtype=torch.uint8, device=self.device)
+        fed = self._fed.clone()  # the warm-up run draws too: the draws of a step in flight are put back afterwards
         stream = torch.cuda.Stream()
         stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream):
@@ -172,6 +189,7 @@ class ModelRunner:
         with torch.cuda.graph(graph, pool=self._graph_pool):
             logits, drawn = self._forward_static(batch, bucket)
         self._graph_pool = graph.pool()
+        self._fed.copy_(fed)
         torch.cuda.synchronize()
         self._graphs[bucket] = (graph, batch, host, logits, drawn)
         return self._graphs[bucket]
@@ -199,4 +217,9 @@ class ModelRunner:
         self.batch = batch
         self._logits = logits[:n]
         self._drawn = None if drawn is None else drawn[:n]
+        if drawn is not None:  # the draws leave the device behind the graph, before a later replay overwrites them
+            turn = self._fed_turn = self._fed_turn ^ 1
+            self._fed_host[turn][:n].copy_(drawn[:n], non_blocking=True)
+            self._fed_done[turn].record()
+            self.last_replay = turn
         return self._logits

@@ -318,3 +318,36 @@ def test_command_line_with_a_random_shape_and_random_prompts():
     assert "served from prefix cache 48" in first  # 20 shared ids: two full pages of 8, three times
     assert [l for l in run(3).splitlines() if l.startswith("A: ")] == answers
     assert [l for l in run(4).splitlines() if l.startswith("A: ")] != answers
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_steps_launched_ahead_change_no_token(peaked, name):
+    """With ``decode_ahead`` the next decode step is launched before this step's tokens are read, its token
+    ids fed on the device. Greedy and sampled generation, end tokens (a request that ends has run one token
+    for nothing), a pool so small that requests are preempted, and graphs captured while a step is in
+    flight (buckets shrink as requests end): the same tokens as with every step settled before the next."""
+    from mini_engine_amd import EngineConfig, LLMEngine, SamplingParams
+
+    folder, pcfg, w = peaked[name]
+    prompts = prompts_for(name, n=11, hi=30, seed=5)
+    want = [plain.greedy_generate(w, pcfg, p, 24) for p in prompts]
+    eos = want[2][5]  # ends some requests early, others not at all
+    outs = {}
+    for ahead in (True, False):
+        for kind, over, params in (("greedy", {}, SamplingParams(max_tokens=24)),
+                                   ("sampled", {"seed": 3}, SamplingParams(max_tokens=17, temperature=0.9)),
+                                   ("squeezed", {"num_blocks": 12}, SamplingParams(max_tokens=24))):
+            eng = LLMEngine.from_pretrained(folder, EngineConfig(**{"block_size": 8, "num_blocks": 128, "dtype": "float32",
+                                                                    "max_num_seqs": 16, "decode_ahead": ahead, **over}))
+            eng.scheduler.eos_token_ids = {eos}
+            outs[ahead, kind] = eng.generate(prompts, params)
+            assert eng.runner.graph_replays > 0 and eng._launched is None
+            assert eng.stats.generated_tokens == sum(len(o) for o in outs[ahead, kind])
+            assert all(len(pool.free_pool) == pool.num_blocks for pool in eng.block_manager.pools)
+            if kind == "squeezed":
+                assert eng.scheduler.num_preemptions > 0
+    cut = [o[: o.index(eos) + 1] if eos in o else o for o in want]
+    assert outs[True, "greedy"] == outs[False, "greedy"] == cut
+    assert outs[True, "squeezed"] == outs[False, "squeezed"] == cut
+    assert outs[True, "sampled"] == outs[False, "sampled"] and outs[True, "sampled"] != [o[:17] for o in cut]
+    assert any(eos in o for o in cut) and any(eos not in o for o in cut)

@@ -200,3 +200,106 @@ def test_random_workloads_finish_with_nothing_held(seed):
     assert all(q.is_finished for q in seqs)
     assert all(1 <= q.num_output_tokens <= q.params.max_tokens for q in seqs)
     check_invariants(s.bm, [])
+
+
+# ------------------------------------------------------------------------------- one step ahead
+def decode_rows(s: Scheduler) -> list[tuple[int, int, int]]:
+    """(handle, first position, tokens) of the planned step's items."""
+    handles, starts, counts, _, _ = s.core.step_items()
+    return list(zip(handles, starts, counts))
+
+
+def test_a_step_is_planned_ahead_and_settled_one_step_late():
+    """Three requests decode. The step after the launched one is planned before its draws are known: every
+    request advances by a stand-in token that the device feeds; the draws arrive a step late and replace
+    the stand-ins. A request that reaches its count of tokens is not planned ahead, one that draws an end
+    token has run one token for nothing, which the next settling passes over."""
+    import numpy as np
+
+    s = make()
+    a, b, c = add(s, 5, max_tokens=8), add(s, 3, max_tokens=2, first=50), add(s, 6, max_tokens=8, first=80)
+    step(s, token=7)  # the prompts; every request has one output now
+    assert s.core.plan() == 3 and decode_rows(s) == [(a._handle, 5, 1), (b._handle, 3, 1), (c._handle, 6, 1)]
+    # launched; b ends with this step by its count, so only a and c go on
+    assert s.core.plan_ahead() == 2
+    assert decode_rows(s) == [(a._handle, 6, 1), (c._handle, 7, 1)]
+    assert len(a) == 7 and a.token_ids[-1] == 0 and len(b) == 4  # a stand-in at a's end, none at b's
+    arr = np.zeros(64, dtype=np.int32)
+    lay = s.core.step_layout()
+    s.core.step_pack(arr, None, 0, 0, 0)
+    source = arr[lay["token_source"]:lay["token_source"] + 2].tolist()
+    assert source == [0, 2]  # a's id is row 0 of the draws in flight, c's is row 2
+    with pytest.raises(RuntimeError, match="in flight"):
+        s.core.plan()
+    done = s.settle_in_flight(np.array([11, 12, EOS], dtype=np.int32))
+    assert set(done) == {b, c} and b.output_token_ids == [7, 12] and c.output_token_ids == [7, EOS]
+    assert a.token_ids[-1] == 11 and a.num_computed_tokens == 6
+    # the step planned ahead is settled like any other; c's item in it counts for nothing
+    assert s.core.plan_ahead() == 0  # c's item is dead: the engine settles and plans from the queues
+    assert s.settle_rows(np.array([13, 99], dtype=np.int32)) == []
+    assert a.output_token_ids == [7, 11, 13] and c.output_token_ids == [7, EOS] and c.is_finished
+    while s.has_unfinished():
+        step(s, token=5)
+    assert a.num_output_tokens == 8 and all(rc == 0 for rc in s.bm.ref_counts)
+
+
+def test_nothing_is_planned_ahead_when_a_request_waits_or_pages_run_out():
+    s = make(max_num_seqs=4)
+    a = add(s, 5, max_tokens=8)
+    step(s, token=7)
+    add(s, 4, max_tokens=8, first=60)  # waits and could be admitted: the next step is planned from the queues
+    assert s.core.plan() == 2 and s.core.plan_ahead() == 0
+    s.settle_rows(__import__("numpy").array([7, 7], dtype="int32"))
+    # a full house is no reason to wait for admissions
+    s2 = make(max_num_seqs=1)
+    x = add(s2, 5, max_tokens=8)
+    add(s2, 4, max_tokens=8, first=60)
+    step(s2, token=7)
+    assert s2.core.plan() == 1 and s2.core.plan_ahead() == 1
+    # no page for the token after next: nothing changes, and the engine settles and plans as usual
+    s3 = make(num_blocks=3)
+    y = add(s3, 7, max_tokens=3)
+    step(s3, token=7)  # 8 tokens: two pages, both full
+    z = add(s3, 1, max_tokens=3, first=90)
+    assert s3.core.plan() == 2  # y decodes, z is admitted to the third page
+    assert s3.core.plan_ahead() == 0 and len(y) == 8 and len(z) == 1
+    assert a is not None and x is not None
+
+
+def test_random_workloads_finish_the_same_with_steps_planned_ahead():
+    """The same requests and the same 'model' (the token is a function of the request and its length) with
+    and without steps planned ahead, under end tokens and a small pool: equal outputs, nothing held."""
+    import numpy as np
+
+    def token_for(handle: int, length: int) -> int:
+        v = (handle * 7919 + length * 104729) % 23
+        return EOS if v == 0 else 3 + v
+
+    def run(ahead: bool, seed: int) -> list[list[int]]:
+        rng = random.Random(seed)
+        s = make(num_blocks=24, max_num_seqs=6, max_num_batched_tokens=32)
+        seqs = [add(s, rng.randint(1, 20), max_tokens=rng.randint(1, 12), first=100 * k) for k in range(14)]
+        launched = None  # (handles, lengths at draw time) of a step whose draws are not settled
+        steps = 0
+        while s.has_unfinished() or launched is not None:
+            steps += 1
+            assert steps < 2000
+            if launched is None:
+                assert s.core.plan() > 0
+                handles, starts, counts, wants, _ = s.core.step_items()
+                launched = [(h, st + n + 1) if w else None for h, st, n, w in zip(handles, starts, counts, wants)]
+            nxt = None
+            if ahead and all(x is not None for x in launched) and s.core.plan_ahead() > 0:
+                handles, starts, counts, wants, _ = s.core.step_items()
+                nxt = [(h, st + n + 1) for h, st, n in zip(handles, starts, counts)]
+            drawn = np.array([token_for(*x) for x in launched if x is not None], dtype=np.int32)
+            if nxt is not None:
+                s.settle_in_flight(drawn)
+            else:
+                s.settle_rows(drawn)
+            launched = nxt
+        assert all(rc == 0 for rc in s.bm.ref_counts)
+        return [q.output_token_ids for q in seqs]
+
+    for seed in range(6):
+        assert run(True, seed) == run(False, seed)
