@@ -68,7 +68,8 @@ class AttentionSpec:
 
 @dataclass(frozen=True)
 class GatedMlpSpec:
-    """Dense gated feed-forward: ``down(act(gate(x)) * up(x))`` without biases."""
+    """Dense gated feed-forward: ``down(act(gate(x)) * up(x))`` without biases; ``activation`` is "silu" or
+    "gelu_tanh"."""
 
     hidden_size: int
     intermediate_size: int

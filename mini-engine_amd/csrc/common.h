@@ -45,6 +45,18 @@ __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
   return r;
 }
 
+// ------------------------------------------------------------------ the activation of a gated feed-forward
+// act(gate) * up: the codes that the entry points' `gated` arguments take (0: the product is not gated).
+enum MeGate { ME_GATE_NONE = 0, ME_GATE_SILU = 1, ME_GATE_GELU_TANH = 2 };
+
+__device__ __forceinline__ float gate_act(float g, int code) {
+  if (code == ME_GATE_GELU_TANH) {  // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+    const float u = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return 0.5f * g * (1.f + tanhf(u));
+  }
+  return g / (1.f + expf(-g));  // silu
+}
+
 // ------------------------------------------------------------------ wave and block reductions
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

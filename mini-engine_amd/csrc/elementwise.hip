@@ -394,10 +394,10 @@ extern "C" int me_rmsnorm(const void* in, const float* w, void* out, int num_row
 }
 
 // ------------------------------------------------------------------------------------ SwiGLU
-// act[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)). A thread handles VEC
+// act[t, i] = a(gu[t, i]) * gu[t, inter + i], a = silu (z / (1 + exp(-z))) or tanh-gelu by `gate`. A thread handles VEC
 // consecutive i (16-byte loads when the row length allows it).
 template <typename T, int VEC>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t total_vec) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t total_vec, int gate) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total_vec) return;
   const int per_row = inter / VEC;
@@ -412,32 +412,33 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int
 #pragma unroll
   for (int k = 0; k < VEC; ++k) {
     const float gf = to_float(g.v[k]);
-    o.v[k] = from_float<T>(gf / (1.f + expf(-gf)) * to_float(u.v[k]));
+    o.v[k] = from_float<T>(gate_act(gf, gate) * to_float(u.v[k]));
   }
   *reinterpret_cast<Pack*>(act + t * inter + i) = o;
 }
 
 template <typename T>
-static void launch_swiglu(const T* gu, T* act, int num_tokens, int inter, hipStream_t stream) {
+static void launch_swiglu(const T* gu, T* act, int num_tokens, int inter, int gate, hipStream_t stream) {
   constexpr int WIDE = 16 / sizeof(T);
   const bool wide = inter % WIDE == 0 && ((uintptr_t)gu % 16 == 0) && ((uintptr_t)act % 16 == 0);
   const int threads = 256;
   if (wide) {
     const size_t total = (size_t)num_tokens * (inter / WIDE);
-    swiglu_kernel<T, WIDE><<<(unsigned)((total + threads - 1) / threads), threads, 0, stream>>>(gu, act, inter, total);
+    swiglu_kernel<T, WIDE><<<(unsigned)((total + threads - 1) / threads), threads, 0, stream>>>(gu, act, inter, total, gate);
   } else {
     const size_t total = (size_t)num_tokens * inter;
-    swiglu_kernel<T, 1><<<(unsigned)((total + threads - 1) / threads), threads, 0, stream>>>(gu, act, inter, total);
+    swiglu_kernel<T, 1><<<(unsigned)((total + threads - 1) / threads), threads, 0, stream>>>(gu, act, inter, total, gate);
   }
 }
 
-extern "C" int me_swiglu(const void* gu, void* act, int num_tokens, int inter, int dtype, hipStream_t stream) {
+extern "C" int me_swiglu(const void* gu, void* act, int num_tokens, int inter, int gate, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (inter <= 0) return me_fail("me_swiglu: intermediate=%d", inter);
+  if (gate != ME_GATE_SILU && gate != ME_GATE_GELU_TANH) return me_fail("me_swiglu: unknown gate activation %d", gate);
   if (dtype == ME_F32)
-    launch_swiglu<float>((const float*)gu, (float*)act, num_tokens, inter, stream);
+    launch_swiglu<float>((const float*)gu, (float*)act, num_tokens, inter, gate, stream);
   else
-    launch_swiglu<bf16_t>((const bf16_t*)gu, (bf16_t*)act, num_tokens, inter, stream);
+    launch_swiglu<bf16_t>((const bf16_t*)gu, (bf16_t*)act, num_tokens, inter, gate, stream);
   return me_check_launch("me_swiglu");
 }
 

@@ -25,7 +25,7 @@ template <int MT, int WAVES, int U, bool NORM, bool SWIGLU, typename OutT, int N
 __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
     const bf16_t* __restrict__ X, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
     const float* __restrict__ w_norm, float eps, float* __restrict__ x_out, const bf16_t* __restrict__ W,
-    OutT* __restrict__ C, int M, int N, int K, int chunks_per_split) {
+    OutT* __restrict__ C, int M, int N, int K, int chunks_per_split, int gate) {
   // ACCS tiles of 16 weight rows per block: gate and up rows of the same 16 columns (SWIGLU), or NT
   // neighbouring tiles of 16 columns, which share the loads of x (products with very many columns)
   static_assert(!SWIGLU || NT == 1, "the gated form computes one tile of columns per block");
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
         }
         v0 *= scale;
         float y = v0;
-        if (SWIGLU) y = v0 / (1.f + expf(-v0)) * (v1 * scale);
+        if (SWIGLU) y = gate_act(v0, gate) * (v1 * scale);
         const int col = nb + tile * 16 + j;
         if (col < N) C[(size_t)m * N + col] = from_float<OutT>(y);
       }
@@ -161,14 +161,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
 }
 
 template <int MT, int WAVES, int U, typename OutT>
-static void launch_variant(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
+static void launch_variant(bool norm, int swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
                            const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
                            int splits, hipStream_t stream) {
   const dim3 blocks((N + 15) / 16, splits);
   const int cps = ((K + 31) / 32 + splits - 1) / splits;
 #define ME_LAUNCH(NORM, SWI)                                                                                  \
   gemm_small_kernel<MT, WAVES, U, NORM, SWI, OutT><<<blocks, WAVES * 64, 0, stream>>>(X, x_in, delta, w_norm, eps, \
-                                                                                      x_out, W, C, M, N, K, cps)
+                                                                                      x_out, W, C, M, N, K, cps, swiglu)
   if (norm && swiglu)
     ME_LAUNCH(true, true);
   else if (norm)
@@ -183,7 +183,7 @@ static void launch_variant(bool norm, bool swiglu, const bf16_t* X, const float*
 #define WIDE_MIN_COLUMNS 32768
 
 template <typename OutT>
-static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
+static void launch_small(bool norm, int swiglu, const bf16_t* X, const float* x_in, const bf16_t* delta,
                          const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K,
                          int splits, hipStream_t stream) {
   const int mt = (M + 15) / 16;
@@ -194,7 +194,7 @@ static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x
     // very many columns (the output head) and more than a row or two: a block computes 64 columns from
     // one set of loads of x (at 8 rows and 151,936 columns 63 us against 69; at one row it is slower)
     gemm_small_kernel<1, 8, 4, false, false, OutT, 4><<<dim3((N + 63) / 64), 8 * 64, 0, stream>>>(
-        X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, chunks);
+        X, x_in, delta, w_norm, eps, x_out, W, C, M, N, K, chunks, 0);
     return;
   }
   if (mt == 1 && chunks > 8 * 8)
@@ -219,7 +219,8 @@ static void launch_small(bool norm, bool swiglu, const bf16_t* X, const float* x
 //   norm == 0: input is X (bfloat16 [M, K]).  norm == 1: input is rmsnorm(x_in + delta) * w_norm, from the
 //   float32 residual stream x_in [M, K], delta (bfloat16 [M, K] or null), w_norm float32 [K]; when delta
 //   is given, x_in + delta is written to x_out (float32 [M, K], not aliasing x_in).
-//   swiglu == 0: W is [N, K].  swiglu == 1: W is [2 N, K] (gate rows, then up rows), C = silu(gate) * up.
+//   swiglu == 0: W is [N, K].  swiglu == 1 or 2 (MeGate): W is [2 N, K] (gate rows, then up rows), C = act(gate) * up
+//   with act silu or tanh-gelu.
 //   out_dtype: ME_BF16 or ME_F32. M <= 64, K % 8 == 0, pointers 16-byte aligned.
 //   k_splits > 1 (plain float32 products only): k is cut into that many runs of whole chunks of 32, each
 //   summed by blocks of its own, and C is [k_splits, M, N]: partial sums for the caller to add up (more
@@ -231,6 +232,7 @@ extern "C" int me_gemm_bf16_small(const void* X, const float* x_in, const void* 
   if (k_splits < 1 || k_splits > 64) return me_fail("me_gemm_bf16_small: %d splits of k", k_splits);
   if (k_splits > 1 && (norm || swiglu || out_dtype != ME_F32))
     return me_fail("me_gemm_bf16_small: partial sums over splits of k are plain float32 products");
+  if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_small: unknown gate activation %d", swiglu);
   if (M > 64) return me_fail("me_gemm_bf16_small: M=%d exceeds 64 rows", M);
   if (K <= 0 || K % 8) return me_fail("me_gemm_bf16_small: K=%d must be a positive multiple of 8", K);
   if (norm) {

@@ -60,7 +60,7 @@ __device__ __forceinline__ void store4(OutT* __restrict__ C, size_t ldc, int m, 
 template <int BM, int BN, int WM, int WN, bool SWIGLU, typename OutT>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_tiled_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                    OutT* __restrict__ C, int M, int N, int K, int m_tiles,
-                                                                   int n_tiles) {
+                                                                   int n_tiles, int gate) {
   constexpr int THREADS = WM * WN * 64;
   constexpr int WMR = BM / WM, WNR = BN / WN;  // rows of x / rows of W per wave
   constexpr int FM = WMR / 16, FN = WNR / 16;  // 16 x 16 fragments per wave
@@ -182,7 +182,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tiled_kernel(const bf16_t* 
         const int n = n0 + wn * (WNR / 2) + a * 16 + 4 * g;
         float v[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = silu_f(acc[a][b][i]) * acc[a + FN / 2][b][i];
+        for (int i = 0; i < 4; ++i)
+          v[i] = (gate == ME_GATE_GELU_TANH ? gate_act(acc[a][b][i], gate) : silu_f(acc[a][b][i])) * acc[a + FN / 2][b][i];
         store4<OutT>(C, ldc, m, n, M, N, v);
       }
     } else {
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tiled_kernel(const bf16_t* 
 }
 
 template <int BM, int BN, int WM, int WN, bool SWIGLU, typename OutT>
-int launch_one(const void* X, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
+int launch_one(const void* X, const void* W, void* C, int M, int N, int K, int gate, hipStream_t stream) {
   constexpr int COLS = SWIGLU ? BN / 2 : BN;
   const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + COLS - 1) / COLS;
   constexpr size_t LDS = (size_t)2 * (BM + BN) * GROW * sizeof(bf16_t);
@@ -210,7 +211,7 @@ int launch_one(const void* X, const void* W, void* C, int M, int N, int K, hipSt
     raised = true;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(WM * WN * 64), LDS, stream, (const bf16_t*)X,
-                     (const bf16_t*)W, (OutT*)C, M, N, K, m_tiles, n_tiles);
+                     (const bf16_t*)W, (OutT*)C, M, N, K, m_tiles, n_tiles, gate);
   return me_check_launch("me_gemm_bf16_tiled");
 }
 
@@ -219,12 +220,12 @@ int launch_tiled(const void* X, const void* W, void* C, int M, int N, int K, int
   if (swiglu) {
     if (out_dtype != ME_BF16) return me_fail("me_gemm_bf16_tiled: the gated form writes bfloat16");
     if constexpr ((BN / WN / 16) % 2 == 0)
-      return launch_one<BM, BN, WM, WN, true, bf16_t>(X, W, C, M, N, K, stream);
+      return launch_one<BM, BN, WM, WN, true, bf16_t>(X, W, C, M, N, K, swiglu, stream);
     else
       return me_fail("me_gemm_bf16_tiled: this tile shape has no gated form");
   }
-  if (out_dtype == ME_BF16) return launch_one<BM, BN, WM, WN, false, bf16_t>(X, W, C, M, N, K, stream);
-  return launch_one<BM, BN, WM, WN, false, float>(X, W, C, M, N, K, stream);
+  if (out_dtype == ME_BF16) return launch_one<BM, BN, WM, WN, false, bf16_t>(X, W, C, M, N, K, 0, stream);
+  return launch_one<BM, BN, WM, WN, false, float>(X, W, C, M, N, K, 0, stream);
 }
 
 // The block tile for a product: all shapes here run at about the same rate per unit of tile area (the
@@ -258,7 +259,8 @@ int choose_shape(int M, int N, int swiglu) {
 
 }  // namespace
 
-// C[M, N] = X[M, K] . W[N, K]^T, or with `swiglu` C[M, N] = silu(X . W[0:N]^T) * (X . W[N:2N]^T).
+// C[M, N] = X[M, K] . W[N, K]^T, or with `swiglu` (1 or 2, a MeGate code) C[M, N] = act(X . W[0:N]^T) * (X . W[N:2N]^T)
+// with act silu or tanh-gelu.
 // K is a multiple of 64. `shape` picks the block tile: 0 lets the entry point choose, others name one
 // (for measurements).
 extern "C" int me_gemm_bf16_tiled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
@@ -268,6 +270,7 @@ extern "C" int me_gemm_bf16_tiled(const void* X, const void* W, void* C, int M, 
   if (!X || !W || !C) return me_fail("me_gemm_bf16_tiled: null operand");
   if (((uintptr_t)X | (uintptr_t)W) & 15) return me_fail("me_gemm_bf16_tiled: operands must be 16-byte aligned");
   if (out_dtype != ME_BF16 && out_dtype != ME_F32) return me_fail("me_gemm_bf16_tiled: unknown output type %d", out_dtype);
+  if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_tiled: unknown gate activation %d", swiglu);
   if (shape == 0) shape = choose_shape(M, N, swiglu);
   switch (shape) {
     case 1: return launch_tiled<128, 128, 2, 2>(X, W, C, M, N, K, swiglu, out_dtype, stream);

@@ -29,7 +29,7 @@ constexpr int kRow = kStepK + 16;    // LDS row stride in elements: 288 bytes, 3
 
 template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                          OutT* __restrict__ C, int M, int N, int K, int steps_per_split) {
+                                                          OutT* __restrict__ C, int M, int N, int K, int steps_per_split, int gate) {
   static_assert(WN * WK == 4, "four waves per block");
   constexpr int KC = kStepK / WK;  // k per wave and step
   constexpr int CH = KC / 32;      // products per wave, step and tile of rows
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       y[j] = acc[t][0][j];
-      if (SWIGLU) y[j] = y[j] / (1.f + expf(-y[j])) * acc[t][1][j];
+      if (SWIGLU) y[j] = gate_act(y[j], gate) * acc[t][1][j];
     }
     OutT* dst = C + (size_t)m * N + nb;
     if (nb + 3 < N && (N & 3) == 0) {
@@ -179,24 +179,24 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
 
 template <int MT, bool SWIGLU, typename OutT>
 void launch_arranged(int wn, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int splits, int steps_per_split,
-                     hipStream_t stream) {
+                     int gate, hipStream_t stream) {
   const dim3 grid(((N + 15) / 16 + wn - 1) / wn, splits);
   if (wn == 4)
-    gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split);
+    gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
   else if (wn == 2)
-    gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split);
+    gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
   else
-    gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split);
+    gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
 }
 
 template <bool SWIGLU, typename OutT>
 void launch_rows(int wn, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int splits, int steps_per_split,
-                 hipStream_t stream) {
+                 int gate, hipStream_t stream) {
   switch ((M + 15) / 16) {
-    case 1: launch_arranged<1, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, stream); break;
-    case 2: launch_arranged<2, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, stream); break;
-    case 3: launch_arranged<3, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, stream); break;
-    default: launch_arranged<4, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, stream); break;
+    case 1: launch_arranged<1, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
+    case 2: launch_arranged<2, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
+    case 3: launch_arranged<3, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
+    default: launch_arranged<4, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
   }
 }
 
@@ -225,12 +225,13 @@ extern "C" int me_gemm_bf16_stream_splits(int N, int K, int compute_units) {
   return (steps + steps_per_split - 1) / steps_per_split;  // no empty run
 }
 
-// C[M, N] = x . W^T (swiglu: W is [2 N, K], gate rows then up rows, and C = silu(gate) * up), X bfloat16 [M, K],
+// C[M, N] = x . W^T (swiglu 1 or 2, a MeGate code: W is [2 N, K], gate rows then up rows, and C = act(gate) * up), X bfloat16 [M, K],
 // M <= 64, K % 8 == 0, pointers 16-byte aligned. out_dtype ME_BF16 or ME_F32. k_splits > 1 (plain float32
 // products only): C is [k_splits, M, N], partial sums over runs of k for the caller to add up.
 extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
                                    int k_splits, int compute_units, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
+  if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_stream: unknown gate activation %d", swiglu);
   if (M > 64) return me_fail("me_gemm_bf16_stream: M=%d exceeds 64 rows", M);
   if (K <= 0 || K % 8) return me_fail("me_gemm_bf16_stream: K=%d must be a positive multiple of 8", K);
   if (!X || !W || !C) return me_fail("me_gemm_bf16_stream: null operand");
@@ -250,10 +251,10 @@ extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M,
   const int wn = me_gemm_bf16_stream_arrangement(M, N, splits, compute_units);
   const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
   if (swiglu)
-    launch_rows<true, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, stream);
+    launch_rows<true, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, swiglu, stream);
   else if (out_dtype == ME_F32)
-    launch_rows<false, float>(wn, x, w, (float*)C, M, N, K, splits, steps_per_split, stream);
+    launch_rows<false, float>(wn, x, w, (float*)C, M, N, K, splits, steps_per_split, 0, stream);
   else
-    launch_rows<false, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, stream);
+    launch_rows<false, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, 0, stream);
   return me_check_launch("me_gemm_bf16_stream");
 }

@@ -192,7 +192,7 @@ class Run {
         add_norm((const float*)op.p[0], op.f[0], bufs_[op.out]);
         break;
       case kOpLinear:
-        product(bufs_[op.in], op.p[1], (int)op.i[0], (int)op.i[1], op.i[2] != 0, dtype_, bufs_[op.out]);
+        product(bufs_[op.in], op.p[1], (int)op.i[0], (int)op.i[1], (int)op.i[2], dtype_, bufs_[op.out]);
         break;
       case kOpLinearDelta:
         linear_delta(op);
@@ -233,14 +233,14 @@ class Run {
   void norm_linear(const Op& op) {
     const float* w_norm = (const float*)op.p[0];
     const int rows_of_w = (int)op.i[0], k = (int)op.i[1];
-    const bool gated = op.i[2] != 0;
+    const int gated = (int)op.i[2];  // 0, or the code of the gate's activation
     if (k != h_) throw Error(kBadValue, "a product behind a norm reads the hidden size");
     const int n = gated ? rows_of_w / 2 : rows_of_w;
     // decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
     // residual buffer, since other blocks of the kernel still read the first
     if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts && !weight_bound(t_, rows_of_w, k)) {
       ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
-                            bufs_[op.out], t_, n, k, 1, gated ? 1 : 0, dtype_, 1, stream_));
+                            bufs_[op.out], t_, n, k, 1, gated, dtype_, 1, stream_));
       if (pending_.delta) std::swap(x_, spare_);
       pending_ = Pending();
       return;
@@ -249,8 +249,8 @@ class Run {
     product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
   }
 
-  // out = x . W^T (gated: silu(gate) * up with W = [gate rows; up rows]).
-  void product(const void* x, const void* w, int rows_of_w, int k, bool gated, int out_dtype, void* out) {
+  // out = x . W^T (gated, the code of an activation: act(gate) * up with W = [gate rows; up rows]).
+  void product(const void* x, const void* w, int rows_of_w, int k, int gated, int out_dtype, void* out) {
     const int m = t_rows_;
     const int n = gated ? rows_of_w / 2 : rows_of_w;
     if (dtype_ == kF32) {  // a true 32-bit product on the vector units, additions in ascending k
@@ -260,30 +260,30 @@ class Run {
       }
       float* both = (float*)arena_.take((size_t)m * rows_of_w * 4);
       ok(me_gemm_f32((const float*)x, (const float*)w, both, m, rows_of_w, k, stream_));
-      ok(me_swiglu(both, out, m, n, kF32, stream_));
+      ok(me_swiglu(both, out, m, n, gated, kF32, stream_));
       return;
     }
     const bool heavy = weight_bound(m, rows_of_w, k);
     if (heavy && m <= kSmallFastRows && (out_dtype == kBF16 || !gated)) {  // up to 16 rows it is ahead of the library too
-      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated ? 1 : 0, out_dtype, 1, compute_units(), stream_));
+      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
       return;
     }
     if (!heavy && m > kSmallFastRows && streams(m, rows_of_w, k) && (out_dtype == kBF16 || !gated)) {
-      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated ? 1 : 0, out_dtype, 1, compute_units(), stream_));
+      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
       return;
     }
     if (!heavy && small_serves(m, k)) {
-      ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, out, m, n, k, 0, gated ? 1 : 0, out_dtype, 1, stream_));
+      ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, out, m, n, k, 0, gated, out_dtype, 1, stream_));
       return;
     }
     if (gated) {
       if (m >= kTiledMinRows && k % 64 == 0 && out_dtype == kBF16) {  // ahead of the library product + SwiGLU kernel
-        ok(me_gemm_bf16_tiled(x, w, out, m, n, k, 1, out_dtype, 0, stream_));
+        ok(me_gemm_bf16_tiled(x, w, out, m, n, k, gated, out_dtype, 0, stream_));
         return;
       }
       void* both = arena_.take((size_t)m * rows_of_w * 2);
       library_product(x, w, both, m, rows_of_w, k, kBF16, stream_);
-      ok(me_swiglu(both, out, m, n, kBF16, stream_));
+      ok(me_swiglu(both, out, m, n, gated, kBF16, stream_));
       return;
     }
     library_product(x, w, out, m, n, k, out_dtype, stream_);
@@ -311,7 +311,7 @@ class Run {
       return;
     }
     const size_t mark = arena_.used;
-    product(x, op.p[1], n, k, false, dtype_, bufs_[op.out]);
+    product(x, op.p[1], n, k, 0, dtype_, bufs_[op.out]);
     arena_.used = mark;
     pending_.delta = bufs_[op.out];
   }

@@ -161,9 +161,13 @@ class StepProgram:
         self._want(weight, torch.float32, (self.hidden,), "norm weight")
         return Normed(self, weight, eps)
 
-    def linear(self, x, weight: torch.Tensor, gated: bool = False) -> int:
-        """``x @ weight.T`` (``gated``: ``silu(gate) * up`` with the weight's rows being gate rows, then up
-        rows) for a value or a :class:`Normed`; returns the value that holds the result."""
+    def linear(self, x, weight: torch.Tensor, gated: "bool | str" = False) -> int:
+        """``x @ weight.T`` (``gated``, True or the name of an activation: ``act(gate) * up`` with the weight's
+        rows being gate rows, then up rows) for a value or a :class:`Normed`; returns the value that holds
+        the result."""
+        from ..ops.kernels import gate_code
+
+        gate = gate_code(gated)
         rows, k = weight.shape
         self._want(weight, self.dtype, None, "weight")
         if gated and rows % 2:
@@ -172,14 +176,14 @@ class StepProgram:
         if isinstance(x, Normed) and x._value is None:
             if k != self.hidden:
                 raise ValueError("a product behind the norm reads the hidden size")
-            self.op(NORM_LINEAR, out=out, ptrs=[x.weight, weight], ints=[rows, k, int(gated)], floats=[x.eps])
+            self.op(NORM_LINEAR, out=out, ptrs=[x.weight, weight], ints=[rows, k, gate], floats=[x.eps])
             x.used = True
             self.pending_consumed()
             return out
         src = x.value() if isinstance(x, Normed) else x
         if self._value_kinds[src][0] != k:
             raise ValueError(f"the weight reads {k} columns, the value has {self._value_kinds[src][0]}")
-        self.op(LINEAR, in_=src, out=out, ptrs=[None, weight], ints=[rows, k, int(gated)])
+        self.op(LINEAR, in_=src, out=out, ptrs=[None, weight], ints=[rows, k, gate])
         return out
 
     def linear_delta(self, x: int, weight: torch.Tensor) -> None:

@@ -186,8 +186,22 @@ def rmsnorm(inp: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tens
     return out
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I]."""
+GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}  # the codes of the kernels' `gated` arguments (MeGate in csrc/common.h)
+
+
+def gate_code(gated) -> int:
+    """0 for a product that is not gated; else the code of the gate's activation. ``True`` means silu."""
+    if not gated:
+        return 0
+    if gated is True:
+        return GATE_ACTIVATIONS["silu"]
+    if gated not in GATE_ACTIVATIONS:
+        raise ValueError(f"unknown gate activation {gated!r}; known: {sorted(GATE_ACTIVATIONS)}")
+    return GATE_ACTIVATIONS[gated]
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None, activation: str = "silu") -> torch.Tensor:
+    """``act(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I]; ``activation`` is "silu" or "gelu_tanh"."""
     _want(gate_up, "gate_up", None, (None, None))
     t, two_i = gate_up.shape
     if two_i % 2:
@@ -196,7 +210,7 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tens
     if out is None:
         out = torch.empty((t, inter), dtype=gate_up.dtype, device=gate_up.device)
     _want(out, "out", gate_up.dtype, (t, inter))
-    check(lib().me_swiglu(_p(gate_up), _p(out), _i(t), _i(inter), _i(_code(gate_up.dtype)), _stream()))
+    check(lib().me_swiglu(_p(gate_up), _p(out), _i(t), _i(inter), _i(gate_code(activation)), _i(_code(gate_up.dtype)), _stream()))
     return out
 
 
@@ -396,7 +410,7 @@ def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=weight.device)
     _want(out, "out", out_dtype, shape)
-    check(lib().me_gemm_bf16_stream(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(1 if swiglu else 0),
+    check(lib().me_gemm_bf16_stream(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
                                     _i(_code(out_dtype)), _i(k_splits), _i(compute_units(x.device)), _stream()))
     return out
 
@@ -440,13 +454,13 @@ def gemm_bf16_small(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bflo
                 raise ValueError("the spare residual buffer must not alias the residual stream")
             x_out = x.spare
         check(lib().me_gemm_bf16_small(_p(None), _p(x.x), _p(x.delta), _p(x.weight), _f(x.eps), _p(x_out), _p(weight),
-                                       _p(out), _i(m), _i(n), _i(k), _i(1), _i(1 if swiglu else 0),
+                                       _p(out), _i(m), _i(n), _i(k), _i(1), _i(gate_code(swiglu)),
                                        _i(_code(out_dtype)), _i(1), _stream()))
         x.residual = x.x if x.delta is None else x.spare
     else:
         _want(x, "x", torch.bfloat16, (m, k))
         check(lib().me_gemm_bf16_small(_p(x), _p(None), _p(None), _p(None), _f(0.0), _p(None), _p(weight), _p(out),
-                                       _i(m), _i(n), _i(k), _i(0), _i(1 if swiglu else 0), _i(_code(out_dtype)),
+                                       _i(m), _i(n), _i(k), _i(0), _i(gate_code(swiglu)), _i(_code(out_dtype)),
                                        _i(k_splits), _stream()))
     return out
 
@@ -477,7 +491,7 @@ def gemm_bf16_tiled(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=weight.device)
     _want(out, "out", out_dtype, (m, n))
-    check(lib().me_gemm_bf16_tiled(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(1 if swiglu else 0),
+    check(lib().me_gemm_bf16_tiled(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
                                    _i(_code(out_dtype)), _i(shape), _stream()))
     return out
 
@@ -511,10 +525,10 @@ def streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False,
+def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: "bool | str" = False,
            as_delta: bool = False):
-    """``x @ weight.T`` for x [M, K], weight [N, K]; with ``gated`` the weight is [2N, K] (gate rows,
-    then up rows) and the result is ``silu(gate) * up``. ``x`` may be a :class:`NormedInput`. With
+    """``x @ weight.T`` for x [M, K], weight [N, K]; with ``gated`` (True or "silu", or "gelu_tanh") the
+    weight is [2N, K] (gate rows, then up rows) and the result is ``act(gate) * up``. ``x`` may be a :class:`NormedInput`. With
     ``as_delta`` the caller says that the result only ever is the pending delta of the residual stream
     (what a mixer or a feed-forward returns): it may then come back as :class:`PartialSums`, which
     :func:`add_rmsnorm` adds up on the way.
@@ -534,7 +548,7 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         if out_dtype is not torch.float32:
             raise TypeError("the float32 path keeps float32 results")
         y = gemm_f32(x, weight)
-        return swiglu(y) if gated else y
+        return swiglu(y, activation="silu" if gated is True else gated) if gated else y
     heavy, few = weight_bound(x, weight), x.shape[0] <= SMALL_FAST_ROWS
     if as_delta and not gated and (heavy or (not few and streams(x, weight))):
         splits = stream_splits(weight.shape[0], x.shape[1], x.device)
@@ -547,8 +561,8 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if gated:
         if tiled_ok(x, weight) and out_dtype is torch.bfloat16:
-            return gemm_bf16_tiled(x, weight, out_dtype, True)  # measured ahead of the library product + SwiGLU kernel
-        return swiglu(linear(x, weight, out_dtype))
+            return gemm_bf16_tiled(x, weight, out_dtype, gated)  # measured ahead of the library product + SwiGLU kernel
+        return swiglu(linear(x, weight, out_dtype), activation="silu" if gated is True else gated)
     return gemm_bf16_library(x, weight, out_dtype)
 
 

@@ -1,6 +1,7 @@
 """Dense gated feed-forward: ``down(act(gate(x)) * up(x))`` without biases
 (reference: ``src/mini_engine/model.py:122-131``). Gate and up weights are stacked at load time so
-that one product feeds the activation kernel."""
+that one product feeds the activation, which is the epilogue of that product where a kernel of this
+package computes it (silu as in the reference, or the tanh form of gelu)."""
 
 from __future__ import annotations
 
@@ -16,8 +17,8 @@ class GatedMlp(FeedForward):
 
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
-        if spec.activation != "silu":
-            raise ValueError(f"gated_mlp supports the silu activation, got {spec.activation!r}")
+        if spec.activation not in K.GATE_ACTIVATIONS:
+            raise ValueError(f"gated_mlp knows the activations {sorted(K.GATE_ACTIVATIONS)}, got {spec.activation!r}")
         self.w_gate_up = self.w_down = None
 
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
@@ -35,11 +36,11 @@ class GatedMlp(FeedForward):
     takes_normed_input = True
 
     def forward(self, h, batch=None) -> torch.Tensor:
-        act = K.linear(h, self.w_gate_up, gated=True)
+        act = K.linear(h, self.w_gate_up, gated=self.spec.activation)
         return K.linear(act, self.w_down, as_delta=True)
 
     def emit(self, program, h) -> None:
-        act = program.linear(h, self.w_gate_up, gated=True)
+        act = program.linear(h, self.w_gate_up, gated=self.spec.activation)
         program.linear_delta(act, self.w_down)
 
 

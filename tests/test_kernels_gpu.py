@@ -72,9 +72,29 @@ def test_rmsnorm_rows(dtype):
 @pytest.mark.parametrize("tokens,inter", [(7, 160), (3, 1001)])
 def test_swiglu(dtype, tokens, inter):
     gu = (torch.randn(tokens, 2 * inter) * 2).to(dtype)
-    out = K().swiglu(dev(gu))
     g, u = gu.float()[:, :inter], gu.float()[:, inter:]
-    torch.testing.assert_close(out.float().cpu(), plain.silu(g) * u, **tol(dtype))
+    torch.testing.assert_close(K().swiglu(dev(gu)).float().cpu(), plain.silu(g) * u, **tol(dtype))
+    gelu = K().swiglu(dev(gu), activation="gelu_tanh").float().cpu()
+    torch.testing.assert_close(gelu, torch.nn.functional.gelu(g, approximate="tanh") * u, **tol(dtype))
+    with pytest.raises(ValueError, match="activation"):
+        K().swiglu(dev(gu), activation="relu")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [2, 16, 33, 64, 130, 300])
+def test_gated_products_with_either_activation(dtype, rows):
+    """``linear(..., gated=name)`` at the row counts of every kernel that computes the gate as its epilogue
+    (the small and the streaming kernel, the tiled one) or after a library product, against the formula."""
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn(rows, 128, generator=g).to(dtype)
+    w = (torch.randn(2 * 200, 128, generator=g) * 0.1).to(dtype)
+    y = x.float() @ w.float().T
+    for name, act in (("silu", plain.silu), ("gelu_tanh", lambda z: torch.nn.functional.gelu(z, approximate="tanh"))):
+        want = act(y[:, :200]) * y[:, 200:]
+        got = K().linear(dev(x), dev(w), gated=name).float().cpu()
+        t = tol(dtype)
+        torch.testing.assert_close(got, want, rtol=t["rtol"], atol=t["atol"] * max(1.0, want.abs().max().item()))
+    assert (act(y[:, :200]) - plain.silu(y[:, :200])).abs().max() > 0.05  # the two activations differ at these values
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 50, 33), (5, 130, 72), (70, 64, 100), (129, 257, 48)])

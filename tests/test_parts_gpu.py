@@ -152,16 +152,24 @@ def test_gated_mlp_part(dtype):
     from mini_engine_amd.parts import FEED_FORWARDS
 
     dt = TORCH[dtype]
-    ffn = FEED_FORWARDS.build(GatedMlpSpec(hidden_size=72, intermediate_size=200), dt, torch.device("cuda"))
-    w = {n: (0.2 * torch.randn(want.shape)).to(dt).float() for n, want in ffn.weight_wants("m").items()}
-    ffn.load({k: v.cuda().to(dt) for k, v in w.items()}, "m")
-    for rows in (3, 150):
-        x = torch.randn(rows, 72).to(dt)
-        want = plain.swiglu_mlp(x.float(), w, "m")
-        scale = max(1.0, want.abs().max().item())  # bfloat16 rounding is relative to the values' size
-        t = tol(dtype)
-        torch.testing.assert_close(ffn.forward(x.cuda()).float().cpu(), want, rtol=t["rtol"], atol=t["atol"] * scale)
-    with pytest.raises(ValueError, match="silu"):
+    for activation in ("silu", "gelu_tanh"):
+        ffn = FEED_FORWARDS.build(GatedMlpSpec(hidden_size=72, intermediate_size=200, activation=activation), dt,
+                                  torch.device("cuda"))
+        w = {n: (0.2 * torch.randn(want.shape)).to(dt).float() for n, want in ffn.weight_wants("m").items()}
+        ffn.load({k: v.cuda().to(dt) for k, v in w.items()}, "m")
+        for rows in (3, 40, 150):
+            x = torch.randn(rows, 72).to(dt)
+            if activation == "silu":
+                want = plain.swiglu_mlp(x.float(), w, "m")
+            else:
+                gate = torch.nn.functional.gelu(x.float() @ w["m.gate_proj.weight"].T, approximate="tanh")
+                want = (gate * (x.float() @ w["m.up_proj.weight"].T)) @ w["m.down_proj.weight"].T
+            scale = max(1.0, want.abs().max().item())  # bfloat16 rounding is relative to the values' size
+            t = tol(dtype)
+            out = ffn.forward(x.cuda())
+            out = out.to_tensor(dt) if hasattr(out, "to_tensor") else out  # a delta may come back as partial sums
+            torch.testing.assert_close(out.float().cpu(), want, rtol=t["rtol"], atol=t["atol"] * scale)
+    with pytest.raises(ValueError, match="activations"):
         FEED_FORWARDS.build(GatedMlpSpec(hidden_size=8, intermediate_size=8, activation="gelu"), dt, torch.device("cuda"))
 
 

@@ -490,9 +490,12 @@ def test_capturable_toy_parts_replay_from_graphs(graphs):
     assert bm.slots.in_use == set()
 
 
-def test_embedding_multiplier_and_logit_scale_in_the_native_step(tiny_folders):
-    """The plan's two scales through the native step program, in both dtypes, against the plain
-    implementation with a scaled embedding table and scaled logits (B's head is not tied)."""
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+def test_plan_scales_and_gate_activation_in_the_native_step(tiny_folders, activation, monkeypatch):
+    """The plan's two scales and the feed-forward's other activation through the native step program, in
+    both dtypes, against the plain implementation with a scaled embedding table, scaled logits and the
+    activation swapped (B's head is not tied). Portions of 33 and 5 tokens and single tokens: the gate is the
+    epilogue of the small and of the streaming product, and follows a library product."""
     import dataclasses
 
     import plain_qwen3 as plain
@@ -508,10 +511,13 @@ def test_embedding_multiplier_and_logit_scale_in_the_native_step(tiny_folders):
 
     folder = tiny_folders["B"]
     _, plan = plan_from_folder(folder)
-    plan = dataclasses.replace(plan, embedding_multiplier=3.0, logit_scale=0.5)
+    layers = tuple(dataclasses.replace(l, ffn=dataclasses.replace(l.ffn, activation=activation)) for l in plan.layers)
+    plan = dataclasses.replace(plan, layers=layers, embedding_multiplier=3.0, logit_scale=0.5)
     pcfg, w = plain.read_config(folder), plain.read_weights(folder)
     w["model.embed_tokens.weight"] = 3.0 * w["model.embed_tokens.weight"]
     tokens = random_prompt(40, pcfg.vocab_size, seed=12)
+    if activation == "gelu_tanh":
+        monkeypatch.setattr(plain, "silu", lambda z: torch.nn.functional.gelu(z, approximate="tanh"))
     want = 0.5 * plain.forward_logits(w, pcfg, tokens)
     for dtype in ("float32", "bfloat16"):
         model = Decoder(plan, TORCH_DTYPES[dtype], "cuda")
@@ -525,4 +531,4 @@ def test_embedding_multiplier_and_logit_scale_in_the_native_step(tiny_folders):
             got.append(engine.runner.step([StepItem(seq, tokens[lo : lo + n], lo, list(range(n)))]).float().cpu())
             seq.num_computed_tokens += n
         engine.block_manager.free(seq)
-        th.assert_logits_close(torch.cat(got), want, dtype, f"scaled embedding and logits, {dtype}")
+        th.assert_logits_close(torch.cat(got), want, dtype, f"scaled embedding and logits, {activation}, {dtype}")
