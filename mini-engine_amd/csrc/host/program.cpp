@@ -18,6 +18,9 @@ constexpr int kF32 = 0, kBF16 = 1;
 constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
 constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
 constexpr int kTiledMinRows = 256;
+constexpr int kHeadStreamRows = 32;  // the head's logits (float32) come from the weight-streaming kernel up to here: at 151,936
+                                     // rows of 1,024 / 4,096 / 5,120 it takes 62-75 / 245-272 / 291-341 us at 8 to 32 rows,
+                                     // the library 62-79 / 260-276 / 319-362; from 48 rows on the library is ahead
 constexpr int kDecodeWaves = 1024;  // waves that a decode attention launch aims at (four per compute unit of 256)
 constexpr int64_t kStreamMinElements = 8ll << 20;  // weights from 16 MiB on: streaming them is the product's time
 constexpr int64_t kStreamMaxBytes = 1ll << 31;     // what the weight-streaming kernel addresses
@@ -48,12 +51,15 @@ struct Pending {
 };
 
 // Which kernel serves a bfloat16 product of m rows (measured on the layer sizes of a 0.6B, an 8B and a 32B model):
-//   up to 16 rows, weights below 16 MiB: the small matrix-core kernel, the residual add and the norm as its prologue
-//     (a launch less; at these sizes a launch is most of a kernel's time);
+//   up to 16 rows, weights below 16 MiB: the small matrix-core kernel; the residual add and the norm are its prologue
+//     where the delta in front is a tensor (a product whose k was not cut);
 //   17 to 64 rows, weights below 16 MiB: the weight-streaming kernel (qkv 5.0-6.7 us, gate/up with SwiGLU 6.6-9.3
 //     against 5.8-7.7 and 7.5-10.3 with the small kernel, 8.2-8.6 and 14.4-14.7 with the library and a SwiGLU kernel);
-//   a delta of the residual stream from 17 rows on, or of a large weight: the weight-streaming kernel with k cut
-//     into runs whose partial sums the next add-and-norm adds up (1,024 columns: 3.9-5.3 us against 7.9-16 and 7.6-9.8);
+//   a delta of the residual stream, at any row count up to 64: the weight-streaming kernel with k cut into runs, so
+//     that every compute unit streams a part of the weight (1,024 columns, 1 to 16 rows: 3.5 and 4.3 us against 4.7-6.1
+//     and 5.8-7.8 with the small kernel; 17 to 64 rows: 3.9-5.3 against 7.9-16 and 7.6-9.8). The add-and-norm behind
+//     it, a kernel of its own (2.9 us), adds the partial sums up; as the prologue of the next product, where every
+//     block would read them, they cost more at every row count (one row: 853 -> 820 tokens/s);
 //   everything else: the GEMM library, as the reference hands every projection to one.
 bool small_serves(int m, int k) { return k % 8 == 0 && m <= kSmallFastRows; }
 
@@ -295,7 +301,7 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
-    if (dtype_ == kBF16 && (weight_bound(t_, n, k) || (t_ > kSmallFastRows && streams(t_, n, k)))) {
+    if (dtype_ == kBF16 && streams(t_, n, k)) {
       const int splits = me_gemm_bf16_stream_splits(n, k, compute_units());
       if (splits > 1) {
         parts_mark_ = arena_.used;
@@ -402,7 +408,7 @@ class Run {
     float* logits = (float*)arena_.take((size_t)rows * vocab * 4);
     if (dtype_ == kF32)
       ok(me_gemm_f32((const float*)picked, (const float*)op.p[1], logits, rows, vocab, h_, stream_));
-    else if (rows > 2 && rows <= kSmallFastRows && weight_bound(rows, vocab, h_))  // 58-61 us against 63-71 at 8 to 16 rows
+    else if (rows > 2 && rows <= kHeadStreamRows && weight_bound(rows, vocab, h_))  // ahead of the small kernel and the library
       ok(me_gemm_bf16_stream(picked, op.p[1], logits, rows, vocab, h_, 0, kF32, 1, compute_units(), stream_));
     else if (rows <= kSmallFastRows && h_ % 8 == 0)
       ok(me_gemm_bf16_small(picked, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], logits, rows, vocab, h_, 0, 0, kF32, 1, stream_));

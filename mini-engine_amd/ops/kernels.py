@@ -507,6 +507,7 @@ def small_ok(x, weight: torch.Tensor, gated: bool = False) -> bool:
     return x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and x.shape[0] <= SMALL_FAST_ROWS
 
 
+HEAD_STREAM_ROWS = 32  # float32 products of large weights (a head's logits) stay with the weight-streaming kernel up to here
 STREAM_MIN_ELEMENTS = 8 << 20  # weights from 16 MiB on: streaming them is the product's time
 STREAM_MAX_BYTES = 1 << 31  # what the weight-streaming kernel addresses
 
@@ -537,7 +538,7 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     weight size as ``csrc/host/program.cpp`` chooses (where the measurements are): up to 16 rows the small
     matrix-core kernel, or the weight-streaming one for weights of 16 MiB and more; 17 to 64 rows the
     weight-streaming kernel (the library for weights of 16 MiB and more); a delta of the residual stream
-    from 17 rows on, or of a large weight, as partial sums over runs of k; the tiled matrix-core kernel with
+    of up to 64 rows as partial sums over runs of k; the tiled matrix-core kernel with
     the SwiGLU as its epilogue for gated products of 256 rows or more; else the GEMM library."""
     if isinstance(x, NormedInput):
         if x.fusable(weight):
@@ -550,13 +551,15 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         y = gemm_f32(x, weight)
         return swiglu(y, activation="silu" if gated is True else gated) if gated else y
     heavy, few = weight_bound(x, weight), x.shape[0] <= SMALL_FAST_ROWS
-    if as_delta and not gated and (heavy or (not few and streams(x, weight))):
+    if as_delta and not gated and streams(x, weight):
         splits = stream_splits(weight.shape[0], x.shape[1], x.device)
         if splits > 1:
             return PartialSums(gemm_bf16_stream(x, weight, torch.float32, k_splits=splits))
         return gemm_bf16_stream(x, weight, out_dtype)
     if (heavy if few else streams(x, weight) and not heavy) and (out_dtype is torch.bfloat16 or not gated):
         return gemm_bf16_stream(x, weight, out_dtype, gated)
+    if heavy and x.shape[0] <= HEAD_STREAM_ROWS and out_dtype is torch.float32 and not gated:  # a head's logits
+        return gemm_bf16_stream(x, weight, out_dtype)
     if small_ok(x, weight, gated) and not heavy:
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if gated:

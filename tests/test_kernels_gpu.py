@@ -212,7 +212,11 @@ def test_linear_hands_back_partial_sums_only_when_asked():
     delta = K().linear(x, w, as_delta=True)
     assert isinstance(delta, K().PartialSums) and delta.shape == (40, 1024)
     torch.testing.assert_close(delta.to_tensor(torch.bfloat16).float(), plain_out.float(), rtol=2e-2, atol=2e-2)
-    assert isinstance(K().linear(x[:8], w, as_delta=True), torch.Tensor)  # up to 16 rows: the fused kernel
+    few = K().linear(x[:8].contiguous(), w, as_delta=True)  # few rows too: k is cut so that every compute unit streams
+    assert isinstance(few, K().PartialSums) and few.shape == (8, 1024)
+    torch.testing.assert_close(few.to_tensor(torch.bfloat16).float(), plain_out[:8].float(), rtol=2e-2, atol=2e-2)
+    narrow = dev((torch.randn(1024, 2048 - 4) * 0.02).bfloat16())  # k no multiple of 8: not the streaming kernel's
+    assert isinstance(K().linear(x[:, :2044].contiguous(), narrow, as_delta=True), torch.Tensor)
 
 
 def test_gemm_f32_rows_do_not_depend_on_the_batch():
