@@ -18,6 +18,10 @@ constexpr int kF32 = 0, kBF16 = 1;
 constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
 constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
 constexpr int kTiledMinRows = 256;
+constexpr int kTiledMaxK = 3072;  // gate/up with the SwiGLU as the tiled kernel's epilogue against the library's product and a
+                                  // SwiGLU kernel: at k = 1,024 (3,072 columns) 15-62 us against 21-67 for 512 to 4,096 rows; at
+                                  // k = 4,096 (12,288 columns) 95-729 against 89-640; at k = 5,120 (25,600) 345-1,973 against
+                                  // 293-1,767: the longer k is, the less a pass over the output weighs against the product
 constexpr int kHeadStreamRows = 32;  // the head's logits (float32) come from the weight-streaming kernel up to here: at 151,936
                                      // rows of 1,024 / 4,096 / 5,120 it takes 62-75 / 245-272 / 291-341 us at 8 to 32 rows,
                                      // the library 62-79 / 260-276 / 319-362; from 48 rows on the library is ahead
@@ -283,7 +287,7 @@ class Run {
       return;
     }
     if (gated) {
-      if (m >= kTiledMinRows && k % 64 == 0 && out_dtype == kBF16) {  // ahead of the library product + SwiGLU kernel
+      if (m >= kTiledMinRows && k % 64 == 0 && k <= kTiledMaxK && out_dtype == kBF16) {  // ahead of the library product + SwiGLU kernel
         ok(me_gemm_bf16_tiled(x, w, out, m, n, k, gated, out_dtype, 0, stream_));
         return;
       }

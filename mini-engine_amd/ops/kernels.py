@@ -507,6 +507,7 @@ def small_ok(x, weight: torch.Tensor, gated: bool = False) -> bool:
     return x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and x.shape[0] <= SMALL_FAST_ROWS
 
 
+TILED_MAX_K = 3072  # gated products of longer k go to the library and a SwiGLU kernel (measured in csrc/host/program.cpp)
 HEAD_STREAM_ROWS = 32  # float32 products of large weights (a head's logits) stay with the weight-streaming kernel up to here
 STREAM_MIN_ELEMENTS = 8 << 20  # weights from 16 MiB on: streaming them is the product's time
 STREAM_MAX_BYTES = 1 << 31  # what the weight-streaming kernel addresses
@@ -563,7 +564,7 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     if small_ok(x, weight, gated) and not heavy:
         return gemm_bf16_small(x, weight, out_dtype, gated)
     if gated:
-        if tiled_ok(x, weight) and out_dtype is torch.bfloat16:
+        if tiled_ok(x, weight) and x.shape[1] <= TILED_MAX_K and out_dtype is torch.bfloat16:
             return gemm_bf16_tiled(x, weight, out_dtype, gated)  # measured ahead of the library product + SwiGLU kernel
         return swiglu(linear(x, weight, out_dtype), activation="silu" if gated is True else gated)
     return gemm_bf16_library(x, weight, out_dtype)
