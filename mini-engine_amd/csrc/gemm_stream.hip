@@ -17,6 +17,8 @@
 // wave (W = [gate rows; up rows]) and writes silu(gate) * up.
 #include "common.h"
 
+#include <algorithm>
+
 typedef __bf16 sbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float sfloat4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t suint4_t __attribute__((ext_vector_type(4)));
@@ -177,6 +179,174 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   }
 }
 
+// The same product for a row or a few with the residual add and the RMSNorm in front of it as its prologue:
+// the input is the float32 residual stream x_in [M, K] plus a delta (a bfloat16 tensor, or float32 partial sums
+// of the product before, added in the order of their runs, or nothing). While the weights of the first steps
+// are on their way, the block forms s = x_in + delta, keeps bf16(s * w_norm) of every row in LDS for the whole
+// of k (no rows of x are fetched in the loop) and sums s^2; the results are multiplied by
+// rsqrt(mean(s^2) + eps) at the end (a row's scale is a common factor of its products). Block 0 writes s to
+// x_out, which must not alias x_in: the other blocks still read it. Every block reads all of x_in and the partial
+// sums, so this is for a row or two; no runs of k across blocks.
+template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES>
+__global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+                                                               const float* __restrict__ parts, int num_parts, size_t part_stride,
+                                                               const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
+                                                               const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N,
+                                                               int K, int gate) {
+  static_assert(WN * WK == 4, "four waves per block");
+  constexpr int KC = kStepK / WK, CH = KC / 32, ACCS = SWIGLU ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char norm_lds[];
+  const int krow = K + 8;  // elements per row of normed x: rows start 16 bytes apart modulo the banks
+  uint16_t* xn = reinterpret_cast<uint16_t*>(norm_lds);                                  // [M][krow]
+  float* sums = reinterpret_cast<float*>(norm_lds + (((size_t)M * krow * 2 + 15) & ~(size_t)15));  // [M][4 waves], then [M]
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int wn = wave % WN, wk = wave / WN;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = (blockIdx.x * WN + wn) * 16;
+  const int n = n0 + r;
+  const int steps = (K + kStepK - 1) / kStepK;
+
+  const uint32_t w_bytes = (uint32_t)((size_t)(SWIGLU ? 2 : 1) * N * K * 2);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(W), 0, w_bytes, kBufferFlags);
+  uint32_t w_base[ACCS];
+#pragma unroll
+  for (int a = 0; a < ACCS; ++a) w_base[a] = n < N ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
+  suint4_t w[STAGES][ACCS][CH];
+  auto load_step = [&](int step, suint4_t (&wd)[ACCS][CH]) {
+    const int k0 = step * kStepK;
+#pragma unroll
+    for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int k = k0 + wk * KC + g * 8 + 32 * c;
+        wd[a][c] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, k < K ? (int)(w_base[a] + (k0 + 32 * c) * 2) : (int)w_bytes, 0, 0);
+      }
+  };
+#pragma unroll
+  for (int p = 0; p < STAGES; ++p) {
+    load_step(p, w[p]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // ---- the prologue: every row's sum, its squares, and bf16(s * w_norm) into LDS
+  const bool writes_x = blockIdx.x == 0 && (delta != nullptr || parts != nullptr);
+  for (int m = 0; m < M; ++m) {
+    float ss = 0.f;
+    for (int v = threadIdx.x; v < K / 4; v += 256) {
+      const size_t at = (size_t)m * K + 4 * v;
+      float4 sv = *reinterpret_cast<const float4*>(x_in + at);
+      if (delta) {
+        const uint2 dv = *reinterpret_cast<const uint2*>(delta + at);
+        sv.x += __uint_as_float(dv.x << 16), sv.y += __uint_as_float(dv.x & 0xffff0000u);
+        sv.z += __uint_as_float(dv.y << 16), sv.w += __uint_as_float(dv.y & 0xffff0000u);
+      }
+      if (parts) {  // in the order of the runs
+        float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+        int q = 0;
+        for (; q + 4 <= num_parts; q += 4) {
+          const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)q * part_stride + at);
+          const float4 b = *reinterpret_cast<const float4*>(parts + (size_t)(q + 1) * part_stride + at);
+          const float4 c = *reinterpret_cast<const float4*>(parts + (size_t)(q + 2) * part_stride + at);
+          const float4 e = *reinterpret_cast<const float4*>(parts + (size_t)(q + 3) * part_stride + at);
+          d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
+          d.x += b.x, d.y += b.y, d.z += b.z, d.w += b.w;
+          d.x += c.x, d.y += c.y, d.z += c.z, d.w += c.w;
+          d.x += e.x, d.y += e.y, d.z += e.z, d.w += e.w;
+        }
+        for (; q < num_parts; ++q) {
+          const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)q * part_stride + at);
+          d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
+        }
+        sv.x += d.x, sv.y += d.y, sv.z += d.z, sv.w += d.w;
+      }
+      if (writes_x) *reinterpret_cast<float4*>(x_out + at) = sv;
+      ss = fmaf(sv.x, sv.x, ss), ss = fmaf(sv.y, sv.y, ss), ss = fmaf(sv.z, sv.z, ss), ss = fmaf(sv.w, sv.w, ss);
+      const float4 wv = *reinterpret_cast<const float4*>(w_norm + 4 * v);
+      uint2 packed;
+      packed.x = (uint32_t)f32_to_bf16_bits(sv.x * wv.x) | ((uint32_t)f32_to_bf16_bits(sv.y * wv.y) << 16);
+      packed.y = (uint32_t)f32_to_bf16_bits(sv.z * wv.z) | ((uint32_t)f32_to_bf16_bits(sv.w * wv.w) << 16);
+      *reinterpret_cast<uint2*>(xn + (size_t)m * krow + 4 * v) = packed;
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) sums[m * 4 + wave] = ss;
+  }
+  __syncthreads();
+  // rows beyond M read row M - 1 and count for nothing: their results are never stored
+  const uint16_t* xrow = xn + (size_t)min(r, M - 1) * krow + wk * KC + g * 8;
+
+  sfloat4_t acc[ACCS];
+#pragma unroll
+  for (int a = 0; a < ACCS; ++a) acc[a] = (sfloat4_t){0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < steps; s0 += STAGES) {  // the last round may run up to STAGES - 1 steps of zero weights
+#pragma unroll
+    for (int u = 0; u < STAGES; ++u) {
+      const int k0 = min(s0 + u, steps - 1) * kStepK;  // (steps past the end multiply zeros with the last step's rows)
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        sbf16x8_t b = sbf16x8_t{};
+        if (k0 + wk * KC + 32 * c + g * 8 < K) b = *reinterpret_cast<const sbf16x8_t*>(xrow + k0 + 32 * c);
+#pragma unroll
+        for (int a = 0; a < ACCS; ++a)
+          acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sbf16x8_t, w[u][a][c]), b, acc[a], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      load_step(s0 + u + STAGES, w[u]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  if (WK > 1) {  // the runs of k within a step: waves wk > 0 hand their sums to wave wk == 0 of their columns
+    __syncthreads();  // every wave has left the rows of x, whose memory the sums take
+    float* red = reinterpret_cast<float*>(norm_lds) + 64;  // [wk - 1][wn][a][j][lane], behind the rows' sums of squares
+    float* keep = reinterpret_cast<float*>(norm_lds);      // [M][4]
+    if (threadIdx.x < M * 4) keep[threadIdx.x] = sums[threadIdx.x];  // (M <= 16; read before, written after a barrier)
+    constexpr int PER_WAVE = ACCS * 4 * 64;
+    __syncthreads();
+    sums = keep;
+    if (wk > 0) {
+      float* mine = red + ((wk - 1) * WN + wn) * PER_WAVE;
+#pragma unroll
+      for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mine[(a * 4 + j) * 64 + lane] = acc[a][j];
+    }
+    __syncthreads();
+    if (wk > 0) return;
+#pragma unroll
+    for (int o = 1; o < WK; ++o) {
+      const float* theirs = red + ((o - 1) * WN + wn) * PER_WAVE;
+#pragma unroll
+      for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[a][j] += theirs[(a * 4 + j) * 64 + lane];
+    }
+  }
+  const int m = r, nb = n0 + 4 * g;
+  if (m >= M) return;
+  const float scale = rsqrtf(((sums[m * 4] + sums[m * 4 + 1]) + (sums[m * 4 + 2] + sums[m * 4 + 3])) / (float)K + eps);
+  float y[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    y[j] = acc[0][j] * scale;
+    if (SWIGLU) y[j] = gate_act(y[j], gate) * (acc[1][j] * scale);
+  }
+  OutT* dst = C + (size_t)m * N + nb;
+  if (nb + 3 < N && (N & 3) == 0) {
+    if (sizeof(OutT) == 4) {
+      *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
+    } else {
+      uint2 packed;
+      packed.x = (uint32_t)f32_to_bf16_bits(y[0]) | ((uint32_t)f32_to_bf16_bits(y[1]) << 16);
+      packed.y = (uint32_t)f32_to_bf16_bits(y[2]) | ((uint32_t)f32_to_bf16_bits(y[3]) << 16);
+      *reinterpret_cast<uint2*>(dst) = packed;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (nb + j < N) dst[j] = from_float<OutT>(y[j]);
+  }
+}
+
 template <int MT, bool SWIGLU, typename OutT>
 void launch_arranged(int wn, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int splits, int steps_per_split,
                      int gate, hipStream_t stream) {
@@ -257,4 +427,70 @@ extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M,
   else
     launch_rows<false, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, 0, stream);
   return me_check_launch("me_gemm_bf16_stream");
+}
+
+namespace {
+
+template <bool SWIGLU, typename OutT>
+int launch_norm(int wn, const float* x_in, const bf16_t* delta, const float* parts, int num_parts, size_t part_stride,
+                const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K, int gate,
+                hipStream_t stream) {
+  const dim3 grid(((N + 15) / 16 + wn - 1) / wn);
+  const int wk = 4 / wn;
+  const size_t rows_bytes = (((size_t)M * (K + 8) * 2 + 15) & ~(size_t)15) + (size_t)M * 4 * sizeof(float);
+  const size_t sums_bytes = (64 + (size_t)(wk - 1) * wn * (SWIGLU ? 2 : 1) * 4 * 64) * sizeof(float);
+  const size_t lds = std::max(rows_bytes, sums_bytes);
+  if (lds > 48 * 1024) return me_fail("me_gemm_bf16_stream_norm: %d rows of %d do not fit the block's memory", M, K);
+#define ME_NORM_LAUNCH(WN, WK, STAGES)                                                                                   \
+  gemm_stream_norm_kernel<WN, WK, SWIGLU, OutT, STAGES><<<grid, 256, lds, stream>>>(x_in, delta, parts, num_parts, part_stride, \
+                                                                                    w_norm, eps, x_out, W, C, M, N, K, gate)
+  if (wn == 4)
+    ME_NORM_LAUNCH(4, 1, (SWIGLU ? 2 : 3));
+  else if (wn == 2)
+    ME_NORM_LAUNCH(2, 2, (SWIGLU ? 3 : 4));
+  else
+    ME_NORM_LAUNCH(1, 4, (SWIGLU ? 4 : 6));
+#undef ME_NORM_LAUNCH
+  return me_check_launch("me_gemm_bf16_stream_norm");
+}
+
+}  // namespace
+
+// Whether me_gemm_bf16_stream_norm takes M rows of K: all rows of the normed input stay in the block's memory.
+extern "C" int me_gemm_bf16_stream_norm_fits(int M, int K) {
+  return M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && (size_t)M * (K + 8) * 2 + 16 + (size_t)M * 16 <= 48 * 1024;
+}
+
+// C[M, N] = rmsnorm(x_in + delta) * w_norm . W^T for a row or a few (M <= 16; every block reads all of x_in and of the
+// delta), with the gate as in me_gemm_bf16_stream. x_in float32 [M, K]; the delta is `delta` (bfloat16 [M, K]) or `parts`
+// (float32 [num_parts] of [M, K], part_stride elements apart, added in their order) or neither; with a delta the sum
+// is written to x_out (float32 [M, K], not aliasing x_in). w_norm float32 [K].
+extern "C" int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, const float* parts, int num_parts,
+                                        long long part_stride, const float* w_norm, float eps, float* x_out, const void* W,
+                                        void* C, int M, int N, int K, int swiglu, int out_dtype, int compute_units,
+                                        hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_stream_norm: unknown gate activation %d", swiglu);
+  if (!me_gemm_bf16_stream_norm_fits(M, K)) return me_fail("me_gemm_bf16_stream_norm: M=%d rows of K=%d are not taken", M, K);
+  if (!x_in || !w_norm || !W || !C) return me_fail("me_gemm_bf16_stream_norm: null operand");
+  if (delta && parts) return me_fail("me_gemm_bf16_stream_norm: a delta or partial sums, not both");
+  if ((delta || parts) && (!x_out || x_out == x_in))
+    return me_fail("me_gemm_bf16_stream_norm: x_out must be given and must not alias x_in");
+  if (parts && (num_parts < 1 || part_stride < (long long)M * K || part_stride % 4))
+    return me_fail("me_gemm_bf16_stream_norm: %d partial sums %lld elements apart for %d rows of %d", num_parts, part_stride, M, K);
+  if (((uintptr_t)x_in | (uintptr_t)parts | (uintptr_t)w_norm | (uintptr_t)x_out | (uintptr_t)W | (uintptr_t)C) & 15 || (uintptr_t)delta & 7)
+    return me_fail("me_gemm_bf16_stream_norm: operands must be 16-byte aligned");
+  if (out_dtype != ME_BF16 && out_dtype != ME_F32) return me_fail("me_gemm_bf16_stream_norm: output type %d", out_dtype);
+  if (swiglu && out_dtype != ME_BF16) return me_fail("me_gemm_bf16_stream_norm: the gated form writes bfloat16");
+  if ((size_t)(swiglu ? 2 : 1) * N * K * 2 >= (1ull << 31))
+    return me_fail("me_gemm_bf16_stream_norm: weights of 2 GiB and more are not addressed by this kernel");
+  if (compute_units < 1) compute_units = 256;
+  const int wn = me_gemm_bf16_stream_arrangement(M, N, 1, compute_units);
+  const bf16_t *d = (const bf16_t*)delta, *w = (const bf16_t*)W;
+  const size_t stride = parts ? (size_t)part_stride : 0;
+  if (swiglu)
+    return launch_norm<true, bf16_t>(wn, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, swiglu, stream);
+  if (out_dtype == ME_F32)
+    return launch_norm<false, float>(wn, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (float*)C, M, N, K, 0, stream);
+  return launch_norm<false, bf16_t>(wn, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, 0, stream);
 }

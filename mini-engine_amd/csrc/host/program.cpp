@@ -17,6 +17,7 @@ namespace {
 constexpr int kF32 = 0, kBF16 = 1;
 constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
 constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
+constexpr int kNormStreamRows = 2;   // up to here the add-and-norm is the prologue of the weight-streaming kernel
 constexpr int kTiledMinRows = 256;
 constexpr int kTiledMaxK = 3072;  // gate/up with the SwiGLU as the tiled kernel's epilogue against the library's product and a
                                   // SwiGLU kernel: at k = 1,024 (3,072 columns) 15-62 us against 21-67 for 512 to 4,096 rows; at
@@ -248,6 +249,18 @@ class Run {
     const int n = gated ? rows_of_w / 2 : rows_of_w;
     // decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
     // residual buffer, since other blocks of the kernel still read the first
+    // a row or two: the weight-streaming kernel adds and norms the rows itself while its first weights are on their
+    // way, whatever the delta is (one row: 857 -> 967 tokens/s, two: 1,605 -> 1,700; from four rows on every block's
+    // reads of the partial sums cost more than the launch they save: 2,749 -> 2,668)
+    if (dtype_ == kBF16 && t_ <= kNormStreamRows && me_gemm_bf16_stream_norm_fits(t_, k) && streams(t_, rows_of_w, k)) {
+      const bool adds = pending_.any();
+      ok(me_gemm_bf16_stream_norm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w_norm, op.f[0],
+                                  adds ? spare_ : nullptr, op.p[1], bufs_[op.out], t_, n, k, gated, dtype_, compute_units(), stream_));
+      if (adds) std::swap(x_, spare_);
+      pending_ = Pending();
+      release_parts();
+      return;
+    }
     if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts && !weight_bound(t_, rows_of_w, k)) {
       ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
                             bufs_[op.out], t_, n, k, 1, gated, dtype_, 1, stream_));

@@ -51,6 +51,10 @@ int me_gemm_bf16_stream_arrangement(int M, int N, int k_splits, int compute_unit
 int me_gemm_bf16_stream_splits(int N, int K, int compute_units);
 int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype, int k_splits,
                         int compute_units, hipStream_t stream);
+int me_gemm_bf16_stream_norm_fits(int M, int K);
+int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, const float* parts, int num_parts, long long part_stride,
+                             const float* w_norm, float eps, float* x_out, const void* W, void* C, int M, int N, int K,
+                             int swiglu, int out_dtype, int compute_units, hipStream_t stream);
 int me_gemm_bf16_tiled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype, int shape,
                        hipStream_t stream);
 int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype, hipStream_t stream);

@@ -367,6 +367,14 @@ class NormedInput:
                 self.residual = self.x
         return self._tensor
 
+    def streams_normed(self, weight: torch.Tensor) -> bool:
+        """Whether add, norm and the product go into one launch of the weight-streaming kernel: a row or two,
+        whatever the delta is (every block adds and norms the rows itself)."""
+        rows, k = self.x.shape
+        return (self.dtype is torch.bfloat16 and self._tensor is None and self.residual is None
+                and rows <= NORM_STREAM_ROWS and weight.dtype is torch.bfloat16 and (self.delta is None or self.spare is not None)
+                and k % 8 == 0 and weight.numel() * 2 < STREAM_MAX_BYTES and weight.data_ptr() % 16 == 0 and stream_norm_fits(rows, k))
+
     def fusable(self, weight: torch.Tensor) -> bool:
         """Whether add, norm and the product with ``weight`` go into one kernel: decode-sized steps whose
         delta is a tensor (partial sums are read once, by the add-and-norm kernel, not by every block of a
@@ -377,6 +385,7 @@ class NormedInput:
                 and weight.numel() < STREAM_MIN_ELEMENTS)
 
 
+NORM_STREAM_ROWS = 2  # up to here the add-and-norm is the prologue of the weight-streaming kernel
 SMALL_MAX_ROWS = 64  # what the kernel accepts
 SMALL_FAST_ROWS = 16  # up to here it beats the GEMM library on every shape, with the norm as its prologue too
 
@@ -412,6 +421,55 @@ def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
     _want(out, "out", out_dtype, shape)
     check(lib().me_gemm_bf16_stream(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
                                     _i(_code(out_dtype)), _i(k_splits), _i(compute_units(x.device)), _stream()))
+    return out
+
+
+def stream_norm_fits(rows: int, k: int) -> bool:
+    """Whether :func:`gemm_bf16_stream_norm` takes this many rows of this length."""
+    return bool(lib().me_gemm_bf16_stream_norm_fits(_i(rows), _i(k)))
+
+
+def gemm_bf16_stream_norm(x: "NormedInput", weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                          swiglu: "bool | str" = False, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``rmsnorm(x.x + x.delta) * x.weight @ weight.T`` for a row or a few in one launch of the weight-streaming
+    kernel: every block adds and norms the rows itself while its first weights are on their way. ``x.delta`` is a
+    bfloat16 tensor, :class:`PartialSums` or None; with a delta the sum goes to ``x.spare``, which becomes
+    ``x.residual``."""
+    m, k = x.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0]
+    if swiglu:
+        if n % 2:
+            raise ValueError(f"a gate/up weight needs an even number of rows, got {n}")
+        n //= 2
+    if not stream_norm_fits(m, k):
+        raise ValueError(f"gemm_bf16_stream_norm does not take {m} rows of {k}")
+    _want(x.x, "x", torch.float32, (m, k))
+    _want(x.weight, "norm weight", torch.float32, (k,))
+    delta = parts = None
+    num_parts = stride = 0
+    if isinstance(x.delta, PartialSums):
+        parts = x.delta.parts
+        _want(parts, "partial sums", torch.float32, (None, m, k))
+        num_parts, stride = parts.shape[0], m * k
+    elif x.delta is not None:
+        delta = x.delta
+        _want(delta, "delta", torch.bfloat16, (m, k))
+    x_out = None
+    if x.delta is not None:
+        if x.spare is None:
+            raise ValueError("the sum of the residual stream and its delta needs a second buffer")
+        x_out = x.spare
+        _want(x_out, "spare", torch.float32, (m, k))
+        if x_out.data_ptr() == x.x.data_ptr():
+            raise ValueError("the second buffer must not be the residual stream itself")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=weight.device)
+    _want(out, "out", out_dtype, (m, n))
+    check(lib().me_gemm_bf16_stream_norm(_p(x.x), _p(delta), _p(parts), _i(num_parts), ctypes.c_longlong(stride), _p(x.weight),
+                                         _f(x.eps), _p(x_out), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
+                                         _i(_code(out_dtype)), _i(compute_units(weight.device)), _stream()))
+    x.residual = x_out if x_out is not None else x.x
     return out
 
 
@@ -542,6 +600,8 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     of up to 64 rows as partial sums over runs of k; the tiled matrix-core kernel with
     the SwiGLU as its epilogue for gated products of 256 rows or more; else the GEMM library."""
     if isinstance(x, NormedInput):
+        if x.streams_normed(weight):
+            return gemm_bf16_stream_norm(x, weight, out_dtype or x.dtype, gated)
         if x.fusable(weight):
             return gemm_bf16_small(x, weight, out_dtype or x.dtype, gated)
         x = x.materialize()

@@ -310,6 +310,58 @@ def test_gemm_bf16_stream(m, n, k, gated):
         assert parts[-1].abs().max() > 0
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 1024), (2, 100, 1000), (3, 1040, 72), (4, 68, 2056), (1, 16, 128), (2, 9000, 648)])
+@pytest.mark.parametrize("delta", ["none", "tensor", "parts3", "parts6"])
+@pytest.mark.parametrize("gated", [False, "silu", "gelu_tanh"])
+def test_gemm_bf16_stream_norm(m, n, k, delta, gated):
+    """Residual add, RMSNorm and product in one launch of the weight-streaming kernel, for a row or a few: every
+    arrangement of a block's waves, k that is no multiple of a step, each kind of delta (none, a tensor, partial sums
+    in odd and even numbers), both output types and both gates; the sum goes to the second buffer and only there."""
+    g = torch.Generator().manual_seed(m * 31 + n + k)
+    x, wn = torch.randn(m, k, generator=g) * 2, 1 + 0.2 * torch.randn(k, generator=g)
+    w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
+    w[n - 1] *= 4
+    s, d = x.clone(), None
+    if delta == "tensor":
+        d = torch.randn(m, k, generator=g).bfloat16()
+        s = x + d.float()
+        d = dev(d)
+    elif delta.startswith("parts"):
+        parts = torch.randn(int(delta[5:]), m, k, generator=g)
+        s = x + parts.sum(0)
+        d = K().PartialSums(dev(parts))
+    normed = plain.rms_norm(s, wn, 1e-5)
+    y = normed @ w.float().T
+    act = {"silu": plain.silu, "gelu_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh")}.get(gated)
+    want = act(y[:, :n]) * y[:, n:] if gated else y
+    scale = max(1.0, want.abs().max().item())
+    for out_dtype in ((torch.bfloat16,) if gated else (torch.bfloat16, torch.float32)):
+        xd, spare = dev(x.clone()), dev(torch.full((m, k), 7.0))
+        h = K().NormedInput(xd, d, dev(wn), 1e-5, torch.bfloat16, spare)
+        got = K().gemm_bf16_stream_norm(h, dev(w), out_dtype, gated).float().cpu()
+        # the operand is rounded to bfloat16 once, as the add-and-norm kernel rounds it: 2^-8 of the largest product
+        assert (got - want).abs().max().item() <= 2**-6 * scale
+        assert torch.equal(xd.cpu(), x)  # other blocks still read it
+        if delta == "none":
+            assert h.residual is xd and torch.equal(spare.cpu(), torch.full((m, k), 7.0))
+        else:
+            assert h.residual is spare
+            torch.testing.assert_close(spare.cpu(), s, rtol=1e-6, atol=1e-6)
+
+
+def test_gemm_bf16_stream_norm_refuses_what_it_cannot_do():
+    wn, w = dev(torch.ones(64)), dev(torch.zeros(32, 64).bfloat16())
+    x = dev(torch.zeros(17, 64))
+    with pytest.raises(ValueError, match="17 rows"):
+        K().gemm_bf16_stream_norm(K().NormedInput(x, None, wn, 1e-6, torch.bfloat16, None), w)
+    assert not K().stream_norm_fits(4, 8192) and K().stream_norm_fits(2, 8192)  # the rows stay in the block's memory
+    x = dev(torch.zeros(2, 64))
+    with pytest.raises(ValueError, match="second buffer"):
+        K().gemm_bf16_stream_norm(K().NormedInput(x, dev(torch.zeros(2, 64).bfloat16()), wn, 1e-6, torch.bfloat16, None), w)
+    with pytest.raises(ValueError, match="residual stream itself"):
+        K().gemm_bf16_stream_norm(K().NormedInput(x, dev(torch.zeros(2, 64).bfloat16()), wn, 1e-6, torch.bfloat16, x), w)
+
+
 def test_gemm_bf16_stream_refuses_what_it_cannot_do():
     x, w = dev(torch.zeros(65, 64).bfloat16()), dev(torch.zeros(32, 64).bfloat16())
     with pytest.raises(ValueError):
