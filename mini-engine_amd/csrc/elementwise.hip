@@ -180,9 +180,10 @@ static bool launch_add_rmsnorm_vec(float* x, const T* delta, const float* parts,
   if (((uintptr_t)x | (uintptr_t)parts | (uintptr_t)w) & 15 || ((uintptr_t)delta | (uintptr_t)h) & (sizeof(T) * 4 - 1) || part_stride % 4)
     return false;
   const int nvec = dim / 4;
-  // a vector per thread where a block can have that many threads: all loads of a row are in flight at once (64 rows of
-  // 1,024 with 6 partial sums: 3.1 us against 3.9 with a wave per row; of 4,096 with 8: 4.1 against 9.8). A function of
-  // the row's length alone.
+  // a vector per thread where a block can have that many threads: all loads of a row are in flight at once (against a
+  // wave per row with the row in its registers: 64 rows of 1,024 with 6 partial sums 3.1 us against 3.9, of 4,096 with 8
+  // 4.1 against 9.8; 512 rows of 4,096 5.9 against 10.0; 2,048 rows of 1,024 5.5 against 6.2). A function of the row's
+  // length alone: a row's sum of squares is added up in the same order whatever the number of rows.
   const int threads = nvec <= 64 ? 64 : (nvec <= 128 ? 128 : (nvec <= 256 ? 256 : (nvec <= 512 ? 512 : 1024)));
   add_rmsnorm_vec_kernel<T><<<num_rows, threads, 0, stream>>>(x, delta, parts, num_parts, part_stride, w, h, rows, dim, eps,
                                                               write_x);
@@ -235,122 +236,12 @@ extern "C" int me_residual_add(void* x, const void* delta, const float* parts, i
   return me_check_launch("me_residual_add");
 }
 
-// The same for more than 16 bfloat16 rows: a wave per row, the row in registers (CHUNKS x 8 elements per lane), 16-byte
-// loads and stores, no LDS and no barrier. dim is a multiple of 8 and at most 512 * CHUNKS.
-template <typename T, int CHUNKS>
-__global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float* __restrict__ x, const T* __restrict__ delta,
-                                                                const float* __restrict__ parts, int num_parts,
-                                                                size_t part_stride, const float* __restrict__ w,
-                                                                T* __restrict__ h, const int* __restrict__ rows,
-                                                                int num_rows, int dim, float eps, int write_x) {
-  const int lane = threadIdx.x & (ME_WAVE - 1);
-  const int r = blockIdx.x * (blockDim.x / ME_WAVE) + threadIdx.x / ME_WAVE;
-  if (r >= num_rows) return;
-  const int src = rows ? rows[r] : r;
-  float* xr = x + (size_t)src * dim;
-  const T* dr = delta ? delta + (size_t)src * dim : nullptr;
-  const float* pr = parts ? parts + (size_t)src * dim : nullptr;
-  float s[CHUNKS][8];
-  float ss = 0.f;
-#pragma unroll
-  for (int c = 0; c < CHUNKS; ++c) {
-    const int e = (c * ME_WAVE + lane) * 8;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) s[c][j] = 0.f;
-    if (e < dim) {
-      const float4 a = *reinterpret_cast<const float4*>(xr + e), b = *reinterpret_cast<const float4*>(xr + e + 4);
-      s[c][0] = a.x, s[c][1] = a.y, s[c][2] = a.z, s[c][3] = a.w, s[c][4] = b.x, s[c][5] = b.y, s[c][6] = b.z, s[c][7] = b.w;
-      if (dr) {
-        struct alignas(sizeof(T) * 8) Pack {
-          T v[8];
-        };
-        const Pack d = *reinterpret_cast<const Pack*>(dr + e);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s[c][j] += to_float(d.v[j]);
-      }
-      if (pr) {  // a delta that still is a sum of partial products: added in the order of the runs
-        float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        auto add = [&](const float4& pa, const float4& pb) {
-          d[0] += pa.x, d[1] += pa.y, d[2] += pa.z, d[3] += pa.w, d[4] += pb.x, d[5] += pb.y, d[6] += pb.z, d[7] += pb.w;
-        };
-        const float* at = pr + e;
-        int p = 0;
-        for (; p + 4 <= num_parts; p += 4) {  // the loads of four runs in flight at once, their sums in the runs' order
-          float4 pa[4], pb[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            pa[q] = *reinterpret_cast<const float4*>(at + (size_t)(p + q) * part_stride);
-            pb[q] = *reinterpret_cast<const float4*>(at + (size_t)(p + q) * part_stride + 4);
-          }
-#pragma unroll
-          for (int q = 0; q < 4; ++q) add(pa[q], pb[q]);
-        }
-        for (; p < num_parts; ++p)
-          add(*reinterpret_cast<const float4*>(at + (size_t)p * part_stride),
-              *reinterpret_cast<const float4*>(at + (size_t)p * part_stride + 4));
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s[c][j] += d[j];
-      }
-      if ((dr || pr) && write_x) {
-        *reinterpret_cast<float4*>(xr + e) = make_float4(s[c][0], s[c][1], s[c][2], s[c][3]);
-        *reinterpret_cast<float4*>(xr + e + 4) = make_float4(s[c][4], s[c][5], s[c][6], s[c][7]);
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ss = fmaf(s[c][j], s[c][j], ss);
-    }
-  }
-  const float inv = rsqrtf(wave_sum(ss) / (float)dim + eps);
-  T* hr = h + (size_t)r * dim;
-#pragma unroll
-  for (int c = 0; c < CHUNKS; ++c) {
-    const int e = (c * ME_WAVE + lane) * 8;
-    if (e < dim) {
-      const float4 a = *reinterpret_cast<const float4*>(w + e), b = *reinterpret_cast<const float4*>(w + e + 4);
-      const float wv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-      struct alignas(sizeof(T) * 8) Pack {
-        T v[8];
-      } o;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) o.v[j] = from_float<T>(s[c][j] * inv * wv[j]);
-      *reinterpret_cast<Pack*>(hr + e) = o;
-    }
-  }
-}
-
-template <typename T>
-static bool launch_add_rmsnorm_rows(float* x, const T* delta, const float* parts, int num_parts, size_t part_stride,
-                                    const float* w, T* h, const int* rows, int num_rows, int dim, float eps, int write_x,
-                                    hipStream_t stream) {
-  if (num_rows <= 64 || dim % 8 || dim > 4096) return false;  // few rows: a block a row has more loads in flight
-  if (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)parts | (uintptr_t)w | (uintptr_t)h) & 15 || part_stride % 4) return false;
-  const int waves = num_rows >= 256 ? 4 : 1;  // few rows: a block each, on compute units of their own
-  const unsigned blocks = (num_rows + waves - 1) / waves;
-#define ME_ROWS_CASE(C)                                                                                             \
-  add_rmsnorm_rows_kernel<T, C><<<blocks, waves * 64, 0, stream>>>(x, delta, parts, num_parts, part_stride, w, h, rows, \
-                                                                   num_rows, dim, eps, write_x)
-  if (dim <= 512)
-    ME_ROWS_CASE(1);
-  else if (dim <= 1024)
-    ME_ROWS_CASE(2);
-  else if (dim <= 2048)
-    ME_ROWS_CASE(4);
-  else
-    ME_ROWS_CASE(8);
-#undef ME_ROWS_CASE
-  return true;
-}
-
 extern "C" int me_add_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
                               const float* w, void* h, const int* rows, int num_rows, int dim, float eps, int write_x,
                               int dtype, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   if (dim <= 0) return me_fail("me_add_rmsnorm: dim=%d", dim);
   if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_add_rmsnorm: %d partial sums", num_parts);
-  // bfloat16 only: in float32 the order of a row's sum stays the same for every number of rows
-  if (dtype == ME_BF16 && launch_add_rmsnorm_rows<bf16_t>((float*)x, (const bf16_t*)delta, parts, num_parts,
-                                                          (size_t)part_stride, w, (bf16_t*)h, rows, num_rows, dim, eps,
-                                                          write_x, stream))
-    return me_check_launch("me_add_rmsnorm");
   if (dtype == ME_F32 ? launch_add_rmsnorm_vec<float>((float*)x, (const float*)delta, parts, num_parts, (size_t)part_stride, w,
                                                       (float*)h, rows, num_rows, dim, eps, write_x, stream)
                       : launch_add_rmsnorm_vec<bf16_t>((float*)x, (const bf16_t*)delta, parts, num_parts, (size_t)part_stride,

@@ -187,8 +187,8 @@ def test_small_gemm_partial_sums_and_their_add_rmsnorm(m, n, k, splits):
 @pytest.mark.parametrize("rows,dim,num_parts", [(3, 5120, 7), (40, 5120, 7), (64, 8192, 16), (8, 1000, 5), (20, 16384, 2), (2, 20000, 3),
                                                 (5, 1002, 4), (1, 16, 9)])
 def test_add_rmsnorm_with_partial_sums_at_every_row_length(dtype, rows, dim, num_parts):
-    """Partial sums stand where a delta stands, for few rows and many, rows longer than the wave-per-row
-    kernel takes, lengths that are no multiple of 4 and lengths beyond the vectorised kernel's."""
+    """Partial sums stand where a delta stands, for few rows and many, rows of one vector and of several vectors per
+    thread, lengths that are no multiple of 4 and lengths beyond the vectorised kernel's."""
     g = torch.Generator().manual_seed(rows * dim + num_parts)
     x, w = torch.randn(rows, dim, generator=g) * 3, 1 + 0.1 * torch.randn(dim, generator=g)
     parts = torch.randn(num_parts, rows, dim, generator=g)
