@@ -319,7 +319,7 @@ class Run {
     const void* x = bufs_[op.in];
     pending_ = Pending();
     if (dtype_ == kBF16 && streams(t_, n, k)) {
-      const int splits = me_gemm_bf16_stream_splits(n, k, compute_units());
+      const int splits = me_gemm_bf16_stream_splits(t_, n, k, compute_units());
       if (splits > 1) {
         parts_mark_ = arena_.used;
         float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);

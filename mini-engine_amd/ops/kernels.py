@@ -394,9 +394,10 @@ def compute_units(device=None) -> int:
     return torch.cuda.get_device_properties(device or torch.cuda.current_device()).multi_processor_count
 
 
-def stream_splits(n: int, k: int, device=None) -> int:
-    """Into how many runs of k :func:`gemm_bf16_stream` cuts a product whose result may stay partial sums."""
-    return int(lib().me_gemm_bf16_stream_splits(_i(n), _i(k), _i(compute_units(device))))
+def stream_splits(n: int, k: int, device=None, rows: int = 1) -> int:
+    """Into how many runs of k :func:`gemm_bf16_stream` cuts a product of ``rows`` rows whose result may stay
+    partial sums."""
+    return int(lib().me_gemm_bf16_stream_splits(_i(rows), _i(n), _i(k), _i(compute_units(device))))
 
 
 def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
@@ -613,7 +614,7 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return swiglu(y, activation="silu" if gated is True else gated) if gated else y
     heavy, few = weight_bound(x, weight), x.shape[0] <= SMALL_FAST_ROWS
     if as_delta and not gated and streams(x, weight):
-        splits = stream_splits(weight.shape[0], x.shape[1], x.device)
+        splits = stream_splits(weight.shape[0], x.shape[1], x.device, x.shape[0])
         if splits > 1:
             return PartialSums(gemm_bf16_stream(x, weight, torch.float32, k_splits=splits))
         return gemm_bf16_stream(x, weight, out_dtype)

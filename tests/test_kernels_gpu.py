@@ -301,7 +301,7 @@ def test_gemm_bf16_stream(m, n, k, gated):
     got = K().gemm_bf16_stream(dev(x), dev(w), torch.float32).cpu()
     assert (got - want).abs().max().item() <= 1e-4 * scale
     steps = -(-k // 128)
-    for splits in sorted({K().stream_splits(n, k), 2, 3, min(steps, 64)} - {1}):
+    for splits in sorted({K().stream_splits(n, k, rows=m), K().stream_splits(n, k), 2, 3, min(steps, 64)} - {1}):
         if steps < splits or -(-steps // -(-steps // splits)) != splits:
             continue  # runs are whole steps, none of them empty
         parts = K().gemm_bf16_stream(dev(x), dev(w), torch.float32, k_splits=splits).cpu()
