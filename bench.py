@@ -298,6 +298,10 @@ def shape_line(shape: str, args) -> dict:
     bench = DecodeBench(cfg, args.dtype, ctx, 64)
     prefill = bench.prefill(min(args.prefill_tokens, ctx - 16))
     tok_s, ms, gbs, _ = bench.decode(64, args.steps, args.warmup)
+    points, fracs = {"decode_b64": round(tok_s, 1)}, {"decode_b64": round(gbs / HBM_PEAK_GBS, 4)}
+    for b in (1, 8):
+        m = bench.decode(b, args.steps, args.warmup)
+        points[f"decode_b{b}"], fracs[f"decode_b{b}"] = round(m[0], 1), round(m[2] / HBM_PEAK_GBS, 4)
     name = {"8b": "Qwen3-8B shape", "32b": "Qwen3-32B shape"}[shape]
     what = {"8b": "64 requests, prompts uniform in [128, 2048], 128 output tokens, 8,192-token step budget",
             "32b": "64 requests of a shared 512-token prefix + 32 tokens, 64 output tokens, prefix cache warm"}[shape]
@@ -310,7 +314,7 @@ def shape_line(shape: str, args) -> dict:
         "workload": work, "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4)},
-        "points": {"decode_b64": round(tok_s, 1)},
+        "points": points, "points_roofline_frac": fracs,
     }
 
 
