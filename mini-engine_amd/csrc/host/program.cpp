@@ -276,7 +276,7 @@ class Run {
   void product(const void* x, const void* w, int rows_of_w, int k, int gated, int out_dtype, void* out) {
     const int m = t_rows_;
     const int n = gated ? rows_of_w / 2 : rows_of_w;
-    if (dtype_ == kF32) {  // a true 32-bit product on the vector units, additions in ascending k
+    if (dtype_ == kF32) {  // a true 32-bit product, additions in ascending k whatever the rows
       if (!gated) {
         ok(me_gemm_f32((const float*)x, (const float*)w, (float*)out, m, n, k, stream_));
         return;

@@ -327,7 +327,8 @@ def attention_general(
 # ------------------------------------------------------------------------------ matrix products
 
 def gemm_f32(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """float32 ``x @ weight.T`` on the vector units, additions in ascending k for every element."""
+    """float32 ``x @ weight.T`` on the matrix cores' float32 instruction (float32 operands, products and sums): an
+    element's products are added two k at a time in ascending k, whatever the number of rows."""
     _want(x, "x", torch.float32, (None, None))
     m, k = x.shape
     _want(weight, "weight", torch.float32, (None, k))
@@ -594,7 +595,7 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     (what a mixer or a feed-forward returns): it may then come back as :class:`PartialSums`, which
     :func:`add_rmsnorm` adds up on the way.
 
-    float32: always the deterministic vector-unit kernel (a true 32-bit product). bfloat16, by rows and
+    float32: always the deterministic float32 kernel (a true 32-bit product). bfloat16, by rows and
     weight size as ``csrc/host/program.cpp`` chooses (where the measurements are): up to 16 rows the small
     matrix-core kernel, or the weight-streaming one for weights of 16 MiB and more; 17 to 64 rows the
     weight-streaming kernel (the library for weights of 16 MiB and more); a delta of the residual stream
