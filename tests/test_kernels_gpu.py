@@ -97,11 +97,21 @@ def test_gated_products_with_either_activation(dtype, rows):
     assert (act(y[:, :200]) - plain.silu(y[:, :200])).abs().max() > 0.05  # the two activations differ at these values
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 50, 33), (5, 130, 72), (70, 64, 100), (129, 257, 48)])
+@pytest.mark.parametrize("m,n,k", [(1, 50, 33), (5, 130, 72), (70, 64, 100), (129, 257, 48), (64, 33, 1028), (65, 300, 1024),
+                                   (200, 96, 2050), (32, 31, 16), (33, 160, 2)])
 def test_gemm_f32(m, n, k):
-    x, w = torch.randn(m, k), torch.randn(n, k)
+    """The float32 product at row counts on both sides of its tile shapes' limits (32, 64), columns that are no
+    multiple of a tile, k that is no multiple of the tile's 16, of 4 (no 16-byte loads) or of the instruction's 2;
+    one column and one row stand out, so that a tile that stops short of them or runs past them shows."""
+    g = torch.Generator().manual_seed(m * 7 + n + k)
+    x, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
+    w[n - 1] *= 8
+    x[m - 1] *= 8
     out = K().gemm_f32(dev(x), dev(w))
-    torch.testing.assert_close(out.cpu(), (x.double() @ w.double().T).float(), rtol=1e-5, atol=1e-5)
+    want = (x.double() @ w.double().T).float()
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-5, atol=1e-5 * max(1.0, want.abs().max().item()))
+    shifted = dev(torch.cat([torch.zeros(1, k), x]))[1:]  # rows that start 4 k bytes into an allocation: not always 16-byte aligned
+    assert torch.equal(K().gemm_f32(shifted, dev(w)).cpu(), out.cpu())  # scalar and 16-byte loads give the same sums
 
 
 @pytest.mark.parametrize("m,n,k,gated", [(130, 200, 128, False), (257, 96, 192, True), (2048, 1024, 1024, False),
@@ -221,9 +231,9 @@ def test_linear_hands_back_partial_sums_only_when_asked():
 
 def test_gemm_f32_rows_do_not_depend_on_the_batch():
     """The value of a row is bit-identical whatever other rows are in the product."""
-    x, w = torch.randn(90, 200), torch.randn(77, 200)
-    whole = K().gemm_f32(dev(x), dev(w)).cpu()
-    for lo, hi in [(0, 1), (63, 65), (89, 90), (10, 80)]:
+    x, w = torch.randn(200, 200), torch.randn(77, 200)
+    whole = K().gemm_f32(dev(x), dev(w)).cpu()  # tiles of 128 rows
+    for lo, hi in [(0, 1), (63, 65), (89, 90), (10, 80), (100, 132), (136, 200), (0, 65)]:  # one-wave tiles, and large ones
         assert torch.equal(K().gemm_f32(dev(x[lo:hi]), dev(w)).cpu(), whole[lo:hi])
 
 
