@@ -39,6 +39,8 @@ def main() -> None:
     parser.add_argument("--temperature", type=float, default=0.0)
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--num-blocks", type=int, default=128)
+    parser.add_argument("--kv-memory-fraction", type=float, default=None,
+                        help="size the KV pool by memory instead: the engine stays within this share of the GPU's memory")
     parser.add_argument("--block-size", type=int, default=16)
     parser.add_argument("--max-num-seqs", type=int, default=16)
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
@@ -64,8 +66,9 @@ def main() -> None:
 
     engine = LLMEngine.from_pretrained(
         args.model,
-        EngineConfig(dtype=args.dtype, num_blocks=args.num_blocks, block_size=args.block_size, seed=args.seed,
-                     max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens),
+        EngineConfig(dtype=args.dtype, num_blocks=args.num_blocks, kv_memory_fraction=args.kv_memory_fraction,
+                     block_size=args.block_size, seed=args.seed, max_num_seqs=args.max_num_seqs,
+                     max_num_batched_tokens=args.max_num_batched_tokens),
     )
     vocab = engine.model.plan.vocab_size
     if args.prompt:

@@ -49,10 +49,35 @@ def kv_cache_bytes_per_token(plan: ModelPlan, dtype: str) -> int:
     return elem * sum(int(getattr(plan.layers[i].mixer, "kv_elements_per_token", 0)) for i in plan.order)
 
 
+def blocks_that_fit(free_bytes: int, total_bytes: int, fraction: float, plan: ModelPlan, dtype: str, block_size: int,
+                    max_num_batched_tokens: int = 0) -> int:
+    """How many pages a pool may have when the engine is to stay within ``fraction`` of the GPU's ``total_bytes``, of
+    which ``free_bytes`` are free now (the weights are loaded): what is left after the other users of memory, and
+    after the workspaces of a step of ``max_num_batched_tokens`` tokens (its float32 logits aside, a few rows of the
+    hidden size per token: counted as 64 bytes per token and hidden element over the widest layer, generously),
+    divided by a page's bytes over all layers. Every cache group has a pool of that many pages."""
+    per_page = kv_cache_bytes_per_token(plan, dtype) * block_size
+    if per_page <= 0:
+        raise ValueError("this model keeps no keys or values: its pool cannot be sized by memory")
+    widest = max([plan.hidden_size] + [int(getattr(layer.ffn, "intermediate_size", 0)) * 2 for layer in plan.layers])
+    workspaces = 64 * max_num_batched_tokens * widest
+    budget = free_bytes - int((1.0 - fraction) * total_bytes) - workspaces
+    if budget < per_page:
+        raise ValueError(f"{fraction:.2f} of the GPU's memory leaves no room for a page of {per_page} bytes "
+                         f"({free_bytes} of {total_bytes} bytes are free)")
+    return int(budget // per_page)
+
+
 class LLMEngine:
     def __init__(self, model: Decoder, config: EngineConfig, eos_token_ids: Iterable[int] = ()):
         if TORCH_DTYPES[config.dtype] is not model.dtype:
             raise ValueError(f"the model was built for {model.dtype}, the engine config says {config.dtype}")
+        if config.kv_memory_fraction is not None:  # the pool takes what the model left of its share of the memory
+            import dataclasses
+            free, total = torch.cuda.mem_get_info()
+            fit = blocks_that_fit(free, total, config.kv_memory_fraction, model.plan, config.dtype, config.block_size,
+                                  config.max_num_batched_tokens)
+            config = dataclasses.replace(config, num_blocks=fit)
         self.config = config
         self.model = model
         eos = set(eos_token_ids)

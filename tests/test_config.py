@@ -99,3 +99,28 @@ def test_engine_config_defaults_and_checks():
         EngineConfig(dtype="float16")
     with pytest.raises(ValueError):
         EngineConfig(block_size=0)
+
+
+def test_pool_sized_by_memory():
+    """A share of the GPU's memory instead of a number of pages: what is left of the share after everything already
+    on the GPU and after a step's workspaces, in pages of all layers (SURVEY: sizing helper
+    ``engine.py:54-56``: 2 x layers x kv heads x head size x element size per token)."""
+    from mini_engine_amd.engine.llm_engine import blocks_that_fit, kv_cache_bytes_per_token
+
+    a = tiny_configs()["A"]
+    plan = plan_from_config(a)
+    per_token = 2 * a.num_hidden_layers * a.num_key_value_heads * a.head_dim
+    assert kv_cache_bytes_per_token(plan, "float32") == 4 * per_token and kv_cache_bytes_per_token(plan, "bfloat16") == 2 * per_token
+    page = 2 * per_token * 16
+    total = 1 << 30
+    assert blocks_that_fit(total, total, 1.0, plan, "bfloat16", 16) == total // page
+    assert blocks_that_fit(total // 2, total, 0.75, plan, "bfloat16", 16) == (total // 4) // page  # half is taken, a quarter stays free
+    with_steps = blocks_that_fit(total, total, 1.0, plan, "bfloat16", 16, max_num_batched_tokens=2048)
+    assert 0 < with_steps < total // page  # a step's workspaces come off first
+    with pytest.raises(ValueError, match="no room"):
+        blocks_that_fit(total // 4, total, 0.5, plan, "bfloat16", 16)  # the others already use more than is left of the share
+    with pytest.raises(ValueError, match="kv_memory_fraction"):
+        EngineConfig(kv_memory_fraction=0.0)
+    with pytest.raises(ValueError, match="kv_memory_fraction"):
+        EngineConfig(kv_memory_fraction=1.5)
+    assert EngineConfig(kv_memory_fraction=0.9).kv_memory_fraction == 0.9

@@ -244,6 +244,23 @@ def test_tiny_a_workload(peaked):
         assert eng.generate(prompts, SamplingParams(max_tokens=8)) == want, over
 
 
+def test_pool_sized_by_a_share_of_the_memory(peaked):
+    """``kv_memory_fraction`` instead of ``num_blocks``: the pool has the pages that fit into that share of the GPU's
+    memory beside what is already on it, and generation is what it is with a pool of a given size."""
+    from mini_engine_amd import SamplingParams
+    from mini_engine_amd.engine.llm_engine import kv_cache_bytes_per_token
+
+    free, total = torch.cuda.mem_get_info()
+    share = (total - free + (64 << 20) + (1 << 30)) / total  # what is in use now, a step's workspaces and a gigabyte of pages
+    eng = engine(peaked["A"][0], "A", kv_memory_fraction=share, num_blocks=1)
+    page = kv_cache_bytes_per_token(eng.model.plan, "float32") * 4
+    assert (1 << 29) // page <= eng.config.num_blocks <= (3 << 29) // page  # about a gigabyte of pages, whatever num_blocks said
+    assert eng.block_manager.num_free_blocks == eng.config.num_blocks
+    assert eng.generate(prompts_for("A"), SamplingParams(max_tokens=MAX_NEW)) == reference(peaked, "A")
+    with pytest.raises(ValueError, match="no room"):
+        engine(peaked["A"][0], "A", kv_memory_fraction=1e-6)
+
+
 def test_requests_that_cannot_fit_are_refused(peaked):
     from mini_engine_amd import SamplingParams
 
