@@ -319,18 +319,26 @@ class Run {
     const void* x = bufs_[op.in];
     pending_ = Pending();
     if (dtype_ == kBF16 && streams(t_, n, k)) {
+      // float32 partial sums over runs of k (one run for short k): the next add-and-norm adds them up, and the delta is
+      // never rounded to bfloat16 on its way into the float32 residual stream
       const int splits = me_gemm_bf16_stream_splits(t_, n, k, compute_units());
-      if (splits > 1) {
-        parts_mark_ = arena_.used;
-        float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);
-        ok(me_gemm_bf16_stream(x, op.p[1], parts, t_, n, k, 0, kF32, splits, compute_units(), stream_));
-        pending_.parts = parts;
-        pending_.num_parts = splits;
-        pending_.stride = (long long)t_ * n;
-        return;
-      }
-      ok(me_gemm_bf16_stream(x, op.p[1], bufs_[op.out], t_, n, k, 0, kBF16, 1, compute_units(), stream_));
-      pending_.delta = bufs_[op.out];
+      parts_mark_ = arena_.used;
+      float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);
+      ok(me_gemm_bf16_stream(x, op.p[1], parts, t_, n, k, 0, kF32, splits, compute_units(), stream_));
+      pending_.parts = parts;
+      pending_.num_parts = splits;
+      pending_.stride = (long long)t_ * n;
+      return;
+    }
+    if (dtype_ == kBF16) {
+      // more rows: the library's product with a float32 result, which stands as one partial sum: the delta is never
+      // rounded to bfloat16 on its way into the float32 residual stream
+      parts_mark_ = arena_.used;
+      float* sum = (float*)arena_.take((size_t)t_ * n * 4);
+      library_product(x, op.p[1], sum, t_, n, k, kF32, stream_);
+      pending_.parts = sum;
+      pending_.num_parts = 1;
+      pending_.stride = (long long)t_ * n;
       return;
     }
     const size_t mark = arena_.used;
@@ -490,7 +498,8 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
   for (const Op& op : ops_) {
     size_t need = 0;
     if (op.kind == kOpNormLinear || op.kind == kOpLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
-    if (op.kind == kOpLinearDelta) need = (size_t)16 * std::min<int64_t>(tokens, kSmallMaxRows) * op.i[0] * 4 + pad;
+    if (op.kind == kOpLinearDelta)  // up to 16 partial sums of up to 64 rows, or one float32 result of all rows
+      need = std::max<size_t>((size_t)16 * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
     if (op.kind == kOpAttention) {
       const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
       const int chunks = (nh / nkv + 15) / 16;
@@ -509,7 +518,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
   const size_t tail = (size_t)rows * hidden_ * elem + (size_t)rows * vocab_ * 4 + (size_t)rows * 4 +
                       (size_t)rows * me_sample_chunks(vocab_) * 8 + 4 * pad;
   // partial sums of the last delta wait beside the head's buffers
-  return fixed + 2 * scratch + tail + (size_t)16 * kSmallMaxRows * hidden_ * 4 + (1 << 16);
+  return fixed + 2 * scratch + tail + std::max<size_t>((size_t)16 * kSmallMaxRows, (size_t)tokens) * hidden_ * 4 + (1 << 16);
 }
 
 }  // namespace me

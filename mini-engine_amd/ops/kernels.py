@@ -616,9 +616,12 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     heavy, few = weight_bound(x, weight), x.shape[0] <= SMALL_FAST_ROWS
     if as_delta and not gated and streams(x, weight):
         splits = stream_splits(weight.shape[0], x.shape[1], x.device, x.shape[0])
-        if splits > 1:
-            return PartialSums(gemm_bf16_stream(x, weight, torch.float32, k_splits=splits))
-        return gemm_bf16_stream(x, weight, out_dtype)
+        parts = gemm_bf16_stream(x, weight, torch.float32, k_splits=splits)
+        return PartialSums(parts if splits > 1 else parts.unsqueeze(0))
+    if as_delta and not gated and out_dtype is torch.bfloat16:
+        # more rows: the library's product with a float32 result, which stands as one partial sum (the delta is never
+        # rounded to bfloat16 on its way into the float32 residual stream)
+        return PartialSums(gemm_bf16_library(x, weight, torch.float32).unsqueeze(0))
     if (heavy if few else streams(x, weight) and not heavy) and (out_dtype is torch.bfloat16 or not gated):
         return gemm_bf16_stream(x, weight, out_dtype, gated)
     if heavy and x.shape[0] <= HEAD_STREAM_ROWS and out_dtype is torch.float32 and not gated:  # a head's logits

@@ -215,18 +215,27 @@ def test_add_rmsnorm_with_partial_sums_at_every_row_length(dtype, rows, dim, num
 
 
 def test_linear_hands_back_partial_sums_only_when_asked():
+    """A bfloat16 product that is only ever a delta of the residual stream comes back as float32 partial sums, never
+    rounded to bfloat16: several runs of k from the streaming kernel up to 64 rows, one sum from the library beyond,
+    and for sizes the streaming kernel does not take."""
     x = dev(torch.randn(40, 2048).bfloat16())
     w = dev((torch.randn(1024, 2048) * 0.02).bfloat16())
     plain_out = K().linear(x, w)
     assert isinstance(plain_out, torch.Tensor)
+    exact = x.float() @ w.float().T
     delta = K().linear(x, w, as_delta=True)
-    assert isinstance(delta, K().PartialSums) and delta.shape == (40, 1024)
-    torch.testing.assert_close(delta.to_tensor(torch.bfloat16).float(), plain_out.float(), rtol=2e-2, atol=2e-2)
+    assert isinstance(delta, K().PartialSums) and delta.shape == (40, 1024) and delta.parts.shape[0] > 1
+    torch.testing.assert_close(delta.parts.sum(0), exact, rtol=1e-4, atol=1e-4)  # float32 all the way
     few = K().linear(x[:8].contiguous(), w, as_delta=True)  # few rows too: k is cut so that every compute unit streams
-    assert isinstance(few, K().PartialSums) and few.shape == (8, 1024)
-    torch.testing.assert_close(few.to_tensor(torch.bfloat16).float(), plain_out[:8].float(), rtol=2e-2, atol=2e-2)
+    assert isinstance(few, K().PartialSums) and few.shape == (8, 1024) and few.parts.shape[0] > 1
+    torch.testing.assert_close(few.parts.sum(0), exact[:8], rtol=1e-4, atol=1e-4)
     narrow = dev((torch.randn(1024, 2048 - 4) * 0.02).bfloat16())  # k no multiple of 8: not the streaming kernel's
-    assert isinstance(K().linear(x[:, :2044].contiguous(), narrow, as_delta=True), torch.Tensor)
+    odd = K().linear(x[:, :2044].contiguous(), narrow, as_delta=True)
+    assert isinstance(odd, K().PartialSums) and odd.parts.shape == (1, 40, 1024) and odd.parts.dtype is torch.float32
+    many = K().linear(dev(torch.randn(300, 2048).bfloat16()), w, as_delta=True)  # beyond 64 rows: one sum from the library
+    assert isinstance(many, K().PartialSums) and many.parts.shape == (1, 300, 1024) and many.parts.dtype is torch.float32
+    short = K().linear(x[:, :256].contiguous(), dev((torch.randn(1024, 256) * 0.02).bfloat16()), as_delta=True)  # one run of k
+    assert isinstance(short, K().PartialSums) and short.parts.shape == (1, 40, 1024)
 
 
 def test_gemm_f32_rows_do_not_depend_on_the_batch():

@@ -98,6 +98,11 @@ def plain_attention(x, w, spec, positions):
     return out.reshape(t, -1) @ w["a.o_proj.weight"].T
 
 
+def dense(out) -> torch.Tensor:
+    """A part's output as a float32 tensor: in bfloat16 a delta of the residual stream comes back as float32 partial sums."""
+    return out.to_tensor(torch.float32) if hasattr(out, "to_tensor") else out.float()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("variant", ["qwen", "no_norm_partial_rotary", "no_position_window", "mha_scaled"])
 def test_attention_part_alone_whole_and_in_portions(dtype, variant):
@@ -118,13 +123,13 @@ def test_attention_part_alone_whole_and_in_portions(dtype, variant):
     x = torch.randn(n, 72).to(TORCH[dtype])
     want = plain_attention(x.float(), w, spec, torch.arange(n))
     table = [[7, 3, 11]]
-    whole = mixer.forward(x.cuda(), batch_for([(table, 0, n)]), cache).float().cpu()
+    whole = dense(mixer.forward(x.cuda(), batch_for([(table, 0, n)]), cache)).cpu()
     close(whole, want, dtype)
     # the same tokens in portions, from the cache the earlier portions left: 20 | 2 | 1 | 22
     cache.k_cache.zero_(), cache.v_cache.zero_()
     outs, lo = [], 0
     for m in (20, 2, 1, 22):
-        outs.append(mixer.forward(x[lo : lo + m].cuda(), batch_for([(table, lo, m)]), cache).float().cpu())
+        outs.append(dense(mixer.forward(x[lo : lo + m].cuda(), batch_for([(table, lo, m)]), cache)).cpu())
         lo += m
     close(torch.cat(outs), want, dtype)
 
