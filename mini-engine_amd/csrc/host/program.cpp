@@ -247,11 +247,11 @@ class Run {
     const int gated = (int)op.i[2];  // 0, or the code of the gate's activation
     if (k != h_) throw Error(kBadValue, "a product behind a norm reads the hidden size");
     const int n = gated ? rows_of_w / 2 : rows_of_w;
-    // decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
-    // residual buffer, since other blocks of the kernel still read the first
-    // a row or two: the weight-streaming kernel adds and norms the rows itself while its first weights are on their
+    // Decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
+    // residual buffer, since other blocks of the kernel still read the first.
+    // A row or two: the weight-streaming kernel adds and norms the rows itself while its first weights are on their
     // way, whatever the delta is (one row: 857 -> 967 tokens/s, two: 1,605 -> 1,700; from four rows on every block's
-    // reads of the partial sums cost more than the launch they save: 2,749 -> 2,668)
+    // reads of the partial sums cost more than the launch they save: 2,749 -> 2,668).
     if (dtype_ == kBF16 && t_ <= kNormStreamRows && me_gemm_bf16_stream_norm_fits(t_, k) && streams(t_, rows_of_w, k)) {
       const bool adds = pending_.any();
       ok(me_gemm_bf16_stream_norm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w_norm, op.f[0],
@@ -261,6 +261,8 @@ class Run {
       release_parts();
       return;
     }
+    // Up to 16 rows with nothing, or a tensor, to add (the first layer's norm; parts of other kinds): the small kernel's
+    // prologue.
     if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts && !weight_bound(t_, rows_of_w, k)) {
       ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
                             bufs_[op.out], t_, n, k, 1, gated, dtype_, 1, stream_));
