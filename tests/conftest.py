@@ -39,10 +39,19 @@ def tiny_configs():
     d = Qwen3Config(vocab_size=448, hidden_size=256, intermediate_size=384, num_hidden_layers=2,
                     num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
                     rope_theta=1e6, max_position_embeddings=4096, tie_word_embeddings=False)
-    return {"A": a, "B": b, "C": c, "D": d}
+    # widths that are no multiple of 8 or of 4 (the bfloat16 products fall to the kernels that take any size, the norms
+    # to the scalar kernel), as many kv heads as heads, pages of 32
+    e = Qwen3Config(vocab_size=5003, hidden_size=113, intermediate_size=101, num_hidden_layers=3,
+                    num_attention_heads=5, num_key_value_heads=5, head_dim=64, rms_norm_eps=3e-6,
+                    rope_theta=50000.0, max_position_embeddings=1024, tie_word_embeddings=True)
+    # a head size that is no power of two and seven heads to a kv head
+    f = Qwen3Config(vocab_size=1000, hidden_size=200, intermediate_size=344, num_hidden_layers=2,
+                    num_attention_heads=21, num_key_value_heads=3, head_dim=96, rms_norm_eps=1e-5,
+                    rope_theta=10000.0, max_position_embeddings=2048, tie_word_embeddings=False)
+    return {"A": a, "B": b, "C": c, "D": d, "E": e, "F": f}
 
 
-BLOCK_SIZES = {"A": 16, "B": 8, "C": 16, "D": 16}
+BLOCK_SIZES = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 32, "F": 16}
 
 
 def write_tiny(folder: str, cfg, seed: int = 0, std: float = 0.02, dtype=torch.bfloat16) -> str:

@@ -50,7 +50,7 @@ def plain_for(folders, name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_replay_matches_plain(tiny_folders, name, dtype, mode):
     reqs = requests_for(name)
@@ -72,7 +72,7 @@ def test_replay_matches_plain(tiny_folders, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 def test_modes_agree_with_each_other_beyond_rounding(tiny_folders, name, dtype):
     """The logits at a position do not depend on the cut: compare the modes directly, row by row
     (float32: the same sums in the same order, so nearly the same bits; bfloat16: the kernels of
