@@ -171,6 +171,48 @@ def test_random_workload_is_the_same_replayed_and_eager(peaked, name):
     assert outs[True] == outs[False]
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_arrivals_temperatures_and_end_tokens_in_every_mode(peaked, name):
+    """Three hundred requests that arrive a few per step while others run, greedy and with two temperatures, half of
+    them ending at an end token: an engine with graphs and steps launched ahead, one with neither, and one with so
+    few pages and seats that it preempts all the time give every request the same tokens in float32 (a draw is
+    keyed on seed, request and position, so temperature requests too)."""
+    import random
+
+    from mini_engine_amd import SamplingParams
+
+    folder, pcfg, _ = peaked[name]
+    rng = random.Random(17)
+    shared = [rng.randrange(1, pcfg.vocab_size) for _ in range(64)]
+    work = []
+    for _ in range(300):
+        p = [rng.randrange(1, pcfg.vocab_size) for _ in range(rng.choice([1, 2, 5, 17, 33, 64, 100, 130]))]
+        if rng.random() < 0.4:
+            p = shared[: rng.choice([16, 32, 48, 64])] + p
+        work.append((p, rng.choice([1, 2, 3, 8, 20, 45, 60]), rng.choice([0.0, 0.0, 0.7, 1.3]), rng.random() < 0.5))
+    outs = {}
+    for mode, (graphs, ahead, seats, blocks) in {"fast": (True, True, 12, 40), "plain": (False, False, 12, 40),
+                                                 "tight": (True, True, 5, 22)}.items():
+        eng = engine(folder, name, block_size=16, num_blocks=blocks, max_num_seqs=seats, max_num_batched_tokens=112,
+                     max_model_len=320, cuda_graphs=graphs, decode_ahead=ahead, seed=11)
+        eng.scheduler.eos_token_ids = set(range(1, pcfg.vocab_size, 13))  # one id in thirteen ends a request
+        arrivals = random.Random(3)
+        seqs, pending = [], list(work)
+        while pending or eng.scheduler.has_unfinished() or eng._launched:
+            for _ in range(arrivals.choice([0, 1, 1, 2, 4])):
+                if pending:
+                    p, m, temp, ignore = pending.pop(0)
+                    seqs.append(eng.add_request(p, SamplingParams(max_tokens=m, temperature=temp, ignore_eos=ignore)))
+            if eng.scheduler.has_unfinished() or eng._launched:
+                eng.step()
+        outs[mode] = [list(s.output_token_ids) for s in seqs]
+        assert all(len(pool.free_pool) == pool.num_blocks for pool in eng.block_manager.pools)
+        assert eng.scheduler.num_preemptions > 0 and eng.scheduler.num_cached_tokens > 0
+        assert (eng.runner.graph_replays > 100) == graphs
+    assert outs["fast"] == outs["plain"] == outs["tight"]
+    assert any(len(o) < m for o, (_, m, _, ignore) in zip(outs["fast"], work) if not ignore)  # some did end at an end token
+
+
 def test_bfloat16_generation_stays_close(peaked):
     """bfloat16 cannot promise equal tokens (near-ties flip, reference DECISIONS.md:80-82): the first
     tokens agree, and each engine token is one the plain logits rank near the top."""
