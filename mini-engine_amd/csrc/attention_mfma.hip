@@ -609,10 +609,27 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   const long long run_waves = (long long)items * nkv * ((nh / nkv + 15) / 16) * run_splits;
   const int depth = (run_keys <= 256 || run_waves <= 1024) ? 2 : 1;
   // Few splits (a step of many items): one block takes all splits of its heads, a wave each, adds their
-  // results up itself and writes the output; the second kernel is not needed then.
+  // results up itself and writes the output; the second kernel is not needed then. Such a block is a whole
+  // (item, kv head) of work and a compute unit takes in only so much per microsecond, so this pays only where the
+  // blocks divide evenly among the compute units: 512 blocks on 256 units yes (batch 64: 5% ahead of one wave a
+  // block and the second kernel), and up to 256 (a block a unit: 17 to 32 items, 3-7% ahead), but 320 or 384 no
+  // (batch 40: 8,280 -> 8,850 tokens/s with a wave a block: a unit had one block or two, and the step waited for
+  // the units with two).
   int block_waves = (num_splits > 1 && num_splits <= DECODE_BLOCK_WAVES(d)) ? num_splits : 1;
   const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
   if ((size_t)block_waves * heads_most * (d + 2) * sizeof(float) > 48 * 1024) block_waves = 1;  // LDS for the sum
+  if (block_waves > 1) {
+    static int cus = 0;
+    if (cus <= 0) {
+      int dev = 0;
+      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+          cus <= 0)
+        cus = 256;
+    }
+    const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);
+    const long long rounds = (blocks + cus - 1) / cus;
+    if (blocks > cus && blocks * 10 < rounds * cus * 9) block_waves = 1;  // rounds that are less than nine tenths full
+  }
   const float sl = scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
 #define ME_DECODE_CASE(DD)                                                                                      \
