@@ -9,7 +9,9 @@
 // waves are arranged WN x WK: WN groups of 16 columns, WK runs of 128 / WK k within a step, whose partial sums
 // are added through LDS at the end. With k_splits > 1 the grid's second dimension cuts k into runs of whole
 // steps, each block writing float32 partial sums behind those of the splits before it, for the caller to add
-// up (the next residual add does): products with few columns then still fill the chip.
+// up (the next residual add does): products with few columns then still fill the chip. The grid's first dimension
+// deals the columns out in fours, as evenly as they go: the host picks arrangement, runs and blocks so that the launch
+// is whole rounds of the compute units where it can (plan_for_runs, plan_with_runs below).
 //
 // Products use v_mfma_f32_16x16x32_bf16 in the transposed arrangement (C^T[n, m] = sum_k W[n, k] X[m, k]):
 // lane l feeds W[n0 + l % 16][8 k] and X[m0 + l % 16][8 k] (k = 32 c + 8 (l / 16) ..) and receives
@@ -41,7 +43,12 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int wn = wave % WN, wk = wave / WN;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = (blockIdx.x * WN + wn) * 16;
+  // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN) blocks gives every
+  // block 16 WN columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
+  const int fours = (N + 3) / 4;
+  const int c0 = (int)((long long)blockIdx.x * fours / gridDim.x) * 4;
+  const int c1 = min(N, (int)((long long)(blockIdx.x + 1) * fours / gridDim.x) * 4);
+  const int n0 = c0 + wn * 16;
   const int n = n0 + r;
 
   const int total_steps = (K + kStepK - 1) / kStepK;
@@ -57,7 +64,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(X), 0, x_bytes, kBufferFlags);
   uint32_t w_base[ACCS];
 #pragma unroll
-  for (int a = 0; a < ACCS; ++a) w_base[a] = n < N ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
+  for (int a = 0; a < ACCS; ++a) w_base[a] = n < c1 ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
   uint32_t x_base[XV];  // row m of thread's i-th vector (rows beyond M lie beyond the buffer)
   int x_k[XV];
 #pragma unroll
@@ -162,6 +169,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
       if (SWIGLU) y[j] = gate_act(y[j], gate) * acc[t][1][j];
     }
     OutT* dst = C + (size_t)m * N + nb;
+    if (nb >= c1) continue;
     if (nb + 3 < N && (N & 3) == 0) {
       if (sizeof(OutT) == 4) {
         *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
@@ -202,7 +210,12 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int wn = wave % WN, wk = wave / WN;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = (blockIdx.x * WN + wn) * 16;
+  // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN) blocks gives every
+  // block 16 WN columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
+  const int fours = (N + 3) / 4;
+  const int c0 = (int)((long long)blockIdx.x * fours / gridDim.x) * 4;
+  const int c1 = min(N, (int)((long long)(blockIdx.x + 1) * fours / gridDim.x) * 4);
+  const int n0 = c0 + wn * 16;
   const int n = n0 + r;
   const int steps = (K + kStepK - 1) / kStepK;
 
@@ -210,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(W), 0, w_bytes, kBufferFlags);
   uint32_t w_base[ACCS];
 #pragma unroll
-  for (int a = 0; a < ACCS; ++a) w_base[a] = n < N ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
+  for (int a = 0; a < ACCS; ++a) w_base[a] = n < c1 ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
   suint4_t w[STAGES][ACCS][CH];
   auto load_step = [&](int step, suint4_t (&wd)[ACCS][CH]) {
     const int k0 = step * kStepK;
@@ -331,6 +344,7 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
     if (SWIGLU) y[j] = gate_act(y[j], gate) * (acc[1][j] * scale);
   }
   OutT* dst = C + (size_t)m * N + nb;
+  if (nb >= c1) return;
   if (nb + 3 < N && (N & 3) == 0) {
     if (sizeof(OutT) == 4) {
       *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
@@ -347,10 +361,75 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
   }
 }
 
+// How a product is laid over the chip: the waves' arrangement (wn groups of 16 columns, 4 / wn runs of k within a
+// step), the runs of k across blocks, and the blocks along the columns.
+struct StreamPlan {
+  int wn, splits, grid;
+};
+
+// A compute unit streams at a fixed rate, so a product takes as long as the unit with the most blocks: the blocks
+// along the columns are as many as there are runs of 16 wn columns, or up to a third more if the launch then is whole
+// rounds of the compute units, or just short of them (every block then has fewer columns, all about as many).
+int whole_rounds(int base, int splits, int compute_units) {
+  const long long rounds = ((long long)base * splits + compute_units - 1) / compute_units;
+  const long long grid = rounds * compute_units / splits;
+  return grid >= base && 3 * grid <= 4ll * base ? (int)grid : base;
+}
+
+int runs_of(int steps, int want) {  // `want` runs of whole steps, none empty
+  const int per = (steps + want - 1) / want;
+  return (steps + per - 1) / per;
+}
+
+// A product with a given number of runs of k (one, for a result that is no partial sum). Up to 16 rows, where x is
+// small: the widest arrangement whose blocks fill whole rounds of the compute units, two rounds for the gated form, which
+// keeps half as many steps in flight per wave (measured, weights of 8 to 524 MB; 6,144 x 4,096 at one row: 12.0 us
+// with 256 blocks of two tiles against 15.4 with 384 of one; the gated 2 x 25,600 x 5,120: 96 us with 512 blocks of 50
+// columns, 109 with 400 of 64), else the widest one with two blocks per unit. With more rows the fetches of x weigh
+// more than an uneven round (10,240 x 5,120 at 64 rows: 41 us with 160 blocks of 64 columns, 54 with 768 of 16): the
+// widest arrangement with half a block per unit.
+StreamPlan plan_for_runs(int M, int N, bool gated, int splits, int compute_units) {
+  const int tiles = (N + 15) / 16;
+  const int least_rounds = gated ? 2 : 1;
+  for (int wn = 4; wn >= 1 && M <= 16; wn >>= 1) {
+    const int base = (tiles + wn - 1) / wn, grid = whole_rounds(base, splits, compute_units);
+    const long long total = (long long)grid * splits, rounds = (total + compute_units - 1) / compute_units;
+    if (rounds >= least_rounds && total * 16 >= rounds * compute_units * 15) return {wn, splits, grid};
+  }
+  const long long want = M <= 16 ? 2ll * compute_units : compute_units / 2;
+  int wn = 4;
+  while (wn > 1 && (long long)((tiles + wn - 1) / wn) * splits < want) wn >>= 1;
+  return {wn, splits, whole_rounds((tiles + wn - 1) / wn, splits, compute_units)};
+}
+
+// A product whose result may stay partial sums over runs of k: the widest arrangement that, with k cut into runs of
+// at least four steps (16 runs at most), gives about one block per compute unit, at least half as many (measured: 4,096 x
+// 12,288 at one row: 19.8 us with 4 runs of 64 blocks of 64 columns against 21.3 with 8 runs of 256 blocks of 16;
+// 5,120 x 25,600: 46 against 51; at 64 rows 65 against 71; 1,024 x 3,072: 4.5-5.0 against 5.2).
+StreamPlan plan_with_runs(int M, int N, int K, int compute_units) {
+  const int tiles = (N + 15) / 16, steps = (K + kStepK - 1) / kStepK;
+  const int most = std::max(1, std::min(steps / 4, 16));
+  for (int wn = 4; wn >= 1; wn >>= 1) {
+    const int base = (tiles + wn - 1) / wn;
+    const int splits = runs_of(steps, std::max(1, std::min(most, (compute_units + base / 2) / base)));
+    if (2ll * base * splits >= compute_units || wn == 1) return {wn, splits, whole_rounds(base, splits, compute_units)};
+  }
+  return {1, 1, tiles};  // (not reached)
+}
+
+StreamPlan plan_of(int M, int N, int K, bool gated, int k_splits, int compute_units) {
+  if (k_splits > 1) {
+    const StreamPlan p = plan_with_runs(M, N, K, compute_units);
+    if (p.splits == k_splits) return p;
+  }
+  return plan_for_runs(M, N, gated, k_splits, compute_units);
+}
+
 template <int MT, bool SWIGLU, typename OutT>
-void launch_arranged(int wn, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int splits, int steps_per_split,
+void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int steps_per_split,
                      int gate, hipStream_t stream) {
-  const dim3 grid(((N + 15) / 16 + wn - 1) / wn, splits);
+  const dim3 grid(plan.grid, plan.splits);
+  const int wn = plan.wn;
   if (wn == 4)
     gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
   else if (wn == 2)
@@ -360,43 +439,28 @@ void launch_arranged(int wn, const bf16_t* X, const bf16_t* W, OutT* C, int M, i
 }
 
 template <bool SWIGLU, typename OutT>
-void launch_rows(int wn, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int splits, int steps_per_split,
-                 int gate, hipStream_t stream) {
+void launch_rows(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int steps_per_split, int gate,
+                 hipStream_t stream) {
   switch ((M + 15) / 16) {
-    case 1: launch_arranged<1, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
-    case 2: launch_arranged<2, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
-    case 3: launch_arranged<3, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
-    default: launch_arranged<4, SWIGLU, OutT>(wn, X, W, C, M, N, K, splits, steps_per_split, gate, stream); break;
+    case 1: launch_arranged<1, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
+    case 2: launch_arranged<2, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
+    case 3: launch_arranged<3, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
+    default: launch_arranged<4, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
   }
 }
 
 }  // namespace
 
-// How many columns' worth of waves a block gets (4, 2 or 1 groups of 16 columns; the other waves cut k): the
-// widest arrangement that still gives the chip enough blocks, since wider blocks fetch x less often. Up to 16
-// rows x is small and two blocks per compute unit stream best; with more rows the fetches of x weigh more and
-// half a block per compute unit is enough (measured at 32 and 64 rows, 6,144 to 25,600 columns: 16-53 us with
-// this rule against 21-63 with the other).
-extern "C" int me_gemm_bf16_stream_arrangement(int M, int N, int k_splits, int compute_units) {
-  const int tiles = (N + 15) / 16;
-  const long long want = M <= 16 ? 2ll * compute_units : compute_units / 2;
-  for (int wn = 4; wn > 1; wn >>= 1)
-    if ((long long)((tiles + wn - 1) / wn) * k_splits >= want) return wn;
-  return 1;
+// Into how many runs of k a product of M rows whose result may stay partial sums is cut (see plan_with_runs).
+extern "C" int me_gemm_bf16_stream_splits(int M, int N, int K, int compute_units) {
+  return plan_with_runs(M, N, K, compute_units < 1 ? 256 : compute_units).splits;
 }
 
-// Into how many runs of k a product of M rows whose result may stay partial sums is cut: blocks of 64 columns, as
-// many runs as fill the chip with whole rounds of blocks, each of at least four steps of 128. Up to 16 rows two
-// blocks per compute unit stream best; with more rows (more of x per block) one does, and a number of blocks just
-// past a multiple of the compute units costs most (64 rows, 5,120 x 25,600: 3 runs of 80 blocks 65 us, 6 runs
-// 69, 7 runs 80; 4,096 x 4,096: 4 runs of 64 blocks 12.0 us, 8 runs 14.2).
-extern "C" int me_gemm_bf16_stream_splits(int M, int N, int K, int compute_units) {
-  const int blocks = ((N + 15) / 16 + 3) / 4;
-  const int steps = (K + kStepK - 1) / kStepK;
-  const int room = (M <= 16 ? 2 : 1) * compute_units;
-  const int want = max(1, min(min(room / blocks, steps / 4), 16));
-  const int steps_per_split = (steps + want - 1) / want;
-  return (steps + steps_per_split - 1) / steps_per_split;  // no empty run
+// What me_gemm_bf16_stream launches for a product: out[0] the groups of 16 columns per block (the other waves cut k
+// within a step), out[1] the runs of k, out[2] the blocks along the columns.
+extern "C" void me_gemm_bf16_stream_plan(int M, int N, int K, int gated, int k_splits, int compute_units, int* out) {
+  const StreamPlan p = plan_of(M, N, K, gated != 0, k_splits, compute_units < 1 ? 256 : compute_units);
+  out[0] = p.wn, out[1] = p.splits, out[2] = p.grid;
 }
 
 // C[M, N] = x . W^T (swiglu 1 or 2, a MeGate code: W is [2 N, K], gate rows then up rows, and C = act(gate) * up), X bfloat16 [M, K],
@@ -422,25 +486,25 @@ extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M,
   const int steps_per_split = (steps + k_splits - 1) / k_splits;
   const int splits = (steps + steps_per_split - 1) / steps_per_split;  // no empty run
   if (splits != k_splits) return me_fail("me_gemm_bf16_stream: K=%d cannot be cut into %d runs of whole steps", K, k_splits);
-  const int wn = me_gemm_bf16_stream_arrangement(M, N, splits, compute_units);
+  const StreamPlan plan = plan_of(M, N, K, swiglu != 0, splits, compute_units);
   const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
   if (swiglu)
-    launch_rows<true, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, swiglu, stream);
+    launch_rows<true, bf16_t>(plan, x, w, (bf16_t*)C, M, N, K, steps_per_split, swiglu, stream);
   else if (out_dtype == ME_F32)
-    launch_rows<false, float>(wn, x, w, (float*)C, M, N, K, splits, steps_per_split, 0, stream);
+    launch_rows<false, float>(plan, x, w, (float*)C, M, N, K, steps_per_split, 0, stream);
   else
-    launch_rows<false, bf16_t>(wn, x, w, (bf16_t*)C, M, N, K, splits, steps_per_split, 0, stream);
+    launch_rows<false, bf16_t>(plan, x, w, (bf16_t*)C, M, N, K, steps_per_split, 0, stream);
   return me_check_launch("me_gemm_bf16_stream");
 }
 
 namespace {
 
 template <bool SWIGLU, typename OutT>
-int launch_norm(int wn, const float* x_in, const bf16_t* delta, const float* parts, int num_parts, size_t part_stride,
+int launch_norm(StreamPlan plan, const float* x_in, const bf16_t* delta, const float* parts, int num_parts, size_t part_stride,
                 const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K, int gate,
                 hipStream_t stream) {
-  const dim3 grid(((N + 15) / 16 + wn - 1) / wn);
-  const int wk = 4 / wn;
+  const dim3 grid(plan.grid);
+  const int wn = plan.wn, wk = 4 / wn;
   const size_t rows_bytes = (((size_t)M * (K + 8) * 2 + 15) & ~(size_t)15) + (size_t)M * 4 * sizeof(float);
   const size_t sums_bytes = (64 + (size_t)(wk - 1) * wn * (SWIGLU ? 2 : 1) * 4 * 64) * sizeof(float);
   const size_t lds = std::max(rows_bytes, sums_bytes);
@@ -489,12 +553,12 @@ extern "C" int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, co
   if ((size_t)(swiglu ? 2 : 1) * N * K * 2 >= (1ull << 31))
     return me_fail("me_gemm_bf16_stream_norm: weights of 2 GiB and more are not addressed by this kernel");
   if (compute_units < 1) compute_units = 256;
-  const int wn = me_gemm_bf16_stream_arrangement(M, N, 1, compute_units);
+  const StreamPlan plan = plan_of(M, N, K, swiglu != 0, 1, compute_units);
   const bf16_t *d = (const bf16_t*)delta, *w = (const bf16_t*)W;
   const size_t stride = parts ? (size_t)part_stride : 0;
   if (swiglu)
-    return launch_norm<true, bf16_t>(wn, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, swiglu, stream);
+    return launch_norm<true, bf16_t>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, swiglu, stream);
   if (out_dtype == ME_F32)
-    return launch_norm<false, float>(wn, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (float*)C, M, N, K, 0, stream);
-  return launch_norm<false, bf16_t>(wn, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, 0, stream);
+    return launch_norm<false, float>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (float*)C, M, N, K, 0, stream);
+  return launch_norm<false, bf16_t>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, 0, stream);
 }

@@ -47,8 +47,8 @@ int me_gemm_plain(const void* A, const void* W, void* C, int M, int N, int K, in
 int me_gemm_bf16_small(const void* X, const float* x_in, const void* delta, const float* w_norm, float eps, float* x_out,
                        const void* W, void* C, int M, int N, int K, int norm, int swiglu, int out_dtype, int k_splits,
                        hipStream_t stream);
-int me_gemm_bf16_stream_arrangement(int M, int N, int k_splits, int compute_units);
 int me_gemm_bf16_stream_splits(int M, int N, int K, int compute_units);
+void me_gemm_bf16_stream_plan(int M, int N, int K, int gated, int k_splits, int compute_units, int* out);
 int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype, int k_splits,
                         int compute_units, hipStream_t stream);
 int me_gemm_bf16_stream_norm_fits(int M, int K);

@@ -401,6 +401,14 @@ def stream_splits(n: int, k: int, device=None, rows: int = 1) -> int:
     return int(lib().me_gemm_bf16_stream_splits(_i(rows), _i(n), _i(k), _i(compute_units(device))))
 
 
+def stream_plan(rows: int, n: int, k: int, gated: bool = False, k_splits: int = 1, device=None) -> tuple[int, int, int]:
+    """What :func:`gemm_bf16_stream` launches for a product: (groups of 16 columns per block, runs of k, blocks along
+    the columns). The columns are dealt to the blocks in fours, as evenly as they go."""
+    out = (ctypes.c_int * 3)()
+    lib().me_gemm_bf16_stream_plan(_i(rows), _i(n), _i(k), _i(int(bool(gated))), _i(k_splits), _i(compute_units(device)), out)
+    return int(out[0]), int(out[1]), int(out[2])
+
+
 def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
                      out: torch.Tensor | None = None, k_splits: int = 1) -> torch.Tensor:
     """bfloat16 ``x @ weight.T`` for at most 64 rows and weights large enough that streaming them is the

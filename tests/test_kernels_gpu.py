@@ -300,12 +300,15 @@ def test_gemm_bf16_small_with_very_many_columns(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 16, 128), (7, 100, 72), (16, 1040, 1000), (17, 4099, 1536), (33, 200, 2056), (48, 68, 8200),
-                                   (64, 9000, 648), (64, 40, 136)])
+                                   (64, 9000, 648), (64, 40, 136), (2, 3072, 264), (8, 6140, 128), (3, 6142, 136), (5, 1000, 3072)])
 @pytest.mark.parametrize("gated", [True, False])
 def test_gemm_bf16_stream(m, n, k, gated):
     """The weight-streaming product at every row-tile count, with column counts that are no multiple of a
     block's (every arrangement of a block's waves: many, some and few columns), k that is no multiple of a
-    step, both output types, the gated form, and partial sums over runs of k whose sum is the product."""
+    step, both output types, the gated form, and partial sums over runs of k whose sum is the product. The
+    last four shapes are dealt to more blocks than they have runs of a block's columns (whole rounds of the
+    compute units), so that blocks begin and end inside a tile of 16, at column counts that are a multiple of 16,
+    of 4, or of neither."""
     g = torch.Generator().manual_seed(m * 977 + n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
     w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
@@ -329,7 +332,8 @@ def test_gemm_bf16_stream(m, n, k, gated):
         assert parts[-1].abs().max() > 0
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 4096, 1024), (2, 100, 1000), (3, 1040, 72), (4, 68, 2056), (1, 16, 128), (2, 9000, 648)])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 1024), (2, 100, 1000), (3, 1040, 72), (4, 68, 2056), (1, 16, 128), (2, 9000, 648),
+                                   (1, 3072, 1024), (2, 6142, 264)])
 @pytest.mark.parametrize("delta", ["none", "tensor", "parts3", "parts6"])
 @pytest.mark.parametrize("gated", [False, "silu", "gelu_tanh"])
 def test_gemm_bf16_stream_norm(m, n, k, delta, gated):
@@ -366,6 +370,33 @@ def test_gemm_bf16_stream_norm(m, n, k, delta, gated):
         else:
             assert h.residual is spare
             torch.testing.assert_close(spare.cpu(), s, rtol=1e-6, atol=1e-6)
+
+
+def test_stream_plan_deals_columns_in_whole_rounds():
+    """What the plan promises, on any number of compute units: the blocks cover all columns, a block has at most
+    its waves' 16 columns each, and the runs of k are whole steps of which none is empty. On 256 compute units: the
+    shapes this file tests the uneven deal with do get one, and the layer shapes the choice was measured on get
+    what was measured best."""
+    cus = K().compute_units(torch.device("cuda:0"))
+    for m in (1, 8, 16, 17, 64):
+        for n, k in ((16, 128), (1000, 3072), (3072, 1024), (4096, 4096), (6142, 136), (10240, 5120), (25600, 5120), (151936, 1024)):
+            for gated in (False, True):
+                for may_split in (False, True):
+                    splits = K().stream_splits(n, k, rows=m) if may_split and not gated else 1
+                    wn, runs, grid = K().stream_plan(m, n, k, gated, splits)
+                    assert wn in (1, 2, 4) and runs == splits
+                    fours = -(-n // 4)
+                    assert grid >= -(-n // (16 * wn)) and -(-fours // grid) * 4 <= 16 * wn, (m, n, k, gated, wn, runs, grid)
+                    steps = -(-k // 128)
+                    assert -(-steps // -(-steps // runs)) == runs
+    if cus != 256:
+        return
+    assert K().stream_plan(2, 3072, 264, True) == (1, 1, 256)  # 192 tiles of 16 columns on 256 blocks of 12
+    assert K().stream_plan(8, 6140, 128) == (2, 1, 256)
+    assert K().stream_plan(5, 1000, 3072, False, K().stream_splits(1000, 3072, rows=5)) == (2, 6, 42)
+    assert K().stream_plan(1, 25600, 5120, True) == (4, 1, 512) and K().stream_plan(1, 6144, 4096) == (2, 1, 256)
+    assert K().stream_plan(1, 4096, 12288, False, K().stream_splits(4096, 12288)) == (4, 4, 64)
+    assert K().stream_plan(64, 10240, 5120) == (4, 1, 160)  # many rows: wide blocks before whole rounds
 
 
 def test_gemm_bf16_stream_norm_refuses_what_it_cannot_do():
