@@ -31,25 +31,25 @@ constexpr int kStepK = 128;          // k per block and step
 constexpr int kBufferFlags = 0x00020000;  // a raw buffer of 32-bit words (gfx9 family)
 constexpr int kRow = kStepK + 16;    // LDS row stride in elements: 288 bytes, 32 off a multiple of 64 (conflict-free 16-byte reads)
 
-template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES>
+template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int NT = 1>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                           OutT* __restrict__ C, int M, int N, int K, int steps_per_split, int gate) {
   static_assert(WN * WK == 4, "four waves per block");
+  static_assert(NT == 1 || WK == 1, "waves with several tiles of columns do not cut k");
   constexpr int KC = kStepK / WK;  // k per wave and step
-  constexpr int CH = KC / 32;      // products per wave, step and tile of rows
-  constexpr int ACCS = SWIGLU ? 2 : 1;
+  constexpr int CH = KC / 32;      // products per wave, step, tile of rows and tile of columns
+  constexpr int ACCS = (SWIGLU ? 2 : 1) * NT;  // tiles of 16 columns per wave: NT of them, gate and up of each in the gated form
   constexpr int XV = MT * 16 * (kStepK / 8) / 256;  // 16-byte vectors of x per thread and step
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][kRow];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int wn = wave % WN, wk = wave / WN;
   const int r = lane & 15, g = lane >> 4;
-  // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN) blocks gives every
-  // block 16 WN columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
+  // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN NT) blocks gives every
+  // block 16 WN NT columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
   const int fours = (N + 3) / 4;
   const int c0 = (int)((long long)blockIdx.x * fours / gridDim.x) * 4;
   const int c1 = min(N, (int)((long long)(blockIdx.x + 1) * fours / gridDim.x) * 4);
-  const int n0 = c0 + wn * 16;
-  const int n = n0 + r;
+  const int n0 = c0 + wn * NT * 16;  // the wave's first tile; tile i begins 16 i columns on
 
   const int total_steps = (K + kStepK - 1) / kStepK;
   const int first = blockIdx.y * steps_per_split;
@@ -62,9 +62,12 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   const uint32_t w_bytes = (uint32_t)((size_t)(SWIGLU ? 2 : 1) * N * K * 2), x_bytes = (uint32_t)((size_t)M * K * 2);
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(W), 0, w_bytes, kBufferFlags);
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(X), 0, x_bytes, kBufferFlags);
-  uint32_t w_base[ACCS];
+  uint32_t w_base[ACCS];  // accumulator a: tile a % NT of the wave, its up rows if a >= NT
 #pragma unroll
-  for (int a = 0; a < ACCS; ++a) w_base[a] = n < c1 ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
+  for (int a = 0; a < ACCS; ++a) {
+    const int n = n0 + (a % NT) * 16 + r;
+    w_base[a] = n < c1 ? (uint32_t)(((a >= NT ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
+  }
   uint32_t x_base[XV];  // row m of thread's i-th vector (rows beyond M lie beyond the buffer)
   int x_k[XV];
 #pragma unroll
@@ -156,33 +159,36 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
           for (int j = 0; j < 4; ++j) acc[t][a][j] += theirs[((t * ACCS + a) * 4 + j) * 64 + lane];
     }
   }
-  // lane (r, g) holds rows m = 16 t + r, columns n0 + 4 g .. +4
-  const int nb = n0 + 4 * g;
+  // lane (r, g) holds rows m = 16 t + r, columns 4 g .. +4 of each of its tiles
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + r;
-    if (m >= M) continue;
-    float y[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      y[j] = acc[t][0][j];
-      if (SWIGLU) y[j] = gate_act(y[j], gate) * acc[t][1][j];
-    }
-    OutT* dst = C + (size_t)m * N + nb;
+  for (int i = 0; i < NT; ++i) {
+    const int nb = n0 + 16 * i + 4 * g;
     if (nb >= c1) continue;
-    if (nb + 3 < N && (N & 3) == 0) {
-      if (sizeof(OutT) == 4) {
-        *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
-      } else {
-        uint2 packed;
-        packed.x = (uint32_t)f32_to_bf16_bits(y[0]) | ((uint32_t)f32_to_bf16_bits(y[1]) << 16);
-        packed.y = (uint32_t)f32_to_bf16_bits(y[2]) | ((uint32_t)f32_to_bf16_bits(y[3]) << 16);
-        *reinterpret_cast<uint2*>(dst) = packed;
-      }
-    } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (nb + j < N) dst[j] = from_float<OutT>(y[j]);
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + r;
+      if (m >= M) continue;
+      float y[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        y[j] = acc[t][i][j];
+        if (SWIGLU) y[j] = gate_act(y[j], gate) * acc[t][NT + i][j];
+      }
+      OutT* dst = C + (size_t)m * N + nb;
+      if (nb + 3 < N && (N & 3) == 0) {
+        if (sizeof(OutT) == 4) {
+          *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
+        } else {
+          uint2 packed;
+          packed.x = (uint32_t)f32_to_bf16_bits(y[0]) | ((uint32_t)f32_to_bf16_bits(y[1]) << 16);
+          packed.y = (uint32_t)f32_to_bf16_bits(y[2]) | ((uint32_t)f32_to_bf16_bits(y[3]) << 16);
+          *reinterpret_cast<uint2*>(dst) = packed;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (nb + j < N) dst[j] = from_float<OutT>(y[j]);
+      }
     }
   }
 }
@@ -364,7 +370,7 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
 // How a product is laid over the chip: the waves' arrangement (wn groups of 16 columns, 4 / wn runs of k within a
 // step), the runs of k across blocks, and the blocks along the columns.
 struct StreamPlan {
-  int wn, splits, grid;
+  int wn, splits, grid, nt;  // nt: tiles of 16 columns per wave
 };
 
 // A compute unit streams at a fixed rate, so a product takes as long as the unit with the most blocks: the blocks
@@ -394,27 +400,34 @@ StreamPlan plan_for_runs(int M, int N, bool gated, int splits, int compute_units
   for (int wn = 4; wn >= 1 && M <= 16; wn >>= 1) {
     const int base = (tiles + wn - 1) / wn, grid = whole_rounds(base, splits, compute_units);
     const long long total = (long long)grid * splits, rounds = (total + compute_units - 1) / compute_units;
-    if (rounds >= least_rounds && total * 16 >= rounds * compute_units * 15) return {wn, splits, grid};
+    if (rounds >= least_rounds && total * 16 >= rounds * compute_units * 15) return {wn, splits, grid, 1};
   }
   const long long want = M <= 16 ? 2ll * compute_units : compute_units / 2;
   int wn = 4;
   while (wn > 1 && (long long)((tiles + wn - 1) / wn) * splits < want) wn >>= 1;
-  return {wn, splits, whole_rounds((tiles + wn - 1) / wn, splits, compute_units)};
+  return {wn, splits, whole_rounds((tiles + wn - 1) / wn, splits, compute_units), 1};
 }
 
 // A product whose result may stay partial sums over runs of k: the widest arrangement that, with k cut into runs of
 // at least four steps (16 runs at most), gives about one block per compute unit, at least half as many (measured: 4,096 x
 // 12,288 at one row: 19.8 us with 4 runs of 64 blocks of 64 columns against 21.3 with 8 runs of 256 blocks of 16;
-// 5,120 x 25,600: 46 against 51; at 64 rows 65 against 71; 1,024 x 3,072: 4.5-5.0 against 5.2).
+// 5,120 x 25,600: 46 against 51; at 64 rows 65 against 71; 1,024 x 3,072: 4.5-5.0 against 5.2). With more than 32 rows
+// a block of 64 columns fetches as many bytes of x as of weights; blocks of 128 columns, two tiles a wave, fetch half as
+// many, but need twice the runs of k to fill the chip, so they are taken where the partial sums of those runs stay small
+// beside the weights (32 x runs x rows <= k: the add-and-norm behind the product reads them too; at 64 rows 5,120 x
+// 25,600: 60 us against 70 and a decode step of that shape 2.4% shorter; 4,096 x 12,288: 27.4 against 30.3 and no gain
+// in the step; 4,096 x 4,096, whose 8 runs write half as many bytes as the weights have: 11.8 against 11.3).
 StreamPlan plan_with_runs(int M, int N, int K, int compute_units) {
   const int tiles = (N + 15) / 16, steps = (K + kStepK - 1) / kStepK;
   const int most = std::max(1, std::min(steps / 4, 16));
-  for (int wn = 4; wn >= 1; wn >>= 1) {
-    const int base = (tiles + wn - 1) / wn;
+  for (int width = (M > 32 ? 8 : 4); width >= 1; width >>= 1) {  // tiles of 16 columns per block
+    const int base = (tiles + width - 1) / width;
     const int splits = runs_of(steps, std::max(1, std::min(most, (compute_units + base / 2) / base)));
-    if (2ll * base * splits >= compute_units || wn == 1) return {wn, splits, whole_rounds(base, splits, compute_units)};
+    if (width == 8 && 32ll * splits * M > K) continue;
+    if (2ll * base * splits >= compute_units || width == 1)
+      return {std::min(width, 4), splits, whole_rounds(base, splits, compute_units), width / std::min(width, 4)};
   }
-  return {1, 1, tiles};  // (not reached)
+  return {1, 1, tiles, 1};  // (not reached)
 }
 
 StreamPlan plan_of(int M, int N, int K, bool gated, int k_splits, int compute_units) {
@@ -430,6 +443,12 @@ void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C,
                      int gate, hipStream_t stream) {
   const dim3 grid(plan.grid, plan.splits);
   const int wn = plan.wn;
+  if constexpr (MT >= 3 && !SWIGLU && sizeof(OutT) == 4) {
+    if (plan.nt == 2) {  // (two steps in flight: 3-15% ahead of three)
+      gemm_stream_kernel<MT, 4, 1, false, OutT, 2, 2><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
+      return;
+    }
+  }
   if (wn == 4)
     gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
   else if (wn == 2)
@@ -460,7 +479,7 @@ extern "C" int me_gemm_bf16_stream_splits(int M, int N, int K, int compute_units
 // within a step), out[1] the runs of k, out[2] the blocks along the columns.
 extern "C" void me_gemm_bf16_stream_plan(int M, int N, int K, int gated, int k_splits, int compute_units, int* out) {
   const StreamPlan p = plan_of(M, N, K, gated != 0, k_splits, compute_units < 1 ? 256 : compute_units);
-  out[0] = p.wn, out[1] = p.splits, out[2] = p.grid;
+  out[0] = p.wn * p.nt, out[1] = p.splits, out[2] = p.grid;
 }
 
 // C[M, N] = x . W^T (swiglu 1 or 2, a MeGate code: W is [2 N, K], gate rows then up rows, and C = act(gate) * up), X bfloat16 [M, K],

@@ -300,15 +300,17 @@ def test_gemm_bf16_small_with_very_many_columns(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 16, 128), (7, 100, 72), (16, 1040, 1000), (17, 4099, 1536), (33, 200, 2056), (48, 68, 8200),
-                                   (64, 9000, 648), (64, 40, 136), (2, 3072, 264), (8, 6140, 128), (3, 6142, 136), (5, 1000, 3072)])
+                                   (64, 9000, 648), (64, 40, 136), (2, 3072, 264), (8, 6140, 128), (3, 6142, 136), (5, 1000, 3072),
+                                   (64, 4096, 16384), (40, 2100, 24576), (33, 4098, 8704)])
 @pytest.mark.parametrize("gated", [True, False])
 def test_gemm_bf16_stream(m, n, k, gated):
     """The weight-streaming product at every row-tile count, with column counts that are no multiple of a
     block's (every arrangement of a block's waves: many, some and few columns), k that is no multiple of a
-    step, both output types, the gated form, and partial sums over runs of k whose sum is the product. The
-    last four shapes are dealt to more blocks than they have runs of a block's columns (whole rounds of the
+    step, both output types, the gated form, and partial sums over runs of k whose sum is the product. Four
+    shapes of up to 8 rows are dealt to more blocks than they have runs of a block's columns (whole rounds of the
     compute units), so that blocks begin and end inside a tile of 16, at column counts that are a multiple of 16,
-    of 4, or of neither."""
+    of 4, or of neither; the last three (more than 32 rows, thousands of columns, long k) take blocks of 128 columns,
+    two tiles a wave, for their partial sums."""
     g = torch.Generator().manual_seed(m * 977 + n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
     w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
@@ -384,7 +386,7 @@ def test_stream_plan_deals_columns_in_whole_rounds():
                 for may_split in (False, True):
                     splits = K().stream_splits(n, k, rows=m) if may_split and not gated else 1
                     wn, runs, grid = K().stream_plan(m, n, k, gated, splits)
-                    assert wn in (1, 2, 4) and runs == splits
+                    assert wn in (1, 2, 4, 8) and runs == splits  # tiles of 16 columns per block
                     fours = -(-n // 4)
                     assert grid >= -(-n // (16 * wn)) and -(-fours // grid) * 4 <= 16 * wn, (m, n, k, gated, wn, runs, grid)
                     steps = -(-k // 128)
@@ -397,6 +399,9 @@ def test_stream_plan_deals_columns_in_whole_rounds():
     assert K().stream_plan(1, 25600, 5120, True) == (4, 1, 512) and K().stream_plan(1, 6144, 4096) == (2, 1, 256)
     assert K().stream_plan(1, 4096, 12288, False, K().stream_splits(4096, 12288)) == (4, 4, 64)
     assert K().stream_plan(64, 10240, 5120) == (4, 1, 160)  # many rows: wide blocks before whole rounds
+    for m, n, k in ((64, 4096, 16384), (40, 2100, 24576), (33, 4098, 8704)):  # blocks of 128 columns, two tiles a wave
+        assert K().stream_plan(m, n, k, False, K().stream_splits(n, k, rows=m))[0] == 8
+    assert K().stream_plan(64, 4096, 4096, False, K().stream_splits(4096, 4096, rows=64))[0] == 4  # its partial sums would weigh too much
 
 
 def test_gemm_bf16_stream_norm_refuses_what_it_cannot_do():
