@@ -28,14 +28,20 @@ typedef uint32_t suint4_t __attribute__((ext_vector_type(4)));
 namespace {
 
 constexpr int kStepK = 128;          // k per block and step
+constexpr int kGroupRows = 64;       // rows per block; more rows are dealt to groups of blocks (the grid's third dimension)
+constexpr int kMaxRows = 256;
 constexpr int kBufferFlags = 0x00020000;  // a raw buffer of 32-bit words (gfx9 family)
 constexpr int kRow = kStepK + 16;    // LDS row stride in elements: 288 bytes, 32 off a multiple of 64 (conflict-free 16-byte reads)
 
 template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int NT = 1>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                          OutT* __restrict__ C, int M, int N, int K, int steps_per_split, int gate) {
+                                                          OutT* __restrict__ C, int rows, int N, int K, int steps_per_split, int gate) {
   static_assert(WN * WK == 4, "four waves per block");
   static_assert(NT == 1 || WK == 1, "waves with several tiles of columns do not cut k");
+  // The grid's third dimension deals the rows out in groups of 16 MT; a block sees its group's rows only.
+  C += (size_t)blockIdx.y * rows * N + (size_t)blockIdx.z * (16 * MT) * N;
+  X += (size_t)blockIdx.z * (16 * MT) * K;
+  const int M = min(16 * MT, rows - (int)blockIdx.z * 16 * MT);
   constexpr int KC = kStepK / WK;  // k per wave and step
   constexpr int CH = KC / 32;      // products per wave, step, tile of rows and tile of columns
   constexpr int ACCS = (SWIGLU ? 2 : 1) * NT;  // tiles of 16 columns per wave: NT of them, gate and up of each in the gated form
@@ -55,7 +61,6 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   const int first = blockIdx.y * steps_per_split;
   const int steps = min(total_steps, first + steps_per_split) - first;
   const int k_end = min(K, (first + steps) * kStepK);  // this block's run of k ends here
-  C += (size_t)blockIdx.y * M * N;
 
   // Loads go through buffer descriptors: an offset at or beyond the buffer's size gives zeros without a
   // branch, which is how rows beyond M or N, k beyond the run and steps beyond the last are handled.
@@ -397,6 +402,8 @@ int runs_of(int steps, int want) {  // `want` runs of whole steps, none empty
 StreamPlan plan_for_runs(int M, int N, bool gated, int splits, int compute_units) {
   const int tiles = (N + 15) / 16;
   const int least_rounds = gated ? 2 : 1;
+  const int groups = (M + kGroupRows - 1) / kGroupRows;  // the same blocks once per group of 64 rows
+  const int across = splits * groups;
   for (int wn = 4; wn >= 1 && M <= 16; wn >>= 1) {
     const int base = (tiles + wn - 1) / wn, grid = whole_rounds(base, splits, compute_units);
     const long long total = (long long)grid * splits, rounds = (total + compute_units - 1) / compute_units;
@@ -404,8 +411,8 @@ StreamPlan plan_for_runs(int M, int N, bool gated, int splits, int compute_units
   }
   const long long want = M <= 16 ? 2ll * compute_units : compute_units / 2;
   int wn = 4;
-  while (wn > 1 && (long long)((tiles + wn - 1) / wn) * splits < want) wn >>= 1;
-  return {wn, splits, whole_rounds((tiles + wn - 1) / wn, splits, compute_units), 1};
+  while (wn > 1 && (long long)((tiles + wn - 1) / wn) * across < want) wn >>= 1;
+  return {wn, splits, whole_rounds((tiles + wn - 1) / wn, across, compute_units), 1};
 }
 
 // A product whose result may stay partial sums over runs of k: the widest arrangement that, with k cut into runs of
@@ -420,12 +427,13 @@ StreamPlan plan_for_runs(int M, int N, bool gated, int splits, int compute_units
 StreamPlan plan_with_runs(int M, int N, int K, int compute_units) {
   const int tiles = (N + 15) / 16, steps = (K + kStepK - 1) / kStepK;
   const int most = std::max(1, std::min(steps / 4, 16));
+  const int groups = (M + kGroupRows - 1) / kGroupRows;  // the same blocks once per group of 64 rows
   for (int width = (M > 32 ? 8 : 4); width >= 1; width >>= 1) {  // tiles of 16 columns per block
-    const int base = (tiles + width - 1) / width;
+    const int base = (tiles + width - 1) / width * groups;
     const int splits = runs_of(steps, std::max(1, std::min(most, (compute_units + base / 2) / base)));
-    if (width == 8 && 32ll * splits * M > K) continue;
+    if (width == 8 && 32ll * splits * std::min(M, kGroupRows) > K) continue;
     if (2ll * base * splits >= compute_units || width == 1)
-      return {std::min(width, 4), splits, whole_rounds(base, splits, compute_units), width / std::min(width, 4)};
+      return {std::min(width, 4), splits, whole_rounds(base / groups, splits * groups, compute_units), width / std::min(width, 4)};
   }
   return {1, 1, tiles, 1};  // (not reached)
 }
@@ -441,7 +449,7 @@ StreamPlan plan_of(int M, int N, int K, bool gated, int k_splits, int compute_un
 template <int MT, bool SWIGLU, typename OutT>
 void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int steps_per_split,
                      int gate, hipStream_t stream) {
-  const dim3 grid(plan.grid, plan.splits);
+  const dim3 grid(plan.grid, plan.splits, (M + kGroupRows - 1) / kGroupRows);
   const int wn = plan.wn;
   if constexpr (MT >= 3 && !SWIGLU && sizeof(OutT) == 4) {
     if (plan.nt == 2) {  // (two steps in flight: 3-15% ahead of three)
@@ -460,7 +468,7 @@ void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C,
 template <bool SWIGLU, typename OutT>
 void launch_rows(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int steps_per_split, int gate,
                  hipStream_t stream) {
-  switch ((M + 15) / 16) {
+  switch ((std::min(M, kGroupRows) + 15) / 16) {
     case 1: launch_arranged<1, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
     case 2: launch_arranged<2, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
     case 3: launch_arranged<3, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
@@ -489,7 +497,7 @@ extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M,
                                    int k_splits, int compute_units, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_stream: unknown gate activation %d", swiglu);
-  if (M > 64) return me_fail("me_gemm_bf16_stream: M=%d exceeds 64 rows", M);
+  if (M > kMaxRows) return me_fail("me_gemm_bf16_stream: M=%d exceeds %d rows", M, kMaxRows);
   if (K <= 0 || K % 8) return me_fail("me_gemm_bf16_stream: K=%d must be a positive multiple of 8", K);
   if (!X || !W || !C) return me_fail("me_gemm_bf16_stream: null operand");
   if (((uintptr_t)X | (uintptr_t)W | (uintptr_t)C) & 15) return me_fail("me_gemm_bf16_stream: operands must be 16-byte aligned");

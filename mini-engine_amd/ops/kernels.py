@@ -386,6 +386,7 @@ class NormedInput:
                 and weight.numel() < STREAM_MIN_ELEMENTS)
 
 
+STREAM_MAX_ROWS = 256  # the weight-streaming product deals more than 64 rows to groups of blocks
 NORM_STREAM_ROWS = 2  # up to here the add-and-norm is the prologue of the weight-streaming kernel
 SMALL_MAX_ROWS = 64  # what the kernel accepts
 SMALL_FAST_ROWS = 16  # up to here it beats the GEMM library on every shape, with the norm as its prologue too
@@ -423,8 +424,8 @@ def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
         if n % 2:
             raise ValueError(f"a gate/up weight needs an even number of rows, got {n}")
         n //= 2
-    if m > SMALL_MAX_ROWS:
-        raise ValueError(f"gemm_bf16_stream takes at most {SMALL_MAX_ROWS} rows, got {m}")
+    if m > STREAM_MAX_ROWS:
+        raise ValueError(f"gemm_bf16_stream takes at most {STREAM_MAX_ROWS} rows, got {m}")
     shape = (k_splits, m, n) if k_splits > 1 else (m, n)
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=weight.device)
@@ -608,7 +609,8 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
     matrix-core kernel, or the weight-streaming one for weights of 16 MiB and more; 17 to 64 rows the
     weight-streaming kernel (the library for weights of 16 MiB and more); a delta of the residual stream
     of up to 64 rows as partial sums over runs of k; the tiled matrix-core kernel with
-    the SwiGLU as its epilogue for gated products of 256 rows or more; else the GEMM library."""
+    the SwiGLU as its epilogue for gated products of 256 rows or more (the weight-streaming kernel up to 256 rows for
+    gated weights below 16 MiB); else the GEMM library."""
     if isinstance(x, NormedInput):
         if x.streams_normed(weight):
             return gemm_bf16_stream_norm(x, weight, out_dtype or x.dtype, gated)
@@ -636,6 +638,9 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return gemm_bf16_stream(x, weight, out_dtype)
     if small_ok(x, weight, gated) and not heavy:
         return gemm_bf16_small(x, weight, out_dtype, gated)
+    if (gated and x.shape[0] <= STREAM_MAX_ROWS and x.shape[1] % 8 == 0 and weight.numel() < STREAM_MIN_ELEMENTS
+            and out_dtype is torch.bfloat16):
+        return gemm_bf16_stream(x, weight, out_dtype, gated)  # 65 to 256 rows of a small gated weight, in groups of 64 rows
     if gated:
         if tiled_ok(x, weight) and x.shape[1] <= TILED_MAX_K and out_dtype is torch.bfloat16:
             return gemm_bf16_tiled(x, weight, out_dtype, gated)  # measured ahead of the library product + SwiGLU kernel

@@ -301,7 +301,8 @@ def test_gemm_bf16_small_with_very_many_columns(m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 16, 128), (7, 100, 72), (16, 1040, 1000), (17, 4099, 1536), (33, 200, 2056), (48, 68, 8200),
                                    (64, 9000, 648), (64, 40, 136), (2, 3072, 264), (8, 6140, 128), (3, 6142, 136), (5, 1000, 3072),
-                                   (64, 4096, 16384), (40, 2100, 24576), (33, 4098, 8704)])
+                                   (64, 4096, 16384), (40, 2100, 24576), (33, 4098, 8704), (65, 520, 264), (130, 3072, 1024),
+                                   (256, 68, 136), (200, 1030, 520)])
 @pytest.mark.parametrize("gated", [True, False])
 def test_gemm_bf16_stream(m, n, k, gated):
     """The weight-streaming product at every row-tile count, with column counts that are no multiple of a
@@ -310,7 +311,8 @@ def test_gemm_bf16_stream(m, n, k, gated):
     shapes of up to 8 rows are dealt to more blocks than they have runs of a block's columns (whole rounds of the
     compute units), so that blocks begin and end inside a tile of 16, at column counts that are a multiple of 16,
     of 4, or of neither; the last three (more than 32 rows, thousands of columns, long k) take blocks of 128 columns,
-    two tiles a wave, for their partial sums."""
+    two tiles a wave, for their partial sums. More than 64 rows go to groups of blocks, 64 rows a group, the last
+    group with fewer."""
     g = torch.Generator().manual_seed(m * 977 + n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
     w = (torch.randn(2 * n if gated else n, k, generator=g) * 0.05).bfloat16()
@@ -418,7 +420,7 @@ def test_gemm_bf16_stream_norm_refuses_what_it_cannot_do():
 
 
 def test_gemm_bf16_stream_refuses_what_it_cannot_do():
-    x, w = dev(torch.zeros(65, 64).bfloat16()), dev(torch.zeros(32, 64).bfloat16())
+    x, w = dev(torch.zeros(257, 64).bfloat16()), dev(torch.zeros(32, 64).bfloat16())
     with pytest.raises(ValueError):
         K().gemm_bf16_stream(x, w)
     x = dev(torch.zeros(4, 68).bfloat16())

@@ -273,8 +273,12 @@ def test_layer_run_twice_shared_cache_and_two_window_groups(dtype):
     assert "model.layers.2.self_attn.k_proj.weight" not in w and "model.layers.2.self_attn.k_norm.weight" not in w
     tokens = torch.randint(1, cfg.vocab_size, (90,), generator=torch.Generator().manual_seed(4)).tolist()
     want = plain_general(plan, w, tokens)
+    # bfloat16: after five runs of a layer single logits of the 34,560 are off by 1.1-2.0% of their row's largest (3 to 3.5
+    # here; measured over eight seeds of tokens, whole and cut alike), which a bound of 0.03 on every element sits in the
+    # middle of; this file's bound for values of that size is relative to the largest of them. float32 keeps the plain one.
+    check = (lambda got: torch.testing.assert_close(got, want, **tol(dtype))) if dtype == "float32" else (lambda got: close(got, want, dtype))
     whole, _ = step_in_portions(runner, tokens, [90])
-    torch.testing.assert_close(whole, want, **tol(dtype))
+    check(whole)
     cut, held = step_in_portions(runner, tokens, [30, 2, 17, 1, 1, 1, 38])
-    torch.testing.assert_close(cut, want, **tol(dtype))
+    check(cut)
     assert held[0] == 6 and held[1] <= 3  # the window group gave passed pages back on the way
