@@ -12,6 +12,9 @@ namespace me {
 namespace {
 
 constexpr int kPieceOverhead = 2;  // what starting another piece of work costs a block, in key tiles (3 us against 1.5)
+constexpr int kCutOverhead = 8;    // what cutting any tile costs a step, in key tiles: partial results written and the kernel that
+                                   // adds them up (one prompt of 65 to 384 tokens: a step 8% longer with cut tiles than without,
+                                   // 512: 3%, 768: the same, 1,024: 2% shorter, 2,048: 5% shorter)
 constexpr long long kPartialBytesMax = 256ll << 20;  // most memory the partial results of cut tiles may take
 
 struct Tile {
@@ -92,7 +95,7 @@ bool wide_blocks_pay(const int* starts, const int* qlens, int items, int tpb, in
 // up to a few thousand tokens, whose causal tiles differ in length by a factor of their number; a short
 // portion over a long context) the tiles are cut into ranges of at most `cap` key tiles, whose partial
 // results a second kernel adds up, and the pieces are packed into one bundle per compute unit; `cap` is
-// the candidate with the shortest longest bundle.
+// the candidate with the shortest longest bundle, where cutting at all counts as kCutOverhead key tiles.
 void build_work_list(const int* starts, const int* qlens, int items, int tpb, int window, int nkv, int slots,
                      long long partial_row_bytes, WorkList& out) {
   std::vector<Tile> tiles;
@@ -133,7 +136,7 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
       if (cap < 1 || (longest + cap - 1) / cap > chunk_limit) continue;
       std::vector<Piece> pieces = cut(tiles, cap);
       std::vector<std::vector<Piece>> loads;
-      const double score = (double)pack(pieces, bins, loads) + 0.01 * (double)pieces.size();
+      const double score = (double)pack(pieces, bins, loads) + (cap < longest ? kCutOverhead : 0) + 0.01 * (double)pieces.size();
       if (!have || score < best_score || (score == best_score && cap < best_cap)) {
         have = true;
         best_score = score;

@@ -63,6 +63,16 @@ def test_causal_prompt_with_one_tile_per_compute_unit_is_evened_out():
     assert max(loads) <= 20 < 32  # whole tiles would give 32 key tiles to the last block
 
 
+def test_short_prompts_are_not_cut():
+    """Cutting costs a step the partial results and the kernel that adds them up: a prompt of a few hundred tokens,
+    whose longest tile walks a few key tiles, is left whole; from about a thousand tokens on it is cut."""
+    for tokens in (65, 128, 256, 512):
+        work, first, max_chunks = check_plan([0], [tokens], 64, 0, 8, 256)
+        assert max_chunks == 1 and work.shape[0] == -(-tokens // 64)
+    for tokens in (1024, 1536):
+        assert check_plan([0], [tokens], 64, 0, 8, 256)[2] > 1
+
+
 def test_short_portion_over_long_context_is_cut_to_fill_the_chip():
     work, first, max_chunks = check_plan([30000, 5], [64, 3], 64, 0, 8, 256)
     assert max_chunks > 8 and len(first) == 32
