@@ -150,16 +150,243 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
   }
 }
 
+// The same attention for steps that bring several tokens per item (prompts, portions): a block takes up to
+// `tq` consecutive tokens of the step and the heads of one kv head, a wave per (token, head), and stages each tile of
+// 64 keys and values in LDS once for all of them, where the kernel above has every wave fetch its own copy (a 2,048-token
+// prompt: 34 GB a layer from the L2). Tokens of a block that belong to different items are served one item after the
+// other. Every wave does the arithmetic of the kernel above in the same order (the products of a score in ascending
+// element, the keys of a tile in ascending position, the same reductions across lanes), so the two kernels give the same
+// bits and a step may use either. float32, head sizes that are a multiple of 4, pages that hold a multiple of 4 keys.
+constexpr int AS_KPAD = 4, AS_VROW = 68;  // LDS rows: a key's d + 4 floats, an element's 64 + 4 keys (16-byte reads of consecutive
+                                           // rows by consecutive lanes without bank conflicts; 8 and 72 measured slower)
+
+// DT: the head size if it is 64, 128 or 256 (loops unroll, no guards), else 0 (any multiple of 4 up to 256).
+template <int DT>
+__global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
+    const float* __restrict__ q, const float* __restrict__ k_cache, const float* __restrict__ v_cache,
+    const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
+    int table_width, float* __restrict__ out, int num_tokens, int nh, int nkv, int d_any, int bs, int bs_shift, int window,
+    float scale, int tq) {
+  constexpr int KMAX = DT ? DT / ME_WAVE : AG_MAX_D / ME_WAVE;  // elements of the output per lane
+  const int d = DT ? DT : d_any, d4 = d / 4;
+  extern __shared__ __attribute__((aligned(16))) float as_lds[];
+  const int waves = blockDim.x / ME_WAVE;
+  float* Ks = as_lds;                      // [64][d + AS_KPAD]
+  float* Vs = Ks + 64 * (d + AS_KPAD);     // [d][AS_VROW]
+  float* qs = Vs + (size_t)d * AS_VROW;    // [waves][d]
+  float* ps = qs + (size_t)waves * d;      // [waves][64]: a tile's weights, for every lane to read
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / ME_WAVE), lane = threadIdx.x & (ME_WAVE - 1);
+  const int group = nh / nkv, kvh = blockIdx.y;
+  // (the step's last tokens first: they are the ones with the most keys before them, and blocks start in this order)
+  const int first = (gridDim.x - 1 - blockIdx.x) * tq, limit = min(first + tq, num_tokens);
+  const int t = first + wave / group, head = kvh * group + wave % group;
+  const bool mine = wave < tq * group && t < limit;
+  float* qw = qs + (size_t)wave * d;
+  float* pw = ps + wave * 64;
+  const int krow_floats = d + AS_KPAD;
+  // staging: a wave copies whole key rows, 64 / dp rows at a time (dp: d4 rounded up to a power of two, lanes beyond d4 idle)
+  int dp_shift = 0;
+  while ((1 << dp_shift) < d4) ++dp_shift;
+  const int k_rows_per_wave = ME_WAVE >> dp_shift, k_row_in_wave = lane >> dp_shift, k_piece = lane & ((1 << dp_shift) - 1);
+  auto page_of = [&](int key, int& slot) {
+    if (bs_shift >= 0) {
+      slot = key & (bs - 1);
+      return key >> bs_shift;
+    }
+    slot = key % bs;
+    return key / bs;
+  };
+
+  for (int seg = first; seg < limit;) {  // runs of tokens of one item (every thread walks the same runs)
+    const int item = token_item[seg];
+    int seg_end = seg + 1;
+    while (seg_end < limit && token_item[seg_end] == item) ++seg_end;
+    const int* table = block_table + (size_t)item * table_width;
+    const int p_first = positions[seg], p_last = positions[seg_end - 1];  // consecutive positions, ascending
+    const int lo_first = window > 0 ? max(p_first - window + 1, 0) : 0;
+    const bool active = mine && t >= seg && t < seg_end;
+    const int p = active ? __builtin_amdgcn_readfirstlane(positions[t]) : 0;
+    const int lo = window > 0 ? max(p - window + 1, 0) : 0;
+    if (active) {
+      const float* qrow = q + ((size_t)t * nh + head) * d;
+      for (int i = lane; i < d; i += ME_WAVE) qw[i] = qrow[i] * scale;
+    }
+    float m = -INFINITY, l = 0.f;
+    float acc[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
+
+    for (int tile = (lo_first / 64) * 64; tile <= p_last; tile += 64) {
+      __syncthreads();  // every wave has left the tile before (and the q rows are written)
+      for (int row = wave * k_rows_per_wave + k_row_in_wave; row < 64; row += waves * k_rows_per_wave) {
+        const int key = tile + row;  // keys up to the last position of the run
+        if (key <= p_last && k_piece < d4) {
+          int slot;
+          const int page = table[page_of(key, slot)];
+          const float* src = k_cache + (((size_t)page * nkv + kvh) * bs + slot) * d + 4 * k_piece;
+          *reinterpret_cast<float4*>(Ks + row * krow_floats + 4 * k_piece) = *reinterpret_cast<const float4*>(src);
+        }
+      }
+      for (int idx = threadIdx.x; idx < d * 16; idx += blockDim.x) {  // four keys of an element at a time (they share a page)
+        const int i = idx >> 4, key = tile + 4 * (idx & 15);
+        if (key <= p_last) {
+          int slot;
+          const int page = table[page_of(key, slot)];
+          const float* src = v_cache + ((size_t)page * nkv + kvh) * d * bs + (size_t)i * bs + slot;
+          *reinterpret_cast<float4*>(Vs + i * AS_VROW + 4 * (idx & 15)) = *reinterpret_cast<const float4*>(src);
+        }
+      }
+      __syncthreads();
+      if (!active || tile > p || tile < (lo / 64) * 64) continue;
+      const int key = tile + lane;
+      const bool valid = key >= lo && key <= p;
+      float s = -INFINITY;
+      if (valid) {
+        const float4* k4 = reinterpret_cast<const float4*>(Ks + lane * krow_floats);
+        const float4* q4 = reinterpret_cast<const float4*>(qw);
+        float dot = 0.f;
+        for (int base = 0; base < d4; base += 8) {  // eight pieces of the row and of q are requested before the first is used
+          float4 kv[8], qv[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int at = DT || base + u < d4 ? base + u : d4 - 1;
+            kv[u] = k4[at], qv[u] = q4[at];
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (DT || base + u < d4) {
+              dot = fmaf(qv[u].x, kv[u].x, dot);
+              dot = fmaf(qv[u].y, kv[u].y, dot);
+              dot = fmaf(qv[u].z, kv[u].z, dot);
+              dot = fmaf(qv[u].w, kv[u].w, dot);
+            }
+        }
+        s = dot;
+      }
+      const float m_new = fmaxf(m, wave_max(s));
+      const float pr = valid ? expf(s - m_new) : 0.f;
+      const float alpha = expf(m - m_new);
+      l = l * alpha + wave_sum(pr);
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) acc[k] *= alpha;
+      m = m_new;
+      pw[lane] = pr;
+      __builtin_amdgcn_wave_barrier();
+      const int j_lo = lo > tile ? lo - tile : 0;
+      const int j_hi = p - tile < 63 ? p - tile : 63;
+      int j = j_lo;
+      for (; j <= j_hi && (j & 3); ++j) {
+        const float pj = pw[j];
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (DT || i < d) acc[k] = fmaf(pj, Vs[i * AS_VROW + j], acc[k]);
+        }
+      }
+      for (; j + 15 <= j_hi; j += 16) {  // four groups of four keys: their values are requested before the first is used
+        float4 vv[4][KMAX], pv[4];
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          pv[gq] = *reinterpret_cast<const float4*>(pw + j + 4 * gq);
+#pragma unroll
+          for (int k = 0; k < KMAX; ++k) {
+            const int i = lane + k * ME_WAVE;
+            vv[gq][k] = *reinterpret_cast<const float4*>(Vs + (DT || i < d ? i : 0) * AS_VROW + j + 4 * gq);
+          }
+        }
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+          for (int k = 0; k < KMAX; ++k)
+            if (DT || lane + k * ME_WAVE < d) {
+              acc[k] = fmaf(pv[gq].x, vv[gq][k].x, acc[k]);
+              acc[k] = fmaf(pv[gq].y, vv[gq][k].y, acc[k]);
+              acc[k] = fmaf(pv[gq].z, vv[gq][k].z, acc[k]);
+              acc[k] = fmaf(pv[gq].w, vv[gq][k].w, acc[k]);
+            }
+      }
+      for (; j + 3 <= j_hi; j += 4) {
+        const float4 pv = *reinterpret_cast<const float4*>(pw + j);
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (DT || i < d) {
+            const float4 vv = *reinterpret_cast<const float4*>(Vs + i * AS_VROW + j);
+            acc[k] = fmaf(pv.x, vv.x, acc[k]);
+            acc[k] = fmaf(pv.y, vv.y, acc[k]);
+            acc[k] = fmaf(pv.z, vv.z, acc[k]);
+            acc[k] = fmaf(pv.w, vv.w, acc[k]);
+          }
+        }
+      }
+      for (; j <= j_hi; ++j) {
+        const float pj = pw[j];
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (DT || i < d) acc[k] = fmaf(pj, Vs[i * AS_VROW + j], acc[k]);
+        }
+      }
+    }
+    if (active) {
+      float* orow = out + ((size_t)t * nh + head) * d;
+      const float inv = 1.f / l;
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (DT || i < d) orow[i] = acc[k] * inv;
+      }
+    }
+    seg = seg_end;
+  }
+}
+
+// `items`: how many items the step's tokens belong to (0: unknown). Steps with two and more tokens per item on
+// average go to the kernel that shares the tiles of keys and values among the tokens of a block; the results are
+// the same bits either way.
 extern "C" int me_attention_general(const void* q, const void* k_cache, const void* v_cache, const int* positions,
                                     const int* token_item, const int* block_table, int table_width, void* out,
                                     int num_tokens, int nh, int nkv, int d, int bs, int window, float scale,
-                                    int dtype, hipStream_t stream) {
+                                    int dtype, int items, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || d > AG_MAX_D) return me_fail("me_attention_general: head_dim=%d must be in 1..%d", d, AG_MAX_D);
   if (nh <= 0 || nkv <= 0 || nh % nkv)
     return me_fail("me_attention_general: %d query heads are not a multiple of %d key/value heads", nh, nkv);
   if (bs <= 0 || table_width <= 0 || window < 0)
     return me_fail("me_attention_general: block_size=%d table_width=%d window=%d", bs, table_width, window);
+  const int group = nh / nkv;
+  if (dtype == ME_F32 && items > 0 && num_tokens >= 2 * items && d % 4 == 0 && bs % 4 == 0 && group <= 16 &&
+      (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0) {
+    const int tq = 16 / group > 0 ? 16 / group : 1, waves = tq * group;
+    const size_t lds = ((size_t)64 * (d + AS_KPAD) + (size_t)d * AS_VROW + (size_t)waves * (d + 64)) * sizeof(float);
+    int bs_shift = -1;
+    if ((bs & (bs - 1)) == 0)
+      for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
+    const dim3 grid((num_tokens + tq - 1) / tq, nkv);
+#define ME_SHARED_LAUNCH(DT)                                                                                                     \
+  do {                                                                                                                           \
+    static size_t allowed = 0; /* grows to the most this head size has asked for */                                             \
+    if (lds > allowed) {                                                                                                         \
+      if (hipFuncSetAttribute((const void*)attention_shared_f32_kernel<DT>, hipFuncAttributeMaxDynamicSharedMemorySize,          \
+                              (int)lds) != hipSuccess)                                                                           \
+        return me_fail("me_attention_general: %zu bytes of block memory for head_dim=%d are refused", lds, d);                   \
+      allowed = lds;                                                                                                             \
+    }                                                                                                                            \
+    attention_shared_f32_kernel<DT><<<grid, waves * 64, lds, stream>>>(                                                          \
+        (const float*)q, (const float*)k_cache, (const float*)v_cache, positions, token_item, block_table, table_width,         \
+        (float*)out, num_tokens, nh, nkv, d, bs, bs_shift, window, scale, tq);                                                   \
+  } while (0)
+    if (d == 64)
+      ME_SHARED_LAUNCH(64);
+    else if (d == 128)
+      ME_SHARED_LAUNCH(128);
+    else if (d == 256)
+      ME_SHARED_LAUNCH(256);
+    else
+      ME_SHARED_LAUNCH(0);
+#undef ME_SHARED_LAUNCH
+    return me_check_launch("me_attention_general");
+  }
   const long long units = (long long)num_tokens * nh;
   const int waves = units < 2048 ? 1 : 4;  // few units (decode steps): a compute unit each
   const unsigned blocks = (unsigned)((units + waves - 1) / waves);

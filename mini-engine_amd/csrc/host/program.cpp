@@ -425,7 +425,7 @@ class Run {
       return;
     }
     ok(me_attention_general(q, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, out, t_, nh, nkv, d, bs, window,
-                            scale, dtype_, stream_));
+                            scale, dtype_, items, stream_));
   }
 
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.

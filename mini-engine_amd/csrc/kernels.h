@@ -24,7 +24,7 @@ int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w,
                             hipStream_t stream);
 int me_attention_general(const void* q, const void* k_cache, const void* v_cache, const int* positions,
                          const int* token_item, const int* block_table, int table_width, void* out, int num_tokens, int nh,
-                         int nkv, int d, int bs, int window, float scale, int dtype, hipStream_t stream);
+                         int nkv, int d, int bs, int window, float scale, int dtype, int items, hipStream_t stream);
 int me_attention_mfma_supported(int d, int bs);
 int me_attention_decode_fused_supported(int d, int bs, int rotary_dim, int group);
 int me_attention_prefill_columns(int wide);

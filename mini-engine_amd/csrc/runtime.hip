@@ -22,4 +22,4 @@ int me_check_launch(const char* what) {
   return 0;
 }
 
-extern "C" int me_abi_version() { return 7; }
+extern "C" int me_abi_version() { return 8; }

@@ -308,8 +308,11 @@ def attention_general(
     scale: float,
     window: int = 0,
     out: torch.Tensor | None = None,
+    shared_tiles: bool = True,
 ) -> torch.Tensor:
-    """Causal grouped-query attention of q [T, nh, d] over the paged cache; returns [T, nh * d]."""
+    """Causal grouped-query attention of q [T, nh, d] over the paged cache; returns [T, nh * d]. float32 steps with
+    two and more tokens per row of the block table go to a kernel whose blocks share the tiles of keys and values among
+    their tokens (``shared_tiles=False``: the kernel with a wave per token and head for every step; the same bits)."""
     _want(q, "q", None, (None, None, None))
     t, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -320,7 +323,8 @@ def attention_general(
     _want(out, "out", q.dtype, (t, nh * d))
     check(lib().me_attention_general(
         _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]),
-        _p(out), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(_code(q.dtype)), _stream()))
+        _p(out), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(_code(q.dtype)),
+        _i(block_table.shape[0] if shared_tiles else 0), _stream()))
     return out
 
 

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
 _lock = threading.Lock()
 _lib: ctypes.CDLL | None = None
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 def _build_module():

@@ -599,6 +599,26 @@ def test_attention_general_mixed_batch(dtype, nh, nkv, d, bs, window):
     torch.testing.assert_close(out.float().cpu(), want, **t)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs", ATTN_SHAPES + [(14, 2, 96, 16), (16, 1, 64, 16), (3, 1, 20, 4)])
+@pytest.mark.parametrize("window", [0, 5, 100])
+def test_attention_general_shares_tiles_without_changing_a_bit(nh, nkv, d, bs, window):
+    """float32 steps with several tokens per item run in the kernel whose blocks share the tiles of keys and values
+    among their tokens: the same bits as a wave per token and head fetching its own, for prompts, portions behind a
+    context, single tokens between them (blocks that serve several items one after the other), windows that end inside
+    and outside a block's tokens, and every group size up to 16 heads per kv head."""
+    items = [(0, 7), (9, 1), (8, 5), (0, 1), (63, 2), (130, 1), (60, 70), (0, 200), (250, 3), (5, 64)]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, torch.float32, num_pages=256)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(6)
+    q = torch.cat([torch.randn(n, nh, d, generator=g) for _, n in items])
+    args = (dev(q), dev(k_cache), dev(v_cache), dev(positions), dev(token_item), dev(table_t), d**-0.5, window)
+    shared = K().attention_general(*args)
+    alone = K().attention_general(*args, shared_tiles=False)
+    assert torch.equal(shared, alone)
+    want = dense_reference(list(torch.split(q, [n for _, n in items])), ks, vs, items, d**-0.5, window)
+    torch.testing.assert_close(shared.cpu(), want, rtol=1e-5, atol=1e-5)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_finds_one_far_key_at_every_page_edge(dtype):
     """One key's score is made to stand out by scaling it and the query; the output must be that
