@@ -103,7 +103,7 @@ def test_engine_config_defaults_and_checks():
 
 def test_pool_sized_by_memory():
     """A share of the GPU's memory instead of a number of pages: what is left of the share after everything already
-    on the GPU and after a step's workspaces, in pages of all layers (SURVEY: sizing helper
+    on the GPU and after a step's workspaces, in pages of all layers (the reference's sizing helper,
     ``engine.py:54-56``: 2 x layers x kv heads x head size x element size per token)."""
     from mini_engine_amd.engine.llm_engine import blocks_that_fit, kv_cache_bytes_per_token
 
