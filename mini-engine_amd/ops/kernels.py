@@ -400,17 +400,20 @@ def compute_units(device=None) -> int:
     return torch.cuda.get_device_properties(device or torch.cuda.current_device()).multi_processor_count
 
 
-def stream_splits(n: int, k: int, device=None, rows: int = 1) -> int:
+def stream_splits(n: int, k: int, device=None, rows: int = 1, units: int | None = None) -> int:
     """Into how many runs of k :func:`gemm_bf16_stream` cuts a product of ``rows`` rows whose result may stay
     partial sums."""
-    return int(lib().me_gemm_bf16_stream_splits(_i(rows), _i(n), _i(k), _i(compute_units(device))))
+    return int(lib().me_gemm_bf16_stream_splits(_i(rows), _i(n), _i(k), _i(units if units is not None else compute_units(device))))
 
 
-def stream_plan(rows: int, n: int, k: int, gated: bool = False, k_splits: int = 1, device=None) -> tuple[int, int, int]:
+def stream_plan(rows: int, n: int, k: int, gated: bool = False, k_splits: int = 1, device=None,
+                units: int | None = None) -> tuple[int, int, int]:
     """What :func:`gemm_bf16_stream` launches for a product: (groups of 16 columns per block, runs of k, blocks along
-    the columns). The columns are dealt to the blocks in fours, as evenly as they go."""
+    the columns). The columns are dealt to the blocks in fours, as evenly as they go. ``units``: plan for this many
+    compute units instead of the device's (a host-side question; no GPU is touched)."""
     out = (ctypes.c_int * 3)()
-    lib().me_gemm_bf16_stream_plan(_i(rows), _i(n), _i(k), _i(int(bool(gated))), _i(k_splits), _i(compute_units(device)), out)
+    lib().me_gemm_bf16_stream_plan(_i(rows), _i(n), _i(k), _i(int(bool(gated))), _i(k_splits),
+                                   _i(units if units is not None else compute_units(device)), out)
     return int(out[0]), int(out[1]), int(out[2])
 
 
