@@ -1,5 +1,6 @@
-// Skinny bfloat16 product y = x . W^T (M <= 64 rows) for weights so large that the kernel's time is the
-// time to stream W from memory once: the projections of models with wide layers, at any decode batch.
+// Skinny bfloat16 product y = x . W^T (M <= 64 rows a block; up to 256 rows in groups of 64, the grid's third
+// dimension) for weights so large that the kernel's time is the time to stream W from memory once: the projections
+// of models with wide layers, at any decode batch.
 //
 // A block of four waves owns 16 * WN output columns and all M rows and walks k in steps of 128. The rows of
 // x that a step needs are staged once per block in LDS (double-buffered, one barrier per step) and shared
@@ -491,7 +492,7 @@ extern "C" void me_gemm_bf16_stream_plan(int M, int N, int K, int gated, int k_s
 }
 
 // C[M, N] = x . W^T (swiglu 1 or 2, a MeGate code: W is [2 N, K], gate rows then up rows, and C = act(gate) * up), X bfloat16 [M, K],
-// M <= 64, K % 8 == 0, pointers 16-byte aligned. out_dtype ME_BF16 or ME_F32. k_splits > 1 (plain float32
+// M <= 256, K % 8 == 0, pointers 16-byte aligned. out_dtype ME_BF16 or ME_F32. k_splits > 1 (plain float32
 // products only): C is [k_splits, M, N], partial sums over runs of k for the caller to add up.
 extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
                                    int k_splits, int compute_units, hipStream_t stream) {

@@ -419,8 +419,8 @@ def stream_plan(rows: int, n: int, k: int, gated: bool = False, k_splits: int = 
 
 def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
                      out: torch.Tensor | None = None, k_splits: int = 1) -> torch.Tensor:
-    """bfloat16 ``x @ weight.T`` for at most 64 rows and weights large enough that streaming them is the
-    kernel's time: x is staged in LDS once per block of columns, the weight goes straight to the matrix
+    """bfloat16 ``x @ weight.T`` for at most 256 rows (64 a block; more rows go to groups of blocks) and weights
+    large enough that streaming them is the kernel's time: x is staged in LDS once per block of columns, the weight goes straight to the matrix
     cores. ``swiglu`` and ``k_splits`` as in :func:`gemm_bf16_small` (``k_splits`` as :func:`stream_splits`
     gives it, or 1)."""
     _want(x, "x", torch.bfloat16, (None, None))
