@@ -202,7 +202,8 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
     int seg_end = seg + 1;
     while (seg_end < limit && token_item[seg_end] == item) ++seg_end;
     const int* table = block_table + (size_t)item * table_width;
-    const int p_first = positions[seg], p_last = positions[seg_end - 1];  // consecutive positions, ascending
+    int p_first = positions[seg], p_last = p_first;  // the run's lowest and highest position (a portion's are consecutive)
+    for (int i = seg + 1; i < seg_end; ++i) p_first = min(p_first, positions[i]), p_last = max(p_last, positions[i]);
     const int lo_first = window > 0 ? max(p_first - window + 1, 0) : 0;
     const bool active = mine && t >= seg && t < seg_end;
     const int p = active ? __builtin_amdgcn_readfirstlane(positions[t]) : 0;
