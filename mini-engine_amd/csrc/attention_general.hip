@@ -5,23 +5,44 @@
 //
 // A token at absolute position p of item b sees keys lo..p of item b, lo = max(0, p - window + 1)
 // (window == 0: lo = 0). Keys are visited in tiles of 64 aligned to absolute position (tile t holds
-// positions 64t .. 64t+63), so the order of every sum depends on p, lo and the head alone, never on
-// how the sequence was cut into steps or on what else is in the batch.
+// positions 64t .. 64t+63), four tiles to a chunk (chunk c holds positions 256c .. 256c+255): the tiles of a
+// chunk update a running (maximum, sum, weighted values) from nothing, and the chunks' results are merged in
+// ascending order. So the order of every sum depends on p, lo and the head alone, never on how the sequence
+// was cut into steps, on what else is in the batch, or on how many waves share the chunks of a token.
 //
 // Cache layout per layer: keys K[page, kv_head, slot, d]; values transposed V[page, kv_head, d, slot].
 #include "common.h"
 
 #define AG_MAX_D 256
 
+#define AG_CHUNK 256  // keys per chunk
+
+// One chunk's result into the running one, the same operations wherever it is called. With nothing before
+// (mt = -inf, lt = 0, acct = 0) the chunk's result comes through unchanged: exp(-inf) = 0 and exp(0) = 1.
+template <int KMAX>
+__device__ __forceinline__ void ag_merge(float& mt, float& lt, float (&acct)[KMAX], float mc, float lc, const float (&accc)[KMAX]) {
+  const float mn = fmaxf(mt, mc);
+  const float at = expf(mt - mn), ac = expf(mc - mn);
+  lt = fmaf(lt, at, lc * ac);
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) acct[k] = fmaf(acct[k], at, accc[k] * ac);
+  mt = mn;
+}
+
+// `wpu` waves per (token, head): 1 (a block of four waves serves four of them), or all waves of the block for one,
+// which then take the chunks in turns, a round of wpu chunks at a time, and wave 0 merges the round's results in order.
 template <typename T>
-__global__ __launch_bounds__(256) void attention_general_kernel(
+__global__ __launch_bounds__(512) void attention_general_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
-    int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int bs, int window, float scale) {
-  __shared__ float qs[4][AG_MAX_D];
+    int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int bs, int window, float scale, int wpu) {
+  constexpr int KMAX = AG_MAX_D / ME_WAVE;
+  __shared__ float qs[8][AG_MAX_D];
+  __shared__ float parts[8][AG_MAX_D + 2];  // with several waves per unit: a round's results (values, maximum, sum)
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
-  const long long unit = (long long)blockIdx.x * (blockDim.x / ME_WAVE) + wave;
-  if (unit >= (long long)num_tokens * nh) return;
+  const int w = wave % wpu;
+  const long long unit = (long long)blockIdx.x * (blockDim.x / ME_WAVE / wpu) + wave / wpu;
+  if (unit >= (long long)num_tokens * nh) return;  // (with several waves per unit: the whole block)
   const int t = (int)(unit / nh), head = (int)(unit % nh);
   const int kvh = head / (nh / nkv);
   const int p = positions[t];
@@ -33,14 +54,23 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
   for (int i = lane; i < d; i += ME_WAVE) qw[i] = to_float(qrow[i]) * scale;
   __builtin_amdgcn_wave_barrier();
 
-  float m = -INFINITY, l = 0.f;
-  float acc[AG_MAX_D / ME_WAVE];
+  float mt = -INFINITY, lt = 0.f;
+  float acct[KMAX];
 #pragma unroll
-  for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) acc[k] = 0.f;
+  for (int k = 0; k < KMAX; ++k) acct[k] = 0.f;
 
   const bool vec_k = sizeof(T) == 4 && d % 4 == 0 && ((uintptr_t)k_cache & 15) == 0;   // a key row in 16-byte pieces
   const bool vec_v = sizeof(T) == 4 && bs % 4 == 0 && ((uintptr_t)v_cache & 15) == 0;  // four keys of a value row at once
-  for (int tile = (lo / 64) * 64; tile <= p; tile += 64) {
+  const int first_chunk = lo / AG_CHUNK, n_chunks = p / AG_CHUNK - first_chunk + 1;
+  for (int round = 0; round * wpu < n_chunks; ++round) {
+  const int ci = round * wpu + w;  // this wave's chunk of the round, if there is one
+  float m = -INFINITY, l = 0.f;
+  float acc[KMAX];
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
+  const int chunk0 = (first_chunk + ci) * AG_CHUNK;
+  const int tile_first = ci < n_chunks ? max(chunk0, (lo / 64) * 64) : 1, tile_last = ci < n_chunks ? min(p, chunk0 + AG_CHUNK - 1) : 0;
+  for (int tile = tile_first; tile <= tile_last; tile += 64) {
     const int key = tile + lane;
     const bool valid = key >= lo && key <= p;
     float s = -INFINITY;
@@ -141,12 +171,32 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
       }
     }
   }
-  T* orow = out + ((size_t)t * nh + head) * d;
-  const float inv = 1.f / l;
+  if (wpu == 1) {
+    ag_merge<KMAX>(mt, lt, acct, m, l, acc);
+  } else {  // the round's results go through LDS to wave 0, which merges them in the order of their chunks
+    if (ci < n_chunks) {
 #pragma unroll
-  for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+      for (int k = 0; k < KMAX; ++k) parts[w][lane + k * ME_WAVE] = acc[k];
+      if (lane == 0) parts[w][AG_MAX_D] = m, parts[w][AG_MAX_D + 1] = l;
+    }
+    __syncthreads();
+    if (w == 0)
+      for (int o = 0; o < wpu && round * wpu + o < n_chunks; ++o) {
+        float accc[KMAX];
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) accc[k] = parts[o][lane + k * ME_WAVE];
+        ag_merge<KMAX>(mt, lt, acct, parts[o][AG_MAX_D], parts[o][AG_MAX_D + 1], accc);
+      }
+    __syncthreads();
+  }
+  }
+  if (w != 0) return;
+  T* orow = out + ((size_t)t * nh + head) * d;
+  const float inv = 1.f / lt;
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
     const int i = lane + k * ME_WAVE;
-    if (i < d) orow[i] = from_float<T>(acc[k] * inv);
+    if (i < d) orow[i] = from_float<T>(acct[k] * inv);
   }
 }
 
@@ -212,10 +262,10 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
       const float* qrow = q + ((size_t)t * nh + head) * d;
       for (int i = lane; i < d; i += ME_WAVE) qw[i] = qrow[i] * scale;
     }
-    float m = -INFINITY, l = 0.f;
-    float acc[KMAX];
+    float m = -INFINITY, l = 0.f, mt = -INFINITY, lt = 0.f;  // the chunk in hand, and the chunks before it merged
+    float acc[KMAX], acct[KMAX];
 #pragma unroll
-    for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
+    for (int k = 0; k < KMAX; ++k) acc[k] = 0.f, acct[k] = 0.f;
 
     for (int tile = (lo_first / 64) * 64; tile <= p_last; tile += 64) {
       __syncthreads();  // every wave has left the tile before (and the q rows are written)
@@ -239,6 +289,12 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
       }
       __syncthreads();
       if (!active || tile > p || tile < (lo / 64) * 64) continue;
+      if (tile % AG_CHUNK == 0 && tile > lo) {  // a chunk begins behind another one of this token: that one is complete
+        ag_merge<KMAX>(mt, lt, acct, m, l, acc);
+        m = -INFINITY, l = 0.f;
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
+      }
       const int key = tile + lane;
       const bool valid = key >= lo && key <= p;
       float s = -INFINITY;
@@ -330,12 +386,13 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
       }
     }
     if (active) {
+      ag_merge<KMAX>(mt, lt, acct, m, l, acc);  // the last chunk
       float* orow = out + ((size_t)t * nh + head) * d;
-      const float inv = 1.f / l;
+      const float inv = 1.f / lt;
 #pragma unroll
       for (int k = 0; k < KMAX; ++k) {
         const int i = lane + k * ME_WAVE;
-        if (DT || i < d) orow[i] = acc[k] * inv;
+        if (DT || i < d) orow[i] = acct[k] * inv;
       }
     }
     seg = seg_end;
@@ -389,15 +446,16 @@ extern "C" int me_attention_general(const void* q, const void* k_cache, const vo
     return me_check_launch("me_attention_general");
   }
   const long long units = (long long)num_tokens * nh;
-  const int waves = units < 2048 ? 1 : 4;  // few units (decode steps): a compute unit each
-  const unsigned blocks = (unsigned)((units + waves - 1) / waves);
+  // few units (decode steps): a block of eight waves each, which share a token's chunks of keys; else four units a block
+  const int wpu = units < 2048 ? 8 : 1, waves = units < 2048 ? 8 : 4;
+  const unsigned blocks = (unsigned)((units + waves / wpu - 1) / (waves / wpu));
   if (dtype == ME_F32)
     attention_general_kernel<float><<<blocks, waves * 64, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, positions, token_item, block_table,
-        table_width, (float*)out, num_tokens, nh, nkv, d, bs, window, scale);
+        table_width, (float*)out, num_tokens, nh, nkv, d, bs, window, scale, wpu);
   else
     attention_general_kernel<bf16_t><<<blocks, waves * 64, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, token_item, block_table,
-        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, bs, window, scale);
+        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, bs, window, scale, wpu);
   return me_check_launch("me_attention_general");
 }

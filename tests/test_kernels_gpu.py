@@ -605,9 +605,11 @@ def test_attention_general_shares_tiles_without_changing_a_bit(nh, nkv, d, bs, w
     """float32 steps with several tokens per item run in the kernel whose blocks share the tiles of keys and values
     among their tokens: the same bits as a wave per token and head fetching its own, for prompts, portions behind a
     context, single tokens between them (blocks that serve several items one after the other), windows that end inside
-    and outside a block's tokens, and every group size up to 16 heads per kv head."""
-    items = [(0, 7), (9, 1), (8, 5), (0, 1), (63, 2), (130, 1), (60, 70), (0, 200), (250, 3), (5, 64)]
-    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, torch.float32, num_pages=256)
+    and outside a block's tokens, contexts of several chunks, and every group size up to 16 heads per kv head. With few
+    heads the kernel it is held against runs eight waves per token and head, which share the chunks; with many, one."""
+    items = [(0, 7), (9, 1), (8, 5), (0, 1), (63, 2), (130, 1), (60, 70), (0, 200), (250, 3), (5, 64),
+             (1000, 40), (767, 2), (255, 1), (256, 1), (511, 3)]  # the last five: several chunks of 256 keys, and their edges
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, torch.float32, num_pages=1200)
     fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
     g = torch.Generator().manual_seed(6)
     q = torch.cat([torch.randn(n, nh, d, generator=g) for _, n in items])
