@@ -92,6 +92,44 @@ def test_modes_agree_with_each_other_beyond_rounding(tiny_folders, name, dtype):
             assert (err <= tol * scale).all(), (name, rid, (err / scale).max().item())
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_long_contexts_in_portions_and_decoded(tiny_folders, name, dtype):
+    """Thousands of keys: a 3,000-token request in portions of 512 (from the second on a short run of queries behind a
+    long context: the prefill attention cuts its tiles into key ranges and a second kernel adds them up; in float32 a
+    run's tiles of keys are shared in LDS over a dozen chunks of 256), a 1,500-token request that joins it in portions
+    of 700, and the last eight tokens of both decoded one by one, side by side (many splits of a long context per
+    item; in float32 eight waves that take a token's chunks in turns). Logits are taken at the end of every portion, at a
+    few places inside, and at every decoded token."""
+    vocab = tiny_configs()[name].vocab_size
+    reqs = {"long": random_prompt(3000, vocab, seed=31), "mid": random_prompt(1500, vocab, seed=32)}
+    cuts = {"long": [512] * 5 + [432] + [1] * 8, "mid": [0, 0, 700, 700, 92] + [0] + [1] * 8}
+    steps, done = [], {"long": 0, "mid": 0}
+    for i in range(len(cuts["long"])):
+        entries = []
+        for rid in ("long", "mid"):
+            n = cuts[rid][i]
+            if n:
+                want = sorted({0, n // 3, n - 1})
+                entries.append({"id": rid, "tokens": reqs[rid][done[rid]:done[rid] + n], "want": want, "at": [done[rid] + j for j in want]})
+                done[rid] += n
+        steps.append({"step": i, "entries": entries, "end": [rid for rid in reqs if done[rid] == len(reqs[rid]) and cuts[rid][i]]})
+    assert done == {"long": 3000, "mid": 1500}
+    from mini_engine_amd.engine.trace import TraceSession, build_session
+
+    session = TraceSession(build_session(tiny_folders[name], dtype, 3008 + 1536, block_size=BLOCK_SIZES[name]))
+    want = th.plain_logits(tiny_folders[name], reqs)
+    for st in steps:
+        out = torch.from_numpy(session.run_step({k: ([{kk: vv for kk, vv in e.items() if kk != "at"} for e in v] if k == "entries" else v)
+                                                 for k, v in st.items()}).copy())
+        r = 0
+        for e in st["entries"]:
+            th.assert_logits_close(out[r:r + len(e["at"])], want[e["id"]][e["at"]], dtype, f"{name} {dtype} step {st['step']} {e['id']}")
+            r += len(e["at"])
+        assert r == out.shape[0]
+    assert not session.live
+
+
 def test_first_tokens_of_a_sequence(tiny_folders):
     """Positions 0 and 1 alone: a one-token prompt, then its second token."""
     for name in ("A", "B"):
