@@ -1,5 +1,5 @@
-// Causal grouped-query attention over the paged cache, for any mix of items in a step: one wave
-// per (new token, query head). It takes every size the cache allows (any page size, any group
+// Causal grouped-query attention over the paged cache, for any mix of items in a step: one wave, or a
+// block of eight, per (new token, query head). It takes every size the cache allows (any page size, any group
 // size, head sizes up to 256 in steps of 2) in float32 or bfloat16 storage, and is the kernel of
 // the 32-bit path; the bfloat16 path uses the matrix-core kernels where their size limits hold.
 //
@@ -20,7 +20,8 @@
 // One chunk's result into the running one, the same operations wherever it is called. With nothing before
 // (mt = -inf, lt = 0, acct = 0) the chunk's result comes through unchanged: exp(-inf) = 0 and exp(0) = 1.
 template <int KMAX>
-__device__ __forceinline__ void ag_merge(float& mt, float& lt, float (&acct)[KMAX], float mc, float lc, const float (&accc)[KMAX]) {
+__device__ __forceinline__ void ag_merge(float& mt, float& lt, float (&acct)[KMAX], float mc, float lc,
+                                         const float (&accc)[KMAX]) {
   const float mn = fmaxf(mt, mc);
   const float at = expf(mt - mn), ac = expf(mc - mn);
   lt = fmaf(lt, at, lc * ac);
@@ -63,132 +64,133 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
   const bool vec_v = sizeof(T) == 4 && bs % 4 == 0 && ((uintptr_t)v_cache & 15) == 0;  // four keys of a value row at once
   const int first_chunk = lo / AG_CHUNK, n_chunks = p / AG_CHUNK - first_chunk + 1;
   for (int round = 0; round * wpu < n_chunks; ++round) {
-  const int ci = round * wpu + w;  // this wave's chunk of the round, if there is one
-  float m = -INFINITY, l = 0.f;
-  float acc[KMAX];
+    const int ci = round * wpu + w;  // this wave's chunk of the round, if there is one
+    float m = -INFINITY, l = 0.f;
+    float acc[KMAX];
 #pragma unroll
-  for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
-  const int chunk0 = (first_chunk + ci) * AG_CHUNK;
-  const int tile_first = ci < n_chunks ? max(chunk0, (lo / 64) * 64) : 1, tile_last = ci < n_chunks ? min(p, chunk0 + AG_CHUNK - 1) : 0;
-  for (int tile = tile_first; tile <= tile_last; tile += 64) {
-    const int key = tile + lane;
-    const bool valid = key >= lo && key <= p;
-    float s = -INFINITY;
-    if (valid) {
-      const int page = table[key / bs];
-      const T* krow = k_cache + (((size_t)page * nkv + kvh) * bs + key % bs) * d;
-      float dot = 0.f;
-      if (vec_k) {  // the same products in the same order; 128 elements of the row are requested before the first is used
-        const float4* k4 = reinterpret_cast<const float4*>(krow);
-        const int n4 = d / 4;
-        for (int base = 0; base < n4; base += 32) {
-          float4 kv[32];
+    for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
+    const int chunk0 = (first_chunk + ci) * AG_CHUNK;
+    const int tile_first = ci < n_chunks ? max(chunk0, (lo / 64) * 64) : 1;  // (no chunk left for this wave: no tiles)
+    const int tile_last = ci < n_chunks ? min(p, chunk0 + AG_CHUNK - 1) : 0;
+    for (int tile = tile_first; tile <= tile_last; tile += 64) {
+      const int key = tile + lane;
+      const bool valid = key >= lo && key <= p;
+      float s = -INFINITY;
+      if (valid) {
+        const int page = table[key / bs];
+        const T* krow = k_cache + (((size_t)page * nkv + kvh) * bs + key % bs) * d;
+        float dot = 0.f;
+        if (vec_k) {  // the same products in the same order; 128 elements of the row are requested before the first is used
+          const float4* k4 = reinterpret_cast<const float4*>(krow);
+          const int n4 = d / 4;
+          for (int base = 0; base < n4; base += 32) {
+            float4 kv[32];
 #pragma unroll
-          for (int u = 0; u < 32; ++u) kv[u] = base + u < n4 ? k4[base + u] : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int u = 0; u < 32; ++u) kv[u] = base + u < n4 ? k4[base + u] : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-          for (int u = 0; u < 32; ++u)
-            if (base + u < n4) {
-              const int i = 4 * (base + u);
-              dot = fmaf(qw[i], kv[u].x, dot);
-              dot = fmaf(qw[i + 1], kv[u].y, dot);
-              dot = fmaf(qw[i + 2], kv[u].z, dot);
-              dot = fmaf(qw[i + 3], kv[u].w, dot);
-            }
+            for (int u = 0; u < 32; ++u)
+              if (base + u < n4) {
+                const int i = 4 * (base + u);
+                dot = fmaf(qw[i], kv[u].x, dot);
+                dot = fmaf(qw[i + 1], kv[u].y, dot);
+                dot = fmaf(qw[i + 2], kv[u].z, dot);
+                dot = fmaf(qw[i + 3], kv[u].w, dot);
+              }
+          }
+        } else {
+          for (int i = 0; i < d; ++i) dot = fmaf(qw[i], to_float(krow[i]), dot);
         }
-      } else {
-        for (int i = 0; i < d; ++i) dot = fmaf(qw[i], to_float(krow[i]), dot);
+        s = dot;
       }
-      s = dot;
-    }
-    const float m_new = fmaxf(m, wave_max(s));  // at least one key of the tile is visible
-    const float pr = valid ? expf(s - m_new) : 0.f;
-    const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first tile
-    l = l * alpha + wave_sum(pr);
+      const float m_new = fmaxf(m, wave_max(s));  // at least one key of the tile is visible
+      const float pr = valid ? expf(s - m_new) : 0.f;
+      const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first tile
+      l = l * alpha + wave_sum(pr);
 #pragma unroll
-    for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) acc[k] *= alpha;
-    m = m_new;
-    const int j_lo = lo > tile ? lo - tile : 0;
-    const int j_hi = p - tile < 63 ? p - tile : 63;
-    int j = j_lo;
-    if (vec_v) {
-      // whole groups of four keys that lie in one page (tiles and groups are aligned to 4, pages hold a multiple of
-      // 4): one 16-byte load per group and element of the head, the sums in the order of the keys as below
-      for (; j <= j_hi && (j & 3); ++j) {
+      for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) acc[k] *= alpha;
+      m = m_new;
+      const int j_lo = lo > tile ? lo - tile : 0;
+      const int j_hi = p - tile < 63 ? p - tile : 63;
+      int j = j_lo;
+      if (vec_v) {
+        // whole groups of four keys that lie in one page (tiles and groups are aligned to 4, pages hold a multiple of
+        // 4): one 16-byte load per group and element of the head, the sums in the order of the keys as below
+        for (; j <= j_hi && (j & 3); ++j) {
+          const float pj = __shfl(pr, j, ME_WAVE);
+          const int kj = tile + j;
+          const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * d * bs + kj % bs;
+#pragma unroll
+          for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+            const int i = lane + k * ME_WAVE;
+            if (i < d) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
+          }
+        }
+        // eight groups of four keys at a time: their values are requested before the first is used
+        const int groups = j <= j_hi ? (j_hi + 1 - j) / 4 : 0;  // whole groups from j on
+        for (int g0 = 0; g0 < groups; g0 += 8) {
+          float4 vv[8][AG_MAX_D / ME_WAVE];
+#pragma unroll
+          for (int gq = 0; gq < 8; ++gq) {
+            const bool there = g0 + gq < groups;
+            const int kj = tile + j + 4 * (there ? g0 + gq : 0);
+            const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * d * bs + kj % bs;
+#pragma unroll
+            for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+              const int i = lane + k * ME_WAVE;
+              vv[gq][k] = make_float4(0.f, 0.f, 0.f, 0.f);
+              if (there && i < d) vv[gq][k] = *reinterpret_cast<const float4*>(vbase + (size_t)i * bs);
+            }
+          }
+#pragma unroll
+          for (int gq = 0; gq < 8; ++gq) {
+            if (g0 + gq < groups) {
+              const int jj = j + 4 * (g0 + gq);
+              const float p0 = __shfl(pr, jj, ME_WAVE), p1 = __shfl(pr, jj + 1, ME_WAVE), p2 = __shfl(pr, jj + 2, ME_WAVE),
+                          p3 = __shfl(pr, jj + 3, ME_WAVE);
+#pragma unroll
+              for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+                if (lane + k * ME_WAVE < d) {
+                  acc[k] = fmaf(p0, vv[gq][k].x, acc[k]);
+                  acc[k] = fmaf(p1, vv[gq][k].y, acc[k]);
+                  acc[k] = fmaf(p2, vv[gq][k].z, acc[k]);
+                  acc[k] = fmaf(p3, vv[gq][k].w, acc[k]);
+                }
+              }
+            }
+          }
+        }
+        j += 4 * groups;
+      }
+      for (; j <= j_hi; ++j) {
         const float pj = __shfl(pr, j, ME_WAVE);
         const int kj = tile + j;
-        const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * d * bs + kj % bs;
+        const int page = table[kj / bs];
+        const T* vbase = v_cache + ((size_t)page * nkv + kvh) * d * bs + kj % bs;
 #pragma unroll
         for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
           const int i = lane + k * ME_WAVE;
           if (i < d) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
         }
       }
-      // eight groups of four keys at a time: their values are requested before the first is used
-      const int groups = j <= j_hi ? (j_hi + 1 - j) / 4 : 0;  // whole groups from j on
-      for (int g0 = 0; g0 < groups; g0 += 8) {
-        float4 vv[8][AG_MAX_D / ME_WAVE];
+    }
+    if (wpu == 1) {
+      ag_merge<KMAX>(mt, lt, acct, m, l, acc);
+    } else {  // the round's results go through LDS to wave 0, which merges them in the order of their chunks
+      if (ci < n_chunks) {
 #pragma unroll
-        for (int gq = 0; gq < 8; ++gq) {
-          const bool there = g0 + gq < groups;
-          const int kj = tile + j + 4 * (there ? g0 + gq : 0);
-          const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * d * bs + kj % bs;
+        for (int k = 0; k < KMAX; ++k) parts[w][lane + k * ME_WAVE] = acc[k];
+        if (lane == 0) parts[w][AG_MAX_D] = m, parts[w][AG_MAX_D + 1] = l;
+      }
+      __syncthreads();
+      if (w == 0)
+        for (int o = 0; o < wpu && round * wpu + o < n_chunks; ++o) {
+          float accc[KMAX];
 #pragma unroll
-          for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
-            const int i = lane + k * ME_WAVE;
-            vv[gq][k] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (there && i < d) vv[gq][k] = *reinterpret_cast<const float4*>(vbase + (size_t)i * bs);
-          }
+          for (int k = 0; k < KMAX; ++k) accc[k] = parts[o][lane + k * ME_WAVE];
+          ag_merge<KMAX>(mt, lt, acct, parts[o][AG_MAX_D], parts[o][AG_MAX_D + 1], accc);
         }
-#pragma unroll
-        for (int gq = 0; gq < 8; ++gq) {
-          if (g0 + gq < groups) {
-            const int jj = j + 4 * (g0 + gq);
-            const float p0 = __shfl(pr, jj, ME_WAVE), p1 = __shfl(pr, jj + 1, ME_WAVE), p2 = __shfl(pr, jj + 2, ME_WAVE),
-                        p3 = __shfl(pr, jj + 3, ME_WAVE);
-#pragma unroll
-            for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
-              if (lane + k * ME_WAVE < d) {
-                acc[k] = fmaf(p0, vv[gq][k].x, acc[k]);
-                acc[k] = fmaf(p1, vv[gq][k].y, acc[k]);
-                acc[k] = fmaf(p2, vv[gq][k].z, acc[k]);
-                acc[k] = fmaf(p3, vv[gq][k].w, acc[k]);
-              }
-            }
-          }
-        }
-      }
-      j += 4 * groups;
+      __syncthreads();
     }
-    for (; j <= j_hi; ++j) {
-      const float pj = __shfl(pr, j, ME_WAVE);
-      const int kj = tile + j;
-      const int page = table[kj / bs];
-      const T* vbase = v_cache + ((size_t)page * nkv + kvh) * d * bs + kj % bs;
-#pragma unroll
-      for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
-        const int i = lane + k * ME_WAVE;
-        if (i < d) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
-      }
-    }
-  }
-  if (wpu == 1) {
-    ag_merge<KMAX>(mt, lt, acct, m, l, acc);
-  } else {  // the round's results go through LDS to wave 0, which merges them in the order of their chunks
-    if (ci < n_chunks) {
-#pragma unroll
-      for (int k = 0; k < KMAX; ++k) parts[w][lane + k * ME_WAVE] = acc[k];
-      if (lane == 0) parts[w][AG_MAX_D] = m, parts[w][AG_MAX_D + 1] = l;
-    }
-    __syncthreads();
-    if (w == 0)
-      for (int o = 0; o < wpu && round * wpu + o < n_chunks; ++o) {
-        float accc[KMAX];
-#pragma unroll
-        for (int k = 0; k < KMAX; ++k) accc[k] = parts[o][lane + k * ME_WAVE];
-        ag_merge<KMAX>(mt, lt, acct, parts[o][AG_MAX_D], parts[o][AG_MAX_D + 1], accc);
-      }
-    __syncthreads();
-  }
   }
   if (w != 0) return;
   T* orow = out + ((size_t)t * nh + head) * d;
