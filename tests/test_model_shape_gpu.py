@@ -1,8 +1,9 @@
 """The layer sizes of the benchmark's model (hidden 1024, 16 query and 8 kv heads of 128, feed-forward
 3072) with two layers and a small vocabulary, in bfloat16, against the plain implementation: the paths
 that only such sizes reach. A 700-token prompt in one step (the tiled matrix-core GEMM with the SwiGLU
-epilogue, prefill attention with tiles cut and packed into bundles), 24 short prompts in one step, then
-all 25 requests decoding side by side (17 to 64 rows: the small matrix-core GEMM, projections as partial
+epilogue, prefill attention over whole tiles of different lengths), a 130-token prompt in a step of its own (the
+gated product in the weight-streaming kernel, three groups of rows), 24 short prompts in one step, then
+all 26 requests decoding side by side (17 to 64 rows: the weight-streaming products, projections as partial
 sums over runs of k, the fused decode attention with its keys dealt to the splits), eagerly and as a
 replayed graph."""
 
@@ -27,7 +28,7 @@ def model(tmp_path_factory):
                       num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
                       rope_theta=1e6, max_position_embeddings=4096, tie_word_embeddings=True)
     folder = write_tiny(str(tmp_path_factory.mktemp("model_shape")), cfg, seed=5, std=0.03)
-    reqs = {"long": random_prompt(700 + EXTRA, cfg.vocab_size, seed=1)}
+    reqs = {"long": random_prompt(700 + EXTRA, cfg.vocab_size, seed=1), "mid": random_prompt(130 + EXTRA, cfg.vocab_size, seed=2)}
     for i in range(24):
         reqs[f"s{i}"] = random_prompt(20 + (7 * i) % 41 + EXTRA, cfg.vocab_size, seed=10 + i)
     return folder, reqs, th.plain_logits(folder, reqs)
@@ -38,9 +39,10 @@ def steps_for(reqs):
         return {"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
 
     steps = [{"step": 0, "entries": [entry("long", 0, len(reqs["long"]) - EXTRA)], "end": []},
-             {"step": 1, "entries": [entry(r, 0, len(t) - EXTRA) for r, t in reqs.items() if r != "long"], "end": []}]
+             {"step": 1, "entries": [entry("mid", 0, len(reqs["mid"]) - EXTRA)], "end": []},
+             {"step": 2, "entries": [entry(r, 0, len(t) - EXTRA) for r, t in reqs.items() if r not in ("long", "mid")], "end": []}]
     for j in range(EXTRA):
-        steps.append({"step": 2 + j, "entries": [entry(r, len(t) - EXTRA + j, len(t) - EXTRA + j + 1) for r, t in reqs.items()],
+        steps.append({"step": 3 + j, "entries": [entry(r, len(t) - EXTRA + j, len(t) - EXTRA + j + 1) for r, t in reqs.items()],
                       "end": list(reqs) if j == EXTRA - 1 else []})
     return steps
 
