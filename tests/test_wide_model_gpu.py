@@ -1,0 +1,61 @@
+"""One layer as wide as a large model's (hidden 5120, feed-forward 12288, 16 query and 8 kv heads of 128, 2,048 tokens
+in the vocabulary), in bfloat16, against the plain implementation: every projection's weight has 16 MiB and more, which
+sends its products down other paths than the small layers of the other tests take. 40 short prompts in one step (the GEMM
+library), then the requests decode side by side while most of them end: 40 rows (qkv and gate/up in the library, o and
+down as partial sums of the weight-streaming kernel, down in blocks of 128 columns; the head in the library), 10 rows
+(everything in the weight-streaming kernel, the head too), 2 rows and 1 (the add-and-norm as that kernel's prologue)."""
+
+from __future__ import annotations
+
+import pytest
+
+import trace_helpers as th
+from conftest import random_prompt, write_tiny
+
+pytestmark = pytest.mark.gpu
+
+LIVE = [40, 40, 10, 10, 2, 2, 1]  # requests that decode in each step after the prompts
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    from mini_engine_amd.models.qwen3 import Qwen3Config
+
+    cfg = Qwen3Config(vocab_size=2048, hidden_size=5120, intermediate_size=12288, num_hidden_layers=1,
+                      num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+                      rope_theta=1e6, max_position_embeddings=4096, tie_word_embeddings=True)
+    folder = write_tiny(str(tmp_path_factory.mktemp("wide_model")), cfg, seed=7, std=0.02)
+    reqs = {f"r{i:02d}": random_prompt(5 + (3 * i) % 8 + sum(1 for n in LIVE if n > i), cfg.vocab_size, seed=40 + i) for i in range(40)}
+    return folder, reqs, th.plain_logits(folder, reqs)
+
+
+def steps_for(reqs):
+    def entry(rid, lo, hi):
+        return {"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
+
+    fed = {rid: len(t) - sum(1 for n in LIVE if n > i) for i, (rid, t) in enumerate(reqs.items())}
+    steps = [{"step": 0, "entries": [entry(rid, 0, fed[rid]) for rid in reqs], "end": []}]
+    for j, n in enumerate(LIVE):
+        live = list(reqs)[:n]
+        entries = [entry(rid, fed[rid], fed[rid] + 1) for rid in live]
+        for rid in live:
+            fed[rid] += 1
+        steps.append({"step": 1 + j, "entries": entries, "end": [rid for rid in live if fed[rid] == len(reqs[rid])]})
+    assert all(fed[rid] == len(reqs[rid]) for rid in reqs)
+    return steps
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_wide_layers_against_plain(model, graphs):
+    from mini_engine_amd.engine.trace import TraceSession, build_session
+    from mini_engine_amd.ops import kernels as K
+
+    folder, reqs, want = model
+    # the paths this test is for: weights that count as bound by their streaming, and the arrangement with two tiles a wave
+    assert 2 * 12288 * 5120 >= K.STREAM_MIN_ELEMENTS and 2048 * 5120 >= K.STREAM_MIN_ELEMENTS
+    steps = steps_for(reqs)
+    session = TraceSession(build_session(folder, "bfloat16", 64 * 40, block_size=16, max_live=40, cuda_graphs=graphs))
+    got = th.collect(steps, th.replay_in_process(session, steps))
+    for rid in reqs:
+        th.assert_logits_close(got[rid], want[rid], "bfloat16", f"graphs={graphs} request {rid}")
+    assert (session.engine.runner.graph_replays > 0) == graphs
