@@ -45,17 +45,29 @@ def steps_for(reqs):
     return steps
 
 
-@pytest.mark.parametrize("graphs", [True, False])
-def test_wide_layers_against_plain(model, graphs):
+@pytest.mark.parametrize("path", ["replayed", "eager", "per kernel"])
+def test_wide_layers_against_plain(model, path):
+    """The native step program, replayed and eager, and the per-kernel path of models with parts of their own, whose
+    choice of kernel per product (``ops/kernels.py::linear``) mirrors the native one."""
+    from types import SimpleNamespace
+
+    from mini_engine_amd.engine.runner import ModelRunner
     from mini_engine_amd.engine.trace import TraceSession, build_session
     from mini_engine_amd.ops import kernels as K
 
     folder, reqs, want = model
-    # the paths this test is for: weights that count as bound by their streaming, and the arrangement with two tiles a wave
+    # the paths this test is for: weights that count as bound by their streaming
     assert 2 * 12288 * 5120 >= K.STREAM_MIN_ELEMENTS and 2048 * 5120 >= K.STREAM_MIN_ELEMENTS
     steps = steps_for(reqs)
-    session = TraceSession(build_session(folder, "bfloat16", 64 * 40, block_size=16, max_live=40, cuda_graphs=graphs))
+    engine = build_session(folder, "bfloat16", 64 * 40, block_size=16, max_live=40, cuda_graphs=path == "replayed")
+    if path == "per kernel":
+        runner = ModelRunner(engine.model, engine.config, native=False)
+        assert runner.program is None
+        engine = SimpleNamespace(runner=runner, core=runner.core, block_manager=runner.new_block_manager())
+    else:
+        assert engine.runner.program is not None
+    session = TraceSession(engine)
     got = th.collect(steps, th.replay_in_process(session, steps))
     for rid in reqs:
-        th.assert_logits_close(got[rid], want[rid], "bfloat16", f"graphs={graphs} request {rid}")
-    assert (session.engine.runner.graph_replays > 0) == graphs
+        th.assert_logits_close(got[rid], want[rid], "bfloat16", f"{path}: request {rid}")
+    assert (engine.runner.graph_replays > 0) == (path == "replayed")
