@@ -47,17 +47,26 @@ def steps_for(reqs):
     return steps
 
 
-@pytest.mark.parametrize("graphs", [True, False])
-def test_benchmark_layer_sizes_against_plain(model, graphs):
+@pytest.mark.parametrize("path", ["replayed", "eager", "per kernel"])
+def test_benchmark_layer_sizes_against_plain(model, path):
+    """The native step program, replayed and eager, and the per-kernel path that models with parts of their own take."""
+    from types import SimpleNamespace
+
+    from mini_engine_amd.engine.runner import ModelRunner
     from mini_engine_amd.engine.trace import TraceSession, build_session
 
     folder, reqs, want = model
     steps = steps_for(reqs)
-    session = TraceSession(build_session(folder, "bfloat16", 4096, block_size=16, max_live=32, cuda_graphs=graphs))
+    engine = build_session(folder, "bfloat16", 4096, block_size=16, max_live=32, cuda_graphs=path == "replayed")
+    if path == "per kernel":
+        runner = ModelRunner(engine.model, engine.config, native=False)
+        assert runner.program is None
+        engine = SimpleNamespace(runner=runner, core=runner.core, block_manager=runner.new_block_manager())
+    session = TraceSession(engine)
     got = th.collect(steps, th.replay_in_process(session, steps))
     for rid in reqs:
-        th.assert_logits_close(got[rid], want[rid], "bfloat16", f"graphs={graphs} request {rid}")
-    assert (session.engine.runner.graph_replays > 0) == graphs
+        th.assert_logits_close(got[rid], want[rid], "bfloat16", f"{path}: request {rid}")
+    assert (engine.runner.graph_replays > 0) == (path == "replayed")
     assert all(len(p.free_pool) == p.num_blocks for p in session.bm.pools)
 
 
