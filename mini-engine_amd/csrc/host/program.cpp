@@ -19,6 +19,7 @@ constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
 constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
 constexpr int kNormStreamRows = 2;   // up to here the add-and-norm is the prologue of the weight-streaming kernel
 constexpr int kTiledMinRows = 256;
+constexpr int kStreamWholeRows = 32;   // up to here the weight-streaming kernel serves wide products whose blocks fill whole rounds
 constexpr int kStreamGroupRows = 256;  // what the weight-streaming kernel accepts, in groups of 64 rows
 constexpr int kTiledMaxK = 3072;  // gate/up with the SwiGLU as the tiled kernel's epilogue against the library's product and a
                                   // SwiGLU kernel: at k = 1,024 (3,072 columns) 15-62 us against 21-67 for 512 to 4,096 rows; at
@@ -84,6 +85,24 @@ bool weight_bound(int m, int rows_of_w, int k) {
 // What the weight-streaming kernel takes at all.
 bool streams(int m, int rows_of_w, int k) {
   return m <= kSmallMaxRows && k % 8 == 0 && (int64_t)rows_of_w * k * 2 < kStreamMaxBytes;
+}
+
+int compute_units();
+
+// Whether the weight-streaming kernel serves a wide product of 17 to 32 rows instead of the library: where its blocks fill
+// whole rounds of the compute units (at least 15/16 of them) and the rows of the weight are a multiple of 4 KiB apart, which
+// costs the library's kernels a quarter of their rate (2 x 12,288 x 4,096 with SwiGLU: 52 us, with k = 4,224 42; the streaming
+// kernel 46 and 39). Measured at 17 and 32 rows: 2 x 12,288 x 4,096 46 us against 52; 6,144 x 4,096 14.1 and 15.6 against
+// 16.3 and 15.9; 2 x 28,672 x 8,192 182 against 191 and 194; a decode step of the 8B shape at batch 20 to 32 4-5% shorter.
+// Where the blocks do not fill their rounds the library is ahead (10,240 x 5,120 on 160 blocks: 32 and 35 against 27 and 30;
+// 5,120 x 4,096: 13.4 against 12.0), with other k it is ahead or level (2 x 25,600 x 5,120: 101 and 105 against 99 and 102),
+// and from 33 rows on it is ahead on as many shapes as not.
+bool stream_serves_mid_rows(int m, int n, int k, bool gated) {
+  if (k % 2048) return false;
+  int plan[3] = {0, 0, 0};
+  me_gemm_bf16_stream_plan(m, n, k, gated ? 1 : 0, 1, compute_units(), plan);
+  const long long cus = compute_units(), rounds = (plan[2] + cus - 1) / cus;
+  return (long long)plan[2] * 16 >= rounds * cus * 15;
 }
 
 int compute_units() {
@@ -291,6 +310,10 @@ class Run {
     }
     const bool heavy = weight_bound(m, rows_of_w, k);
     if (heavy && m <= kSmallFastRows && (out_dtype == kBF16 || !gated)) {  // up to 16 rows it is ahead of the library too
+      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
+      return;
+    }
+    if (heavy && m <= kStreamWholeRows && (out_dtype == kBF16 || !gated) && stream_serves_mid_rows(m, n, k, gated != 0)) {
       ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
       return;
     }

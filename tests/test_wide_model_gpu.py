@@ -1,9 +1,11 @@
-"""One layer as wide as a large model's (hidden 5120, feed-forward 12288, 16 query and 8 kv heads of 128, 2,048 tokens
-in the vocabulary), in bfloat16, against the plain implementation: every projection's weight has 16 MiB and more, which
-sends its products down other paths than the small layers of the other tests take. 40 short prompts in one step (the GEMM
-library), then the requests decode side by side while most of them end: 40 rows (qkv and gate/up in the library, o and
-down as partial sums of the weight-streaming kernel, down in blocks of 128 columns; the head in the library), 10 rows
-(everything in the weight-streaming kernel, the head too), 2 rows and 1 (the add-and-norm as that kernel's prologue)."""
+"""One layer as wide as a large model's (hidden 5120 with 16 query heads, or hidden 4096 with 32; feed-forward 12288, 8 kv
+heads of 128, 2,048 tokens in the vocabulary), in bfloat16, against the plain implementation: every projection's weight
+has 16 MiB and more, which sends its products down other paths than the small layers of the other tests take. 40 short
+prompts in one step (the GEMM library), then the requests decode side by side while most of them end: 40 rows (qkv and
+gate/up in the library, o and down as partial sums of the weight-streaming kernel, down in blocks of 128 columns at hidden
+5120; the head in the library), 24 rows (at hidden 4096, whose weights' rows lie a multiple of 4 KiB apart and whose
+products fill whole rounds of blocks, qkv and gate/up in the weight-streaming kernel too), 10 rows (everything in that
+kernel, the head too), 2 rows and 1 (the add-and-norm as that kernel's prologue)."""
 
 from __future__ import annotations
 
@@ -14,19 +16,20 @@ from conftest import random_prompt, write_tiny
 
 pytestmark = pytest.mark.gpu
 
-LIVE = [40, 40, 10, 10, 2, 2, 1]  # requests that decode in each step after the prompts
+LIVE = [40, 40, 24, 24, 10, 10, 2, 2, 1]  # requests that decode in each step after the prompts
 
 
-@pytest.fixture(scope="module")
-def model(tmp_path_factory):
+@pytest.fixture(scope="module", params=[(5120, 16), (4096, 32)], ids=["hidden5120", "hidden4096"])
+def model(request, tmp_path_factory):
     from mini_engine_amd.models.qwen3 import Qwen3Config
 
-    cfg = Qwen3Config(vocab_size=2048, hidden_size=5120, intermediate_size=12288, num_hidden_layers=1,
-                      num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+    hidden, heads = request.param
+    cfg = Qwen3Config(vocab_size=2048, hidden_size=hidden, intermediate_size=12288, num_hidden_layers=1,
+                      num_attention_heads=heads, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
                       rope_theta=1e6, max_position_embeddings=4096, tie_word_embeddings=True)
     folder = write_tiny(str(tmp_path_factory.mktemp("wide_model")), cfg, seed=7, std=0.02)
     reqs = {f"r{i:02d}": random_prompt(5 + (3 * i) % 8 + sum(1 for n in LIVE if n > i), cfg.vocab_size, seed=40 + i) for i in range(40)}
-    return folder, reqs, th.plain_logits(folder, reqs)
+    return folder, reqs, th.plain_logits(folder, reqs), hidden
 
 
 def steps_for(reqs):
@@ -55,9 +58,12 @@ def test_wide_layers_against_plain(model, path):
     from mini_engine_amd.engine.trace import TraceSession, build_session
     from mini_engine_amd.ops import kernels as K
 
-    folder, reqs, want = model
-    # the paths this test is for: weights that count as bound by their streaming
-    assert 2 * 12288 * 5120 >= K.STREAM_MIN_ELEMENTS and 2048 * 5120 >= K.STREAM_MIN_ELEMENTS
+    folder, reqs, want, hidden = model
+    # the paths this test is for: weights that count as bound by their streaming; at hidden 4096 the products of 24 rows that
+    # the weight-streaming kernel takes from the library
+    assert 2 * 12288 * hidden >= K.STREAM_MIN_ELEMENTS and 2048 * hidden >= K.STREAM_MIN_ELEMENTS
+    assert K.stream_serves_mid_rows(24, 12288, hidden, True) == (hidden == 4096)
+    assert K.stream_serves_mid_rows(24, 6144, 4096, False) and not K.stream_serves_mid_rows(24, 5120, 4096, False)
     steps = steps_for(reqs)
     engine = build_session(folder, "bfloat16", 64 * 40, block_size=16, max_live=40, cuda_graphs=path == "replayed")
     if path == "per kernel":
