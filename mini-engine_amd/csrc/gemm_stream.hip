@@ -36,7 +36,8 @@ constexpr int kRow = kStepK + 16;    // LDS row stride in elements: 288 bytes, 3
 
 template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int NT = 1>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                          OutT* __restrict__ C, int rows, int N, int K, int steps_per_split, int gate) {
+                                                          OutT* __restrict__ C, int rows, int N, int K, int steps_per_split, int gate,
+                                                          int rotate) {
   static_assert(WN * WK == 4, "four waves per block");
   static_assert(NT == 1 || WK == 1, "waves with several tiles of columns do not cut k");
   // The grid's third dimension deals the rows out in groups of 16 MT; a block sees its group's rows only.
@@ -93,8 +94,13 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   // number of steps ahead: loads complete in the order of their issue, so a step that waited for rows of x
   // fetched later than its weights would wait for every weight in flight.
   suint4_t w[STAGES][ACCS][CH], xreg[STAGES][XV];
+  // With `rotate` a block walks its steps of k from a step of its own on, around the end of its run: the blocks that start
+  // together then read different memory channels (rows of W that lie a multiple of 4 KiB apart begin in the same one).
+  const int rot = rotate ? (int)((blockIdx.x * 5u + blockIdx.z) % (unsigned)max(steps, 1)) : 0;
   auto load_step = [&](int step, suint4_t (&wd)[ACCS][CH], suint4_t (&xd)[XV]) {
-    const int k0 = (first + step) * kStepK;
+    int turned = step + rot;
+    if (turned >= steps) turned -= steps;
+    const int k0 = (first + (step < steps ? turned : steps)) * kStepK;  // (steps past the run: beyond its end, nothing is fetched)
 #pragma unroll
     for (int i = 0; i < XV; ++i)
       xd[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, k0 + x_k[i] < k_end ? (int)(x_base[i] + k0 * 2) : (int)x_bytes, 0, 0);
@@ -452,18 +458,24 @@ void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C,
                      int gate, hipStream_t stream) {
   const dim3 grid(plan.grid, plan.splits, (M + kGroupRows - 1) / kGroupRows);
   const int wn = plan.wn;
+  // Rows of W that lie a multiple of 4 KiB apart begin in the same memory channel: blocks that all start at k = 0 then
+  // queue for a few channels (2 x 12,288 x 4,096 with SwiGLU at 32 rows: 46.7 us; with k = 4,224 38.8). Each block starts its
+  // walk over k at a step of its own instead (39.4 us; at 1 and 8 rows 42.7 -> 40.5 and 43.1 -> 41.0; 6,144 x 4,096 at 32
+  // rows 15.5 -> 14.3). Runs of k across blocks start at different k already, and other strides spread by themselves
+  // (k = 5,120: no change either way), so those keep the plain walk.
+  const int rotate = plan.splits == 1 && K % 2048 == 0;
   if constexpr (MT >= 3 && !SWIGLU && sizeof(OutT) == 4) {
     if (plan.nt == 2) {  // (two steps in flight: 3-15% ahead of three)
-      gemm_stream_kernel<MT, 4, 1, false, OutT, 2, 2><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
+      gemm_stream_kernel<MT, 4, 1, false, OutT, 2, 2><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
       return;
     }
   }
   if (wn == 4)
-    gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
+    gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
   else if (wn == 2)
-    gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
+    gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
   else
-    gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate);
+    gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
 }
 
 template <bool SWIGLU, typename OutT>

@@ -19,7 +19,8 @@ constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
 constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
 constexpr int kNormStreamRows = 2;   // up to here the add-and-norm is the prologue of the weight-streaming kernel
 constexpr int kTiledMinRows = 256;
-constexpr int kStreamWholeRows = 32;   // up to here the weight-streaming kernel serves wide products whose blocks fill whole rounds
+constexpr int kStreamWholeRows = 32;   // up to here the weight-streaming kernel serves wide plain products whose blocks fill whole
+                                       // rounds (gated ones up to 64)
 constexpr int kStreamGroupRows = 256;  // what the weight-streaming kernel accepts, in groups of 64 rows
 constexpr int kTiledMaxK = 3072;  // gate/up with the SwiGLU as the tiled kernel's epilogue against the library's product and a
                                   // SwiGLU kernel: at k = 1,024 (3,072 columns) 15-62 us against 21-67 for 512 to 4,096 rows; at
@@ -97,8 +98,11 @@ int compute_units();
 // Where the blocks do not fill their rounds the library is ahead (10,240 x 5,120 on 160 blocks: 32 and 35 against 27 and 30;
 // 5,120 x 4,096: 13.4 against 12.0), with other k it is ahead or level (2 x 25,600 x 5,120: 101 and 105 against 99 and 102),
 // and from 33 rows on it is ahead on as many shapes as not.
+// With each block's walk over k starting at a step of its own (what the kernel does for such k) the gated products stay ahead
+// up to 64 rows: 2 x 12,288 x 4,096 38-43 us against 48-50 at 17 to 64 rows, 2 x 14,336 x 4,096 45-48 against 58-65, 2 x 28,672
+// x 8,192 169-180 against 192-216; the plain 6,144 x 4,096 up to 32 (14.3 and 15.1 against 15.1 and 15.4; 19.4 against 17.6 at 64).
 bool stream_serves_mid_rows(int m, int n, int k, bool gated) {
-  if (k % 2048) return false;
+  if (k % 2048 || m > (gated ? kSmallMaxRows : kStreamWholeRows)) return false;
   int plan[3] = {0, 0, 0};
   me_gemm_bf16_stream_plan(m, n, k, gated ? 1 : 0, 1, compute_units(), plan);
   const long long cus = compute_units(), rounds = (plan[2] + cus - 1) / cus;
@@ -313,7 +317,7 @@ class Run {
       ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
       return;
     }
-    if (heavy && m <= kStreamWholeRows && (out_dtype == kBF16 || !gated) && stream_serves_mid_rows(m, n, k, gated != 0)) {
+    if (heavy && (out_dtype == kBF16 || !gated) && stream_serves_mid_rows(m, n, k, gated != 0)) {
       ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
       return;
     }

@@ -417,14 +417,14 @@ def stream_plan(rows: int, n: int, k: int, gated: bool = False, k_splits: int = 
     return int(out[0]), int(out[1]), int(out[2])
 
 
-STREAM_WHOLE_ROWS = 32  # up to here the weight-streaming kernel serves wide products whose blocks fill whole rounds
+STREAM_WHOLE_ROWS = 32  # up to here the weight-streaming kernel serves wide plain products whose blocks fill whole rounds (gated: 64)
 
 
 def stream_serves_mid_rows(rows: int, n: int, k: int, gated: bool, device=None) -> bool:
-    """Whether the weight-streaming kernel serves a wide product of 17 to 32 rows instead of the GEMM library: its blocks
+    """Whether the weight-streaming kernel serves a wide product of 17 to 32 rows (64 for a gated one) instead of the GEMM library: its blocks
     fill whole rounds of the compute units (15/16 of them at least) and the weight's rows are a multiple of 4 KiB apart
     (the measurements are in ``csrc/host/program.cpp``)."""
-    if k % 2048:
+    if k % 2048 or rows > (SMALL_MAX_ROWS if gated else STREAM_WHOLE_ROWS):
         return False
     units = compute_units(device)
     grid = stream_plan(rows, n, k, gated, 1, units=units)[2]
@@ -656,7 +656,7 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated:
         return PartialSums(gemm_bf16_library(x, weight, torch.float32).unsqueeze(0))
     if (heavy if few else streams(x, weight) and not heavy) and (out_dtype is torch.bfloat16 or not gated):
         return gemm_bf16_stream(x, weight, out_dtype, gated)
-    if (heavy and x.shape[0] <= STREAM_WHOLE_ROWS and (out_dtype is torch.bfloat16 or not gated)
+    if (heavy and (out_dtype is torch.bfloat16 or not gated)
             and stream_serves_mid_rows(x.shape[0], weight.shape[0] // (2 if gated else 1), x.shape[1], bool(gated), x.device)):
         return gemm_bf16_stream(x, weight, out_dtype, gated)  # 17 to 32 rows of a wide product (see stream_serves_mid_rows)
     if heavy and x.shape[0] <= HEAD_STREAM_ROWS and out_dtype is torch.float32 and not gated:  # a head's logits
