@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
                                                                const float* __restrict__ parts, int num_parts, size_t part_stride,
                                                                const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
                                                                const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N,
-                                                               int K, int gate) {
+                                                               int K, int gate, int rotate) {
   static_assert(WN * WK == 4, "four waves per block");
   constexpr int KC = kStepK / WK, CH = KC / 32, ACCS = SWIGLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char norm_lds[];
@@ -243,8 +243,11 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
 #pragma unroll
   for (int a = 0; a < ACCS; ++a) w_base[a] = n < c1 ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
   suint4_t w[STAGES][ACCS][CH];
+  // (with `rotate` the block's walk over k starts at a step of its own and goes around the end, as in the kernel above)
+  const int rot = rotate ? (int)((blockIdx.x * 5u) % (unsigned)steps) : 0;
+  auto turned = [&](int step) { return step + rot < steps ? step + rot : step + rot - steps; };
   auto load_step = [&](int step, suint4_t (&wd)[ACCS][CH]) {
-    const int k0 = step * kStepK;
+    const int k0 = (step < steps ? turned(step) : steps) * kStepK;  // (steps past the end: beyond K, nothing is fetched)
 #pragma unroll
     for (int a = 0; a < ACCS; ++a)
 #pragma unroll
@@ -311,7 +314,7 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
   for (int s0 = 0; s0 < steps; s0 += STAGES) {  // the last round may run up to STAGES - 1 steps of zero weights
 #pragma unroll
     for (int u = 0; u < STAGES; ++u) {
-      const int k0 = min(s0 + u, steps - 1) * kStepK;  // (steps past the end multiply zeros with the last step's rows)
+      const int k0 = turned(min(s0 + u, steps - 1)) * kStepK;  // (steps past the end multiply zero weights with some step's rows)
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         sbf16x8_t b = sbf16x8_t{};
@@ -551,7 +554,8 @@ int launch_norm(StreamPlan plan, const float* x_in, const bf16_t* delta, const f
   if (lds > 48 * 1024) return me_fail("me_gemm_bf16_stream_norm: %d rows of %d do not fit the block's memory", M, K);
 #define ME_NORM_LAUNCH(WN, WK, STAGES)                                                                                   \
   gemm_stream_norm_kernel<WN, WK, SWIGLU, OutT, STAGES><<<grid, 256, lds, stream>>>(x_in, delta, parts, num_parts, part_stride, \
-                                                                                    w_norm, eps, x_out, W, C, M, N, K, gate)
+                                                                                    w_norm, eps, x_out, W, C, M, N, K, gate, \
+                                                                                    K % 2048 == 0)
   if (wn == 4)
     ME_NORM_LAUNCH(4, 1, (SWIGLU ? 2 : 3));
   else if (wn == 2)
