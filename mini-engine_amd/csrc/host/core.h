@@ -119,6 +119,7 @@ struct Request {
   // stand-in for that draw, which a step planned ahead feeds from row `fed_row` of the draws on the device.
   bool pending = false;
   int fed_row = -1;
+  mutable uint64_t seen_in_check = 0;  // the last check of a step that met this request (finds one named twice)
 
   int size() const { return (int)tokens.size(); }
   int uncomputed() const { return size() - num_computed; }
@@ -234,6 +235,7 @@ class Core {
   std::deque<Request*> waiting_;
   std::vector<Request*> running_;
   std::vector<StepItem> step_;
+  mutable uint64_t check_stamp_ = 0;
   std::vector<StepItem> in_flight_;  // the step launched before step_ whose draws are not settled yet
   void reap(Request* r);
   void finish(Request* r, std::vector<int64_t>& finished);

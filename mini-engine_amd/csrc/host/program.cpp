@@ -9,29 +9,16 @@
 #include <tuple>
 
 #include "../kernels.h"
+#include "choice.h"
+
+int me_fail(const char* fmt, ...);
 
 namespace me {
 
 namespace {
 
 constexpr int kF32 = 0, kBF16 = 1;
-constexpr int kSmallMaxRows = 64;   // what the small matrix-core kernel accepts
-constexpr int kSmallFastRows = 16;  // up to here it beats the GEMM library on every shape, the norm as its prologue too
-constexpr int kNormStreamRows = 2;   // up to here the add-and-norm is the prologue of the weight-streaming kernel
-constexpr int kTiledMinRows = 256;
-constexpr int kStreamWholeRows = 32;   // up to here the weight-streaming kernel serves wide plain products whose blocks fill whole
-                                       // rounds (gated ones up to 64)
-constexpr int kStreamGroupRows = 256;  // what the weight-streaming kernel accepts, in groups of 64 rows
-constexpr int kTiledMaxK = 3072;  // gate/up with the SwiGLU as the tiled kernel's epilogue against the library's product and a
-                                  // SwiGLU kernel: at k = 1,024 (3,072 columns) 15-62 us against 21-67 for 512 to 4,096 rows; at
-                                  // k = 4,096 (12,288 columns) 95-729 against 89-640; at k = 5,120 (25,600) 345-1,973 against
-                                  // 293-1,767: the longer k is, the less a pass over the output weighs against the product
-constexpr int kHeadStreamRows = 32;  // the head's logits (float32) come from the weight-streaming kernel up to here: at 151,936
-                                     // rows of 1,024 / 4,096 / 5,120 it takes 62-75 / 245-272 / 291-341 us at 8 to 32 rows,
-                                     // the library 62-79 / 260-276 / 319-362; from 48 rows on the library is ahead
 constexpr int kDecodeWaves = 1024;  // waves that a decode attention launch aims at (four per compute unit of 256)
-constexpr int64_t kStreamMinElements = 8ll << 20;  // weights from 16 MiB on: streaming them is the product's time
-constexpr int64_t kStreamMaxBytes = 1ll << 31;     // what the weight-streaming kernel addresses
 
 void ok(int code) {
   if (code) throw Error(kBadState, me_last_error());
@@ -57,57 +44,6 @@ struct Pending {
   long long stride = 0;
   bool any() const { return delta || parts; }
 };
-
-// Which kernel serves a bfloat16 product of m rows (measured on the layer sizes of a 0.6B, an 8B and a 32B model):
-//   up to 16 rows, weights below 16 MiB: the small matrix-core kernel; the residual add and the norm are its prologue
-//     where the delta in front is a tensor (a product whose k was not cut);
-//   17 to 64 rows, weights below 16 MiB: the weight-streaming kernel (qkv 5.0-6.7 us, gate/up with SwiGLU 6.6-9.3
-//     against 5.8-7.7 and 7.5-10.3 with the small kernel, 8.2-8.6 and 14.4-14.7 with the library and a SwiGLU kernel);
-//   a delta of the residual stream, at any row count up to 64: the weight-streaming kernel with k cut into runs, so
-//     that every compute unit streams a part of the weight (1,024 columns, 1 to 16 rows: 3.5 and 4.3 us against 4.7-6.1
-//     and 5.8-7.8 with the small kernel; 17 to 64 rows: 3.9-5.3 against 7.9-16 and 7.6-9.8). The add-and-norm behind
-//     it, a kernel of its own (2.9 us), adds the partial sums up; as the prologue of the next product, where every
-//     block would read them, they cost more at every row count (one row: 853 -> 820 tokens/s);
-//   everything else: the GEMM library, as the reference hands every projection to one.
-bool small_serves(int m, int k) { return k % 8 == 0 && m <= kSmallFastRows; }
-
-// Whether a product of up to 64 rows is bound by streaming its weight: the layers of wide models. Their
-// deltas go to the weight-streaming kernel with k cut into runs (measured at 4,096 and 5,120 columns, k of 4,096
-// to 25,600: 8.7-29 us and 21-80 us against 9.4-65 and 27-245 with the small kernel, 10-38 and 20-156 with
-// the library); their other products go to the same kernel up to 16 rows (qkv and gate/up 14.7-43 and 24-117 us
-// against 15-51 and 26-139 with the small kernel) and to the library from 17 to 64 rows (qkv 15-33 us against
-// 21-56 with the streaming kernel, whose time grows with the rows). The norm before such a product is a kernel
-// of its own: the partial sums it adds up are read once, not by every block of a product.
-bool weight_bound(int m, int rows_of_w, int k) {
-  const int64_t elements = (int64_t)rows_of_w * k;
-  return m <= kSmallMaxRows && k % 8 == 0 && elements >= kStreamMinElements && elements * 2 < kStreamMaxBytes;
-}
-
-// What the weight-streaming kernel takes at all.
-bool streams(int m, int rows_of_w, int k) {
-  return m <= kSmallMaxRows && k % 8 == 0 && (int64_t)rows_of_w * k * 2 < kStreamMaxBytes;
-}
-
-int compute_units();
-
-// Whether the weight-streaming kernel serves a wide product of 17 to 32 rows instead of the library: where its blocks fill
-// whole rounds of the compute units (at least 15/16 of them) and the rows of the weight are a multiple of 4 KiB apart, which
-// costs the library's kernels a quarter of their rate (2 x 12,288 x 4,096 with SwiGLU: 52 us, with k = 4,224 42; the streaming
-// kernel 46 and 39). Measured at 17 and 32 rows: 2 x 12,288 x 4,096 46 us against 52; 6,144 x 4,096 14.1 and 15.6 against
-// 16.3 and 15.9; 2 x 28,672 x 8,192 182 against 191 and 194; a decode step of the 8B shape at batch 20 to 32 4-5% shorter.
-// Where the blocks do not fill their rounds the library is ahead (10,240 x 5,120 on 160 blocks: 32 and 35 against 27 and 30;
-// 5,120 x 4,096: 13.4 against 12.0), with other k it is ahead or level (2 x 25,600 x 5,120: 101 and 105 against 99 and 102),
-// and from 33 rows on it is ahead on as many shapes as not.
-// With each block's walk over k starting at a step of its own (what the kernel does for such k) the gated products stay ahead
-// up to 64 rows: 2 x 12,288 x 4,096 38-43 us against 48-50 at 17 to 64 rows, 2 x 14,336 x 4,096 45-48 against 58-65, 2 x 28,672
-// x 8,192 169-180 against 192-216; the plain 6,144 x 4,096 up to 32 (14.3 and 15.1 against 15.1 and 15.4; 19.4 against 17.6 at 64).
-bool stream_serves_mid_rows(int m, int n, int k, bool gated) {
-  if (k % 2048 || m > (gated ? kSmallMaxRows : kStreamWholeRows)) return false;
-  int plan[3] = {0, 0, 0};
-  me_gemm_bf16_stream_plan(m, n, k, gated ? 1 : 0, 1, compute_units(), plan);
-  const long long cus = compute_units(), rounds = (plan[2] + cus - 1) / cus;
-  return (long long)plan[2] * 16 >= rounds * cus * 15;
-}
 
 int compute_units() {
   static int units = 0;
@@ -271,82 +207,62 @@ class Run {
     const int gated = (int)op.i[2];  // 0, or the code of the gate's activation
     if (k != h_) throw Error(kBadValue, "a product behind a norm reads the hidden size");
     const int n = gated ? rows_of_w / 2 : rows_of_w;
-    // Decode-sized steps: the residual add and the norm are the product's prologue; the sum goes to the second
-    // residual buffer, since other blocks of the kernel still read the first.
-    // A row or two: the weight-streaming kernel adds and norms the rows itself while its first weights are on their
-    // way, whatever the delta is (one row: 857 -> 967 tokens/s, two: 1,605 -> 1,700; from four rows on every block's
-    // reads of the partial sums cost more than the launch they save: 2,749 -> 2,668).
-    if (dtype_ == kBF16 && t_ <= kNormStreamRows && me_gemm_bf16_stream_norm_fits(t_, k) && streams(t_, rows_of_w, k)) {
-      const bool adds = pending_.any();
-      ok(me_gemm_bf16_stream_norm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w_norm, op.f[0],
-                                  adds ? spare_ : nullptr, op.p[1], bufs_[op.out], t_, n, k, gated, dtype_, compute_units(), stream_));
-      if (adds) std::swap(x_, spare_);
-      pending_ = Pending();
-      release_parts();
-      return;
+    const int pending = pending_.parts ? kPendingParts : pending_.delta ? kPendingTensor : kPendingNone;
+    // Where the add and the norm ride on the product the sum goes to the second residual buffer, since other blocks
+    // of the kernel still read the first.
+    switch (choose_norm_fusion(dtype_, t_, rows_of_w, k, pending, compute_units(), true)) {
+      case kNormInStream: {
+        const bool adds = pending_.any();
+        ok(me_gemm_bf16_stream_norm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w_norm, op.f[0],
+                                    adds ? spare_ : nullptr, op.p[1], bufs_[op.out], t_, n, k, gated, dtype_, compute_units(),
+                                    stream_));
+        if (adds) std::swap(x_, spare_);
+        pending_ = Pending();
+        release_parts();
+        return;
+      }
+      case kNormInSmall:
+        ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
+                              bufs_[op.out], t_, n, k, 1, gated, dtype_, 1, stream_));
+        if (pending_.delta) std::swap(x_, spare_);
+        pending_ = Pending();
+        return;
+      default:
+        add_norm(w_norm, op.f[0], normed_);
+        product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
     }
-    // Up to 16 rows with nothing, or a tensor, to add (the first layer's norm; parts of other kinds): the small kernel's
-    // prologue.
-    if (dtype_ == kBF16 && t_ <= kSmallFastRows && k % 8 == 0 && !pending_.parts && !weight_bound(t_, rows_of_w, k)) {
-      ok(me_gemm_bf16_small(nullptr, x_, pending_.delta, w_norm, op.f[0], pending_.delta ? spare_ : nullptr, op.p[1],
-                            bufs_[op.out], t_, n, k, 1, gated, dtype_, 1, stream_));
-      if (pending_.delta) std::swap(x_, spare_);
-      pending_ = Pending();
-      return;
-    }
-    add_norm(w_norm, op.f[0], normed_);
-    product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
   }
 
-  // out = x . W^T (gated, the code of an activation: act(gate) * up with W = [gate rows; up rows]).
-  void product(const void* x, const void* w, int rows_of_w, int k, int gated, int out_dtype, void* out) {
-    const int m = t_rows_;
+  // out = x . W^T (gated, the code of an activation: act(gate) * up with W = [gate rows; up rows]), by the kernel
+  // that choose_product names.
+  void product(const void* x, const void* w, int rows_of_w, int k, int gated, int out_dtype, void* out, int role = kRolePlain,
+               int rows = -1) {
+    const int m = rows < 0 ? t_ : rows;
     const int n = gated ? rows_of_w / 2 : rows_of_w;
-    if (dtype_ == kF32) {  // a true 32-bit product, additions in ascending k whatever the rows
-      if (!gated) {
-        ok(me_gemm_f32((const float*)x, (const float*)w, (float*)out, m, n, k, stream_));
-        return;
-      }
-      float* both = (float*)arena_.take((size_t)m * rows_of_w * 4);
-      ok(me_gemm_f32((const float*)x, (const float*)w, both, m, rows_of_w, k, stream_));
-      ok(me_swiglu(both, out, m, n, gated, kF32, stream_));
-      return;
+    const ProductChoice c = choose_product(dtype_, role, m, rows_of_w, k, gated, out_dtype, compute_units(), true);
+    void* dst = out;
+    const int cols = c.gate_after ? rows_of_w : n;
+    const int inner_dtype = c.gate_after ? dtype_ : out_dtype;
+    if (c.gate_after) dst = arena_.take((size_t)m * rows_of_w * elem_);
+    const int epilogue = c.gate_after ? 0 : gated;
+    switch (c.kernel) {
+      case kProductF32:
+        ok(me_gemm_f32((const float*)x, (const float*)w, (float*)dst, m, cols, k, stream_));
+        break;
+      case kProductSmall:
+        ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, dst, m, cols, k, 0, epilogue, inner_dtype, 1, stream_));
+        break;
+      case kProductStream:
+        ok(me_gemm_bf16_stream(x, w, dst, m, cols, k, epilogue, c.partial_sums ? kF32 : inner_dtype, c.runs, compute_units(),
+                               stream_));
+        break;
+      case kProductTiled:
+        ok(me_gemm_bf16_tiled(x, w, dst, m, cols, k, epilogue, inner_dtype, 0, stream_));
+        break;
+      default:
+        library_product(x, w, dst, m, cols, k, c.partial_sums ? kF32 : inner_dtype, stream_);
     }
-    const bool heavy = weight_bound(m, rows_of_w, k);
-    if (heavy && m <= kSmallFastRows && (out_dtype == kBF16 || !gated)) {  // up to 16 rows it is ahead of the library too
-      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
-      return;
-    }
-    if (heavy && (out_dtype == kBF16 || !gated) && stream_serves_mid_rows(m, n, k, gated != 0)) {
-      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
-      return;
-    }
-    if (!heavy && m > kSmallFastRows && streams(m, rows_of_w, k) && (out_dtype == kBF16 || !gated)) {
-      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
-      return;
-    }
-    if (!heavy && small_serves(m, k)) {
-      ok(me_gemm_bf16_small(x, nullptr, nullptr, nullptr, 0.f, nullptr, w, out, m, n, k, 0, gated, out_dtype, 1, stream_));
-      return;
-    }
-    if (gated && m <= kStreamGroupRows && k % 8 == 0 && (int64_t)rows_of_w * k < kStreamMinElements && out_dtype == kBF16) {
-      // 65 to 256 rows of a small gated weight: the weight-streaming kernel, its blocks once per group of 64 rows (2 x 3,072 x
-      // 1,024: 10.7-13.1 us against 15.5-19.1 with the library and a SwiGLU kernel, 16 with the tiled kernel; the plain
-      // products of that size are no faster than the library's: 9.2 against 8.8-9.2, 7.8 against 7.6-8.3)
-      ok(me_gemm_bf16_stream(x, w, out, m, n, k, gated, out_dtype, 1, compute_units(), stream_));
-      return;
-    }
-    if (gated) {
-      if (m >= kTiledMinRows && k % 64 == 0 && k <= kTiledMaxK && out_dtype == kBF16) {  // ahead of the library product + SwiGLU kernel
-        ok(me_gemm_bf16_tiled(x, w, out, m, n, k, gated, out_dtype, 0, stream_));
-        return;
-      }
-      void* both = arena_.take((size_t)m * rows_of_w * 2);
-      library_product(x, w, both, m, rows_of_w, k, kBF16, stream_);
-      ok(me_swiglu(both, out, m, n, gated, kBF16, stream_));
-      return;
-    }
-    library_product(x, w, out, m, n, k, out_dtype, stream_);
+    if (c.gate_after) ok(me_swiglu(dst, out, m, n, gated, dtype_, stream_));
   }
 
   // A product whose result only ever is the pending delta of the residual stream.
@@ -355,31 +271,18 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
-    if (dtype_ == kBF16 && streams(t_, n, k)) {
-      // float32 partial sums over runs of k (one run for short k): the next add-and-norm adds them up, and the delta is
-      // never rounded to bfloat16 on its way into the float32 residual stream
-      const int splits = me_gemm_bf16_stream_splits(t_, n, k, compute_units());
+    const ProductChoice c = choose_product(dtype_, kRoleDelta, t_, n, k, 0, dtype_, compute_units(), true);
+    if (c.partial_sums) {  // float32 sums over runs of k (or one whole sum) that wait for the next add-and-norm
       parts_mark_ = arena_.used;
-      float* parts = (float*)arena_.take((size_t)splits * t_ * n * 4);
-      ok(me_gemm_bf16_stream(x, op.p[1], parts, t_, n, k, 0, kF32, splits, compute_units(), stream_));
+      float* parts = (float*)arena_.take((size_t)c.runs * t_ * n * 4);
+      product(x, op.p[1], n, k, 0, kF32, parts, kRoleDelta);
       pending_.parts = parts;
-      pending_.num_parts = splits;
-      pending_.stride = (long long)t_ * n;
-      return;
-    }
-    if (dtype_ == kBF16) {
-      // more rows: the library's product with a float32 result, which stands as one partial sum: the delta is never
-      // rounded to bfloat16 on its way into the float32 residual stream
-      parts_mark_ = arena_.used;
-      float* sum = (float*)arena_.take((size_t)t_ * n * 4);
-      library_product(x, op.p[1], sum, t_, n, k, kF32, stream_);
-      pending_.parts = sum;
-      pending_.num_parts = 1;
+      pending_.num_parts = c.runs;
       pending_.stride = (long long)t_ * n;
       return;
     }
     const size_t mark = arena_.used;
-    product(x, op.p[1], n, k, 0, dtype_, bufs_[op.out]);
+    product(x, op.p[1], n, k, 0, dtype_, bufs_[op.out], kRoleDelta);
     arena_.used = mark;
     pending_.delta = bufs_[op.out];
   }
@@ -468,14 +371,7 @@ class Run {
                       idx(s_.lay.want_rows), rows, h_, op.f[0], 0, dtype_, stream_));
     pending_ = Pending();
     float* logits = (float*)arena_.take((size_t)rows * vocab * 4);
-    if (dtype_ == kF32)
-      ok(me_gemm_f32((const float*)picked, (const float*)op.p[1], logits, rows, vocab, h_, stream_));
-    else if (rows > 2 && rows <= kHeadStreamRows && weight_bound(rows, vocab, h_))  // ahead of the small kernel and the library
-      ok(me_gemm_bf16_stream(picked, op.p[1], logits, rows, vocab, h_, 0, kF32, 1, compute_units(), stream_));
-    else if (rows <= kSmallFastRows && h_ % 8 == 0)
-      ok(me_gemm_bf16_small(picked, nullptr, nullptr, nullptr, 0.f, nullptr, op.p[1], logits, rows, vocab, h_, 0, 0, kF32, 1, stream_));
-    else
-      library_product(picked, op.p[1], logits, rows, vocab, h_, kF32, stream_);
+    product(picked, op.p[1], vocab, h_, 0, kF32, logits, kRoleHead, rows);
     if (op.f[1] != 1.f) ok(me_scale_f32(logits, op.f[1], (long long)rows * vocab, stream_));
     result_.logits = logits;
   }
@@ -496,7 +392,6 @@ class Run {
   int32_t* fed_tokens_;
   hipStream_t stream_;
   const int dtype_, elem_, t_, h_;
-  const int& t_rows_ = t_;
   float *x_, *spare_;
   void* normed_;
   std::vector<void*> bufs_;
@@ -536,7 +431,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
     size_t need = 0;
     if (op.kind == kOpNormLinear || op.kind == kOpLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
     if (op.kind == kOpLinearDelta)  // up to 16 partial sums of up to 64 rows, or one float32 result of all rows
-      need = std::max<size_t>((size_t)16 * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
+      need = std::max<size_t>((size_t)kMaxRuns * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
     if (op.kind == kOpAttention) {
       const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
       const int chunks = (nh / nkv + 15) / 16;
@@ -555,7 +450,18 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
   const size_t tail = (size_t)rows * hidden_ * elem + (size_t)rows * vocab_ * 4 + (size_t)rows * 4 +
                       (size_t)rows * me_sample_chunks(vocab_) * 8 + 4 * pad;
   // partial sums of the last delta wait beside the head's buffers
-  return fixed + 2 * scratch + tail + std::max<size_t>((size_t)16 * kSmallMaxRows, (size_t)tokens) * hidden_ * 4 + (1 << 16);
+  return fixed + 2 * scratch + tail + std::max<size_t>((size_t)kMaxRuns * kSmallMaxRows, (size_t)tokens) * hidden_ * 4 + (1 << 16);
 }
 
 }  // namespace me
+
+// A plain bfloat16 product through the GEMM library, with this folder's kernels where the library has no algorithm:
+// what the step program calls for a product that choose_product leaves to the library, for callers outside it.
+extern "C" int me_gemm_bf16_any(const void* x, const void* w, void* out, int m, int n, int k, int out_dtype, hipStream_t stream) {
+  try {
+    me::library_product(x, w, out, m, n, k, out_dtype, stream);
+    return 0;
+  } catch (const std::exception& e) {
+    return me_fail("%s", e.what());
+  }
+}

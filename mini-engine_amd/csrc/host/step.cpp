@@ -63,10 +63,23 @@ uint64_t Core::draw_key(const Request* r) const {
 void Core::check_step(int vocab_size, bool scan_pages) const {
   if (step_.empty()) throw Error(kBadValue, "a step needs at least one item");
   const int bs = config_.block_size;
+  // A request named twice would advance twice when the step is settled, and its second item would read keys that the
+  // first writes in the same launch.
+  const uint64_t stamp = ++check_stamp_;
+  for (const StepItem& it : step_) {
+    if (it.request->seen_in_check == stamp)
+      throw Error(kBadValue, "request " + std::to_string(it.request->handle) + " appears twice in one step");
+    it.request->seen_in_check = stamp;
+  }
   for (const StepItem& it : step_) {
     const Request* r = it.request;
     if (it.count < 1) throw Error(kBadValue, "an item needs at least one token");
     if (it.start < 0) throw Error(kBadValue, "item starts at negative position " + std::to_string(it.start));
+    // Positions between the computed ones and the item's first would hold whatever the page's owner before left there,
+    // and every later token would see them under the causal mask.
+    if (it.start > r->num_computed)
+      throw Error(kBadValue, "item starts at position " + std::to_string(it.start) + " but only " +
+                                 std::to_string(r->num_computed) + " tokens of its request are computed: a step may not leave a gap");
     if (it.start + it.count > r->size()) throw Error(kBadValue, "an item reaches beyond its request's tokens");
     if (it.start + it.count > config_.max_model_len)
       throw Error(kBadValue, "item reaches position " + std::to_string(it.start + it.count) + ", beyond the limit of " +
@@ -192,7 +205,7 @@ void Core::refill(int32_t* dst, const StepLayout& lay, std::vector<RowMemo>& row
     memcpy(dst + lay.sample_keys + 2 * i, &key, 8);
     RowMemo& memo = rows[i];
     if (!is_live) {
-      if (memo.handle >= 0 || memo.written.empty()) {
+      if (memo.handle != -1 || memo.written.empty()) {  // also a row whose last refill threw half-way (-2)
         for (size_t g = 0; g < lay.widths.size(); ++g)
           std::fill_n(dst + lay.tables[g] + (size_t)i * lay.widths[g], lay.widths[g], spare_page);
         memo.handle = -1;

@@ -372,28 +372,38 @@ class NormedInput:
                 self.residual = self.x
         return self._tensor
 
-    def streams_normed(self, weight: torch.Tensor) -> bool:
-        """Whether add, norm and the product go into one launch of the weight-streaming kernel: a row or two,
-        whatever the delta is (every block adds and norms the rows itself)."""
+    def fusion(self, weight: torch.Tensor) -> int:
+        """How add, norm and the product with ``weight`` are launched: :data:`NORM_ALONE`, :data:`NORM_IN_STREAM` (one
+        launch of the weight-streaming kernel: a row or two, whatever the delta is) or :data:`NORM_IN_SMALL` (the small
+        matrix-core kernel's prologue: decode-sized steps whose delta is a tensor). The rule is the native step
+        program's (``csrc/host/choice.cpp``); what is asked here on top is that the add has not happened yet and that
+        a sum has a second buffer to go to."""
+        if (self.dtype is not torch.bfloat16 or weight.dtype is not torch.bfloat16 or self._tensor is not None
+                or self.residual is not None or (self.delta is not None and self.spare is None)):
+            return NORM_ALONE
         rows, k = self.x.shape
-        return (self.dtype is torch.bfloat16 and self._tensor is None and self.residual is None
-                and rows <= NORM_STREAM_ROWS and weight.dtype is torch.bfloat16 and (self.delta is None or self.spare is not None)
-                and k % 8 == 0 and weight.numel() * 2 < STREAM_MAX_BYTES and weight.data_ptr() % 16 == 0 and stream_norm_fits(rows, k))
+        pending = 0 if self.delta is None else 2 if isinstance(self.delta, PartialSums) else 1
+        return int(lib().me_norm_fusion_choice(_i(_code(self.dtype)), _i(rows), _i(weight.shape[0]), _i(k), _i(pending),
+                                               _i(compute_units(weight.device)), _i(int(weight.data_ptr() % 16 == 0))))
 
-    def fusable(self, weight: torch.Tensor) -> bool:
-        """Whether add, norm and the product with ``weight`` go into one kernel: decode-sized steps whose
-        delta is a tensor (partial sums are read once, by the add-and-norm kernel, not by every block of a
-        product) and whose weight is not so large that the weight-streaming kernel serves it."""
-        return (self.dtype is torch.bfloat16 and self._tensor is None and self.x.shape[0] <= SMALL_FAST_ROWS
-                and self.x.shape[1] % 8 == 0 and (self.delta is None or self.spare is not None)
-                and not isinstance(self.delta, PartialSums) and weight.dtype is torch.bfloat16
-                and weight.numel() < STREAM_MIN_ELEMENTS)
+
+NORM_ALONE, NORM_IN_STREAM, NORM_IN_SMALL = 0, 1, 2  # csrc/host/choice.h: NormFusion
+PRODUCT_F32, PRODUCT_SMALL, PRODUCT_STREAM, PRODUCT_TILED, PRODUCT_LIBRARY = range(5)  # csrc/host/choice.h: ProductKernel
+ROLE_PLAIN, ROLE_DELTA, ROLE_HEAD = range(3)  # csrc/host/choice.h: ProductRole
+
+
+def product_choice(dtype: torch.dtype, role: int, rows: int, rows_of_w: int, k: int, gated: bool, out_dtype: torch.dtype,
+                   units: int, aligned: bool = True) -> tuple[int, int, bool, bool]:
+    """Which kernel serves a product: (kernel, runs of k, the result is float32 partial sums, the gate is a kernel of
+    its own behind the product). The one rule of the tree, in ``csrc/host/choice.cpp``; no GPU is touched."""
+    out = (ctypes.c_int * 4)()
+    lib().me_product_choice(_i(_code(dtype)), _i(role), _i(rows), _i(rows_of_w), _i(k), _i(int(bool(gated))), _i(_code(out_dtype)),
+                            _i(units), _i(int(aligned)), out)
+    return int(out[0]), int(out[1]), bool(out[2]), bool(out[3])
 
 
 STREAM_MAX_ROWS = 256  # the weight-streaming product deals more than 64 rows to groups of blocks
-NORM_STREAM_ROWS = 2  # up to here the add-and-norm is the prologue of the weight-streaming kernel
-SMALL_MAX_ROWS = 64  # what the kernel accepts
-SMALL_FAST_ROWS = 16  # up to here it beats the GEMM library on every shape, with the norm as its prologue too
+SMALL_MAX_ROWS = 64  # what the small matrix-core kernel accepts
 
 
 def compute_units(device=None) -> int:
@@ -415,21 +425,6 @@ def stream_plan(rows: int, n: int, k: int, gated: bool = False, k_splits: int = 
     lib().me_gemm_bf16_stream_plan(_i(rows), _i(n), _i(k), _i(int(bool(gated))), _i(k_splits),
                                    _i(units if units is not None else compute_units(device)), out)
     return int(out[0]), int(out[1]), int(out[2])
-
-
-STREAM_WHOLE_ROWS = 32  # up to here the weight-streaming kernel serves wide plain products whose blocks fill whole rounds (gated: 64)
-
-
-def stream_serves_mid_rows(rows: int, n: int, k: int, gated: bool, device=None) -> bool:
-    """Whether the weight-streaming kernel serves a wide product of 17 to 32 rows (64 for a gated one) instead of the GEMM library: its blocks
-    fill whole rounds of the compute units (15/16 of them at least) and the weight's rows are a multiple of 4 KiB apart
-    (the measurements are in ``csrc/host/program.cpp``)."""
-    if k % 2048 or rows > (SMALL_MAX_ROWS if gated else STREAM_WHOLE_ROWS):
-        return False
-    units = compute_units(device)
-    grid = stream_plan(rows, n, k, gated, 1, units=units)[2]
-    rounds = -(-grid // units)
-    return grid * 16 >= rounds * units * 15
 
 
 def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
@@ -562,7 +557,6 @@ def gemm_bf16_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
     return gemm_bf16_small(x, weight, out_dtype, False, out)
 
 
-TILED_MIN_ROWS = 256
 
 
 def gemm_bf16_tiled(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
@@ -587,93 +581,47 @@ def gemm_bf16_tiled(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
     return out
 
 
-def tiled_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    return (x.shape[0] >= TILED_MIN_ROWS and x.shape[1] % 64 == 0 and x.data_ptr() % 16 == 0
-            and weight.data_ptr() % 16 == 0)
-
-
-def small_ok(x, weight: torch.Tensor, gated: bool = False) -> bool:
-    """Whether the small matrix-core kernel serves this product: up to 16 rows (with more rows the
-    weight-streaming kernel, which fetches x once per block of columns, is ahead)."""
-    return x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and x.shape[0] <= SMALL_FAST_ROWS
-
-
-TILED_MAX_K = 3072  # gated products of longer k go to the library and a SwiGLU kernel (measured in csrc/host/program.cpp)
-HEAD_STREAM_ROWS = 32  # float32 products of large weights (a head's logits) stay with the weight-streaming kernel up to here
-STREAM_MIN_ELEMENTS = 8 << 20  # weights from 16 MiB on: streaming them is the product's time
-STREAM_MAX_BYTES = 1 << 31  # what the weight-streaming kernel addresses
-
-
-def weight_bound(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether a product of up to 64 rows is bound by streaming its weight (the layers of wide models): their
-    deltas go to the weight-streaming kernel with k cut into runs, their other products of 17 to 64 rows to
-    the library (the same rule as ``csrc/host/program.cpp``, where the measurements are)."""
-    return (x.shape[0] <= SMALL_MAX_ROWS and x.shape[1] % 8 == 0 and STREAM_MIN_ELEMENTS <= weight.numel()
-            and weight.numel() * 2 < STREAM_MAX_BYTES and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
-
-
-def streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """What the weight-streaming kernel takes at all."""
-    return (x.shape[0] <= SMALL_MAX_ROWS and x.shape[1] % 8 == 0 and weight.numel() * 2 < STREAM_MAX_BYTES
-            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
-
-
 def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None, gated: "bool | str" = False,
-           as_delta: bool = False):
+           as_delta: bool = False, head: bool = False):
     """``x @ weight.T`` for x [M, K], weight [N, K]; with ``gated`` (True or "silu", or "gelu_tanh") the
     weight is [2N, K] (gate rows, then up rows) and the result is ``act(gate) * up``. ``x`` may be a :class:`NormedInput`. With
     ``as_delta`` the caller says that the result only ever is the pending delta of the residual stream
     (what a mixer or a feed-forward returns): it may then come back as :class:`PartialSums`, which
-    :func:`add_rmsnorm` adds up on the way.
+    :func:`add_rmsnorm` adds up on the way. ``head``: the product gives the logits of the wanted rows.
 
-    float32: always the deterministic float32 kernel (a true 32-bit product). bfloat16, by rows and
-    weight size as ``csrc/host/program.cpp`` chooses (where the measurements are): up to 16 rows the small
-    matrix-core kernel, or the weight-streaming one for weights of 16 MiB and more; 17 to 64 rows the
-    weight-streaming kernel (the library for weights of 16 MiB and more); a delta of the residual stream
-    of up to 64 rows as partial sums over runs of k; the tiled matrix-core kernel with
-    the SwiGLU as its epilogue for gated products of 256 rows or more (the weight-streaming kernel up to 256 rows for
-    gated weights below 16 MiB); else the GEMM library."""
+    float32: always the deterministic float32 kernel (a true 32-bit product). bfloat16: the kernel that the native step
+    program would take for the same sizes (:func:`product_choice`; the rule and its measurements are in
+    ``csrc/host/choice.cpp``)."""
+    activation = "silu" if gated is True else gated
     if isinstance(x, NormedInput):
-        if x.streams_normed(weight):
+        how = x.fusion(weight)
+        if how == NORM_IN_STREAM:
             return gemm_bf16_stream_norm(x, weight, out_dtype or x.dtype, gated)
-        if x.fusable(weight):
+        if how == NORM_IN_SMALL:
             return gemm_bf16_small(x, weight, out_dtype or x.dtype, gated)
         x = x.materialize()
     out_dtype = out_dtype or x.dtype
-    if x.dtype is torch.float32:
-        if out_dtype is not torch.float32:
-            raise TypeError("the float32 path keeps float32 results")
+    if x.dtype is torch.float32 and out_dtype is not torch.float32:
+        raise TypeError("the float32 path keeps float32 results")
+    role = ROLE_DELTA if as_delta and not gated else ROLE_HEAD if head else ROLE_PLAIN
+    aligned = x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+    kernel, runs, partial, gate_after = product_choice(x.dtype, role, x.shape[0], weight.shape[0], x.shape[1], bool(gated),
+                                                       out_dtype, compute_units(x.device), aligned)
+    epilogue = False if gate_after else gated
+    inner = torch.float32 if partial else x.dtype if gate_after else out_dtype
+    if kernel == PRODUCT_F32:
         y = gemm_f32(x, weight)
-        return swiglu(y, activation="silu" if gated is True else gated) if gated else y
-    heavy, few = weight_bound(x, weight), x.shape[0] <= SMALL_FAST_ROWS
-    if as_delta and not gated and streams(x, weight):
-        splits = stream_splits(weight.shape[0], x.shape[1], x.device, x.shape[0])
-        parts = gemm_bf16_stream(x, weight, torch.float32, k_splits=splits)
-        return PartialSums(parts if splits > 1 else parts.unsqueeze(0))
-    if as_delta and not gated and out_dtype is torch.bfloat16:
-        # more rows: the library's product with a float32 result, which stands as one partial sum (the delta is never
-        # rounded to bfloat16 on its way into the float32 residual stream)
-        return PartialSums(gemm_bf16_library(x, weight, torch.float32).unsqueeze(0))
-    if (heavy if few else streams(x, weight) and not heavy) and (out_dtype is torch.bfloat16 or not gated):
-        return gemm_bf16_stream(x, weight, out_dtype, gated)
-    if (heavy and (out_dtype is torch.bfloat16 or not gated)
-            and stream_serves_mid_rows(x.shape[0], weight.shape[0] // (2 if gated else 1), x.shape[1], bool(gated), x.device)):
-        return gemm_bf16_stream(x, weight, out_dtype, gated)  # 17 to 32 rows of a wide product (see stream_serves_mid_rows)
-    if heavy and x.shape[0] <= HEAD_STREAM_ROWS and out_dtype is torch.float32 and not gated:  # a head's logits
-        return gemm_bf16_stream(x, weight, out_dtype)
-    if small_ok(x, weight, gated) and not heavy:
-        return gemm_bf16_small(x, weight, out_dtype, gated)
-    if (gated and x.shape[0] <= STREAM_MAX_ROWS and x.shape[1] % 8 == 0 and weight.numel() < STREAM_MIN_ELEMENTS
-            and out_dtype is torch.bfloat16):
-        return gemm_bf16_stream(x, weight, out_dtype, gated)  # 65 to 256 rows of a small gated weight, in groups of 64 rows
-    if gated:
-        if tiled_ok(x, weight) and x.shape[1] <= TILED_MAX_K and out_dtype is torch.bfloat16:
-            return gemm_bf16_tiled(x, weight, out_dtype, gated)  # measured ahead of the library product + SwiGLU kernel
-        return swiglu(linear(x, weight, out_dtype), activation="silu" if gated is True else gated)
-    return gemm_bf16_library(x, weight, out_dtype)
-
-
-_LIBRARY_REFUSED: set = set()  # (N, K, output type) of products the direct library call has no algorithm for
+    elif kernel == PRODUCT_SMALL:
+        y = gemm_bf16_small(x, weight, inner, epilogue)
+    elif kernel == PRODUCT_STREAM:
+        y = gemm_bf16_stream(x, weight, inner, epilogue, k_splits=runs)
+    elif kernel == PRODUCT_TILED:
+        y = gemm_bf16_tiled(x, weight, inner, epilogue)
+    else:
+        y = gemm_bf16_library(x, weight, inner)
+    if partial:
+        return PartialSums(y if runs > 1 else y.unsqueeze(0))
+    return swiglu(y, activation=activation) if gate_after else y
 
 
 def gemm_bf16_library(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
@@ -681,7 +629,7 @@ def gemm_bf16_library(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dt
     """bfloat16 ``x @ weight.T`` through the GEMM library with float32 accumulation, as bfloat16 or as
     float32 (logits, not rounded to bfloat16). The library is called directly (a third of the host time
     of a call through torch); where it has no algorithm for the sizes (widths that are no multiple of
-    8), torch's product stands in, and for float32 results slices of 64 rows through the matrix-core kernel."""
+    8), the kernels of this package stand in, as in the native step program."""
     _want(x, "x", torch.bfloat16, (None, None))
     m, k = x.shape
     _want(weight, "weight", torch.bfloat16, (None, k))
@@ -689,21 +637,8 @@ def gemm_bf16_library(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dt
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _want(out, "out", out_dtype, (m, n))
-    shape_class = (n, k, out_dtype)
-    if shape_class not in _LIBRARY_REFUSED:
-        if lib().me_gemm_bf16_library(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(_code(out_dtype)), _stream()) == 0:
-            return out
-        _LIBRARY_REFUSED.add(shape_class)
-    if out_dtype is torch.float32:
-        try:
-            return torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
-        except (TypeError, RuntimeError):
-            if k % 8:
-                raise
-            for lo in range(0, m, SMALL_MAX_ROWS):
-                gemm_bf16_small(x[lo:lo + SMALL_MAX_ROWS], weight, torch.float32, False, out[lo:lo + SMALL_MAX_ROWS])
-            return out
-    return torch.matmul(x, weight.t(), out=out)
+    check(lib().me_gemm_bf16_any(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(_code(out_dtype)), _stream()))
+    return out
 
 
 # -------------------------------------------------------------------------------------- sampling

@@ -118,7 +118,7 @@ class Decoder:
             if pending is not None:
                 K.residual_add(x, pending)
             h = self.final_norm.forward(x.index_select(0, rows.long()))
-        logits = K.linear(h, self.head, torch.float32)
+        logits = K.linear(h, self.head, torch.float32, head=True)
         if self.plan.logit_scale not in (None, 1.0):
             K.scale_(logits, self.plan.logit_scale)
         return logits

@@ -200,3 +200,50 @@ def temperature_probs(logits: torch.Tensor, temperature: float) -> torch.Tensor:
     z = z - z.max(dim=-1, keepdim=True).values
     p = z.exp()
     return p / p.sum(dim=-1, keepdim=True)
+
+
+# ------------------------------------------------------------- the same model, as a bfloat16 engine rounds it
+
+
+def _bf16(x: torch.Tensor) -> torch.Tensor:
+    return x.to(torch.bfloat16).to(torch.float32)
+
+
+def forward_logits_rounded(w: dict[str, torch.Tensor], cfg: PlainConfig, tokens: list[int]) -> torch.Tensor:
+    """:func:`forward_logits` with every operand of a matrix product rounded to bfloat16 where a bfloat16 engine holds
+    it in bfloat16 (the normed activations, q, k and v as projected and again as rotated, the softmax weights before
+    they multiply the values, the attention output, the gated activation, the rows in front of the head) and every sum,
+    the residual stream, the norms and the softmax in float32. The weights are expected to be bfloat16 values already.
+    What is left between this and a bfloat16 engine is the order of float32 sums and the few places where kernels of
+    different step sizes round differently; what is left between this and :func:`forward_logits` is bfloat16 itself."""
+    ids = torch.tensor(tokens, dtype=torch.long)
+    x = w["model.embed_tokens.weight"][ids]
+    t = len(tokens)
+    positions = torch.arange(t)
+    group = cfg.num_heads // cfg.num_kv_heads
+    mask = visible(t, t)
+    for layer in range(cfg.num_layers):
+        p = f"model.layers.{layer}"
+        a = f"{p}.self_attn"
+        h = _bf16(rms_norm(x, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps))
+        q = _bf16(h @ w[f"{a}.q_proj.weight"].T).view(t, cfg.num_heads, cfg.head_dim)
+        k = _bf16(h @ w[f"{a}.k_proj.weight"].T).view(t, cfg.num_kv_heads, cfg.head_dim)
+        v = _bf16(h @ w[f"{a}.v_proj.weight"].T).view(t, cfg.num_kv_heads, cfg.head_dim)
+        cos, sin = rope_tables(positions, cfg.head_dim, cfg.rope_theta)
+        q = _bf16(apply_rope(rms_norm(q, w[f"{a}.q_norm.weight"], cfg.rms_norm_eps), cos, sin))
+        k = _bf16(apply_rope(rms_norm(k, w[f"{a}.k_norm.weight"], cfg.rms_norm_eps), cos, sin))
+        out = torch.empty_like(q)
+        for head in range(cfg.num_heads):
+            kv = head // group
+            s = (q[:, head] @ k[:, kv].T) * cfg.head_dim**-0.5
+            s = s.masked_fill(~mask, float("-inf"))
+            e = (s - s.max(dim=-1, keepdim=True).values).exp()
+            out[:, head] = (_bf16(e) @ v[:, kv]) / e.sum(dim=-1, keepdim=True)
+        x = x + _bf16(out.reshape(t, -1)) @ w[f"{a}.o_proj.weight"].T
+        h = _bf16(rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], cfg.rms_norm_eps))
+        m = f"{p}.mlp"
+        act = _bf16(silu(h @ w[f"{m}.gate_proj.weight"].T) * (h @ w[f"{m}.up_proj.weight"].T))
+        x = x + act @ w[f"{m}.down_proj.weight"].T
+    x = _bf16(rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps))
+    head = w["model.embed_tokens.weight"] if cfg.tie_word_embeddings else w["lm_head.weight"]
+    return x @ head.T

@@ -80,12 +80,12 @@ def test_padding_items_write_to_the_spare_page():
 
 
 def test_checks_catch_what_would_make_a_kernel_fault():
-    def check(tokens, start, count, want, pages_for=None, vocab=10, window=0, computed=0, passed=False):
+    def check(tokens, start, count, want, pages_for=None, vocab=10, window=0, computed=None, passed=False):
         core = HostCore(BS, [(window, 32)], max_model_len=64)
         seq = Sequence(tokens, core=core)
         assert core.grow(seq._handle, len(tokens) if pages_for is None else pages_for)
+        seq.num_computed_tokens = start if computed is None else computed
         if passed:
-            seq.num_computed_tokens = computed
             core.drop_passed(seq._handle)
         core.step_add(seq._handle, start, count, want)
         core.step_check(vocab)
@@ -105,11 +105,30 @@ def test_checks_catch_what_would_make_a_kernel_fault():
         check([1] * 80, 0, 80, [])
     with pytest.raises(ValueError, match="at least one"):
         HostCore(BS, [(0, 4)]).step_check(10)
+    # an item that starts beyond what is computed would leave positions that nothing ever wrote under the mask
+    with pytest.raises(ValueError, match="gap"):
+        check([1, 2, 3, 4, 5], 2, 3, [2], computed=1)
+    check([1, 2, 3, 4, 5], 2, 3, [2], computed=2)
+
     # in a window group only pages the window still covers have to be there: with 6 tokens computed and a
     # window of 3 the first page is given back; a step at position 6 needs keys from 4 on
     check([1] * 7, 6, 1, [], window=3, computed=6, passed=True)
     with pytest.raises(ValueError, match="given back"):  # position 4 sees keys from 2 on, which are gone
         check([1] * 7, 4, 1, [], window=3, computed=6, passed=True)
+
+
+def test_a_request_may_appear_once_in_a_step():
+    core = HostCore(BS, [(0, 16)])
+    a, b = held(core, [1, 2, 3, 4]), held(core, [5, 6])
+    core.step_add(a._handle, 0, 2, [])
+    core.step_add(b._handle, 0, 2, [1])
+    core.step_check(10)
+    core.step_add(a._handle, 0, 2, [1])
+    with pytest.raises(ValueError, match="twice"):
+        core.step_check(10)
+    core.step_clear()
+    core.step_add(a._handle, 0, 4, [3])  # the check before left nothing behind
+    core.step_check(10)
 
 
 def test_refill_extends_rows_and_rewrites_what_changed():
@@ -137,6 +156,31 @@ def test_refill_extends_rows_and_rewrites_what_changed():
     assert core.grow(a._handle, 9)
     assert replay([a, b])[0] == a.block_table + [31]
     assert replay([b]) == [[2, 3, 4, 31], [31, 31, 31, 31]] and section(buf, lay, "live_items", 1) == [1]
+
+
+def test_a_refill_that_throws_leaves_no_half_written_row_behind():
+    # two groups: one keeps every key, the other a window of 3, whose passed pages are given back
+    core = HostCore(BS, [(0, 32), (3, 32)], seed=3)
+    a, b = held(core, [1] * 5, computed=4), held(core, [2] * 13, computed=12)
+    core.drop_passed(b._handle)
+    widths, lay = [4, 4], step_layout(2, 2, 2, [4, 4])
+    buf = np.zeros(lay["total"], dtype=np.int32)
+    core.pack_padding(buf, widths, 2, 31, 0)
+    table = lambda g: buf[lay["tables"][g]:lay["tables"][g] + 8].reshape(2, 4).tolist()
+    core.step_add(a._handle, 4, 1, [0])
+    core.step_add(b._handle, 12, 1, [0])
+    core.step_refill(2, buf, widths, 31, 0)  # a good refill first: the row remembers whose table it holds
+    core.step_clear()
+    core.step_add(a._handle, 4, 1, [0])
+    core.step_add(b._handle, 6, 1, [0])  # position 6 would see keys from 4 on: the window group's page is gone
+    with pytest.raises(ValueError, match="given back"):
+        core.step_refill(2, buf, widths, 31, 0)
+    assert table(0)[1] != [31] * 4  # the first group's row holds pages of b
+    core.step_clear()
+    core.step_add(a._handle, 4, 1, [0])  # the second row is padding now: it keeps nothing of the failed refill
+    core.step_refill(2, buf, widths, 31, 0)
+    assert table(0)[1] == [31] * 4 and table(1)[1] == [31] * 4
+    assert table(0)[0] == a.block_tables[0] + [31, 31]
 
 
 def test_buckets_match_the_reference():  # cuda_graphs.py:28-30, tests/test_gpu.py:47

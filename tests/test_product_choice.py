@@ -1,0 +1,83 @@
+"""The one rule that says which kernel serves a matrix product (``csrc/host/choice.cpp``), which the native step program
+and ``ops.kernels.linear`` both ask: swept over the projections of five model shapes and every row count a step may
+bring, every answer must be one that the named kernel accepts. No GPU is touched."""
+
+import pytest
+import torch
+
+from mini_engine_amd.ops import kernels as K
+
+# hidden, heads, kv heads, head size, intermediate (Qwen3 0.6B, 1.7B, 4B, 8B, 32B: their config.json sizes)
+SHAPES = {
+    "0.6b": (1024, 16, 8, 128, 3072),
+    "1.7b": (2048, 16, 8, 128, 6144),
+    "4b": (2560, 32, 8, 128, 9728),
+    "8b": (4096, 32, 8, 128, 12288),
+    "32b": (5120, 64, 8, 128, 25600),
+}
+VOCAB = 151936
+BF16, F32 = torch.bfloat16, torch.float32
+
+
+def projections(shape):
+    hidden, heads, kv, d, inter = SHAPES[shape]
+    return [("qkv", (heads + 2 * kv) * d, hidden, False, K.ROLE_PLAIN), ("o", hidden, heads * d, False, K.ROLE_DELTA),
+            ("gate_up", 2 * inter, hidden, True, K.ROLE_PLAIN), ("down", hidden, inter, False, K.ROLE_DELTA),
+            ("head", VOCAB, hidden, False, K.ROLE_HEAD)]
+
+
+def accepted(kernel, rows, rows_of_w, k, gated, runs, partial, out_dtype):
+    """What each kernel's entry point takes (the limits its wrapper in ops/kernels.py states)."""
+    if kernel == K.PRODUCT_SMALL:
+        return rows <= K.SMALL_MAX_ROWS and k % 8 == 0 and runs == 1
+    if kernel == K.PRODUCT_STREAM:
+        plain_f32 = not gated and (partial or out_dtype is F32)
+        return (rows <= K.STREAM_MAX_ROWS and k % 8 == 0 and rows_of_w * k * 2 < 2**31 and (runs == 1 or plain_f32)
+                and 1 <= runs <= 16 and (runs == 1 or rows <= 64))
+    if kernel == K.PRODUCT_TILED:
+        return k % 64 == 0 and runs == 1
+    return kernel == K.PRODUCT_LIBRARY and runs == 1
+
+
+@pytest.mark.parametrize("shape", sorted(SHAPES))
+@pytest.mark.parametrize("units", [256, 304, 104])
+def test_every_choice_is_one_its_kernel_accepts(shape, units):
+    kernels_seen = set()
+    for name, rows_of_w, k, gated, role in projections(shape):
+        out_dtype = F32 if role == K.ROLE_HEAD else BF16
+        for rows in list(range(1, 301)) + [512, 2048, 8192]:
+            kernel, runs, partial, gate_after = K.product_choice(BF16, role, rows, rows_of_w, k, gated, out_dtype, units)
+            assert accepted(kernel, rows, rows_of_w, k, gated and not gate_after, runs, partial, out_dtype), (name, rows, kernel, runs)
+            assert partial == (role == K.ROLE_DELTA) and (not gate_after or gated)
+            if gate_after:  # a gate behind the product needs the whole product first
+                assert kernel == K.PRODUCT_LIBRARY
+            kernels_seen.add(kernel)
+            # the float32 path knows one product
+            assert K.product_choice(F32, role, rows, rows_of_w, k, gated, F32, units) == (K.PRODUCT_F32, 1, False, gated)
+    assert K.PRODUCT_STREAM in kernels_seen and K.PRODUCT_LIBRARY in kernels_seen
+
+
+def test_sizes_no_kernel_of_the_package_takes_go_to_the_library():
+    for rows in (1, 16, 64, 300):
+        assert K.product_choice(BF16, K.ROLE_PLAIN, rows, 100, 36, False, BF16, 256)[0] == K.PRODUCT_LIBRARY  # k % 8
+        assert K.product_choice(BF16, K.ROLE_PLAIN, rows, 96, 64, False, BF16, 256, aligned=False)[0] == K.PRODUCT_LIBRARY
+        kernel, runs, partial, _ = K.product_choice(BF16, K.ROLE_DELTA, rows, 100, 36, False, BF16, 256)
+        assert (kernel, runs, partial) == (K.PRODUCT_LIBRARY, 1, True)
+    for rows in (1, 8, 32, 64):  # 2 GiB of weight: beyond what the weight-streaming kernel addresses
+        for role in (K.ROLE_PLAIN, K.ROLE_DELTA, K.ROLE_HEAD):
+            assert K.product_choice(BF16, role, rows, 2**20, 1024, False, BF16, 256)[0] != K.PRODUCT_STREAM
+
+
+def test_the_measured_rules_at_their_shapes():
+    """What the measurements beside the rules decided, at the sizes they were taken at."""
+    pick = lambda role, rows, rows_of_w, k, gated=False, out=BF16: K.product_choice(BF16, role, rows, rows_of_w, k, gated, out, 256)[:2]
+    assert pick(K.ROLE_PLAIN, 8, 4096, 1024) == (K.PRODUCT_SMALL, 1) and pick(K.ROLE_PLAIN, 32, 4096, 1024) == (K.PRODUCT_STREAM, 1)
+    assert pick(K.ROLE_PLAIN, 8, 6144, 4096) == (K.PRODUCT_STREAM, 1) and pick(K.ROLE_PLAIN, 48, 6144, 4096) == (K.PRODUCT_LIBRARY, 1)
+    assert pick(K.ROLE_DELTA, 8, 1024, 3072) == (K.PRODUCT_STREAM, 6) and pick(K.ROLE_DELTA, 65, 1024, 3072) == (K.PRODUCT_LIBRARY, 1)
+    assert pick(K.ROLE_PLAIN, 128, 6144, 1024, True) == (K.PRODUCT_STREAM, 1) and pick(K.ROLE_PLAIN, 2048, 6144, 1024, True) == (K.PRODUCT_TILED, 1)
+    assert pick(K.ROLE_PLAIN, 2048, 24576, 4096, True) == (K.PRODUCT_LIBRARY, 1)
+    assert pick(K.ROLE_HEAD, 1, VOCAB, 1024, out=F32) == (K.PRODUCT_SMALL, 1) and pick(K.ROLE_HEAD, 8, VOCAB, 1024, out=F32) == (K.PRODUCT_STREAM, 1)
+    assert pick(K.ROLE_HEAD, 64, VOCAB, 1024, out=F32) == (K.PRODUCT_LIBRARY, 1)
+    fusion = lambda rows, rows_of_w, k, pending: K.lib().me_norm_fusion_choice(1, rows, rows_of_w, k, pending, 256, 1)
+    assert fusion(1, 4096, 1024, 2) == K.NORM_IN_STREAM and fusion(8, 4096, 1024, 1) == K.NORM_IN_SMALL
+    assert fusion(8, 4096, 1024, 2) == K.NORM_ALONE and fusion(8, 6144, 4096, 1) == K.NORM_ALONE and fusion(17, 4096, 1024, 0) == K.NORM_ALONE

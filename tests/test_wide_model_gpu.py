@@ -61,9 +61,13 @@ def test_wide_layers_against_plain(model, path):
     folder, reqs, want, hidden = model
     # the paths this test is for: weights that count as bound by their streaming; at hidden 4096 the products of 24 rows that
     # the weight-streaming kernel takes from the library
-    assert 2 * 12288 * hidden >= K.STREAM_MIN_ELEMENTS and 2048 * hidden >= K.STREAM_MIN_ELEMENTS
-    assert K.stream_serves_mid_rows(24, 12288, hidden, True) == (hidden == 4096)
-    assert K.stream_serves_mid_rows(24, 6144, 4096, False) and not K.stream_serves_mid_rows(24, 5120, 4096, False)
+    import torch
+
+    units, bf16 = K.compute_units(), torch.bfloat16
+    choice = lambda rows, rows_of_w, k, gated: K.product_choice(bf16, K.ROLE_PLAIN, rows, rows_of_w, k, gated, bf16, units)[0]
+    assert choice(8, 2 * 12288, hidden, True) == K.PRODUCT_STREAM and choice(8, 2048, hidden, False) == K.PRODUCT_STREAM
+    assert (choice(24, 2 * 12288, hidden, True) == K.PRODUCT_STREAM) == (hidden == 4096)
+    assert choice(24, 6144, 4096, False) == K.PRODUCT_STREAM and choice(24, 5120, 4096, False) == K.PRODUCT_LIBRARY
     steps = steps_for(reqs)
     engine = build_session(folder, "bfloat16", 64 * 40, block_size=16, max_live=40, cuda_graphs=path == "replayed")
     if path == "per kernel":
