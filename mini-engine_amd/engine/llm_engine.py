@@ -113,7 +113,9 @@ class LLMEngine:
     @classmethod
     def from_random(cls, architecture: str, arch_config, config: EngineConfig | None = None, seed: int = 0,
                     std: float = 0.02) -> "LLMEngine":
-        """Build the architecture with seeded random weights generated on the GPU (no files)."""
+        """Build the architecture with seeded random weights generated on the GPU (no files). The values come from the
+        GPU's generator: they are other values than those of a model folder written for the same seed
+        (``weights.random_init.write_model_folder`` draws on the CPU), with the same distribution."""
         config = config or EngineConfig()
         plan = get_architecture(architecture).plan_from_config(arch_config)
         model = Decoder(plan, TORCH_DTYPES[config.dtype], "cuda")

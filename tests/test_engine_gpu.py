@@ -410,3 +410,43 @@ def test_steps_launched_ahead_change_no_token(peaked, name):
     assert outs[True, "squeezed"] == outs[False, "squeezed"] == cut
     assert outs[True, "sampled"] == outs[False, "sampled"] and outs[True, "sampled"] != [o[:17] for o in cut]
     assert any(eos in o for o in cut) and any(eos not in o for o in cut)
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("D", "bfloat16")])
+def test_from_random_fills_every_tensor(tmp_path, name, dtype):
+    """``LLMEngine.from_random`` (engine.py:136-141 there; the loader of every benchmark number here) draws its weights on
+    the GPU, so they are other values than a model folder written for the same seed holds. The same source, asked
+    tensor by tensor, gives the tensors to write a folder from; the plain implementation on that folder must agree
+    with the engine: every wanted tensor was filled, the norm weights lie around 1, a tied head is the embedding."""
+    import trace_helpers as th
+    from mini_engine_amd import EngineConfig, LLMEngine, SamplingParams
+    from mini_engine_amd.engine.batch import StepItem
+    from mini_engine_amd.engine.sequence import Sequence
+    from mini_engine_amd.weights import RandomSource
+    from mini_engine_amd.weights.safetensors_io import write_file
+    import json
+
+    cfg = tiny_configs()[name]
+    torch_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
+    eng = LLMEngine.from_random("Qwen3ForCausalLM", cfg, EngineConfig(block_size=BLOCK_SIZES[name], num_blocks=64, dtype=dtype,
+                                                                      max_model_len=256), seed=5, std=0.2 if dtype == "float32" else 0.05)
+    wants = eng.model.weight_wants()
+    src = RandomSource(wants, 5, std=0.2 if dtype == "float32" else 0.05, device="cuda")
+    tensors = {n: src.get(n).to(torch.float32 if wants[n].role == "vector" else torch_dtype).cpu() for n in wants}
+    assert ("lm_head.weight" in tensors) == (not cfg.tie_word_embeddings)
+    norms = [t for n, t in tensors.items() if wants[n].role == "vector"]
+    assert norms and all(abs(t.mean().item() - 1) < 0.05 and 0 < t.std().item() < 0.05 for t in norms)
+    folder = str(tmp_path)
+    write_file(os.path.join(folder, "model.safetensors"), tensors, {"format": "pt"})
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg.to_config_json(), f)
+    pcfg, w = plain.read_config(folder), plain.read_weights(folder)
+    tokens = random_prompt(40, cfg.vocab_size, seed=2)
+    want = plain.forward_logits(w, pcfg, tokens)
+    seq = Sequence(tokens, core=eng.core)
+    assert eng.block_manager.try_allocate(seq, len(tokens))
+    got = eng.runner.step([StepItem(seq, tokens, 0, list(range(len(tokens))))]).float().cpu()
+    eng.block_manager.free(seq)
+    th.assert_logits_close(got, want, dtype, f"from_random {name} {dtype}")
+    if dtype == "float32":
+        assert eng.generate([tokens[:9]], SamplingParams(max_tokens=6))[0] == plain.greedy_generate(w, pcfg, tokens[:9], 6)

@@ -71,6 +71,26 @@ def test_rope_is_a_rotation_of_pairs_j_and_j_plus_half_by_pos_times_theta_pow():
     torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
 
 
+def test_rope_on_a_vector_worked_by_hand_from_the_reference_lines():
+    """model.py:75 with d = 4, theta = 10000: inv_freq = [10000^0, 10000^(-2/4)] = [1, 0.01]. model.py:86-90 at
+    position 1 on x = [1, 2, 3, 4]: x1 = [1, 2], x2 = [3, 4], cat(-x2, x1) = [-3, -4, 1, 2], angles [1, 0.01, 1, 0.01]:
+      out = [1 cos 1 - 3 sin 1, 2 cos 0.01 - 4 sin 0.01, 3 cos 1 + 1 sin 1, 4 cos 0.01 + 2 sin 0.01]
+    with cos 1 = 0.5403023, sin 1 = 0.8414710, cos 0.01 = 0.99995, sin 0.01 = 0.00999983 (the literals below are
+    worked out from these by hand). Pairs (2j, 2j+1) would give -1.1426 first; the exponent j/d would give the
+    second angle as 0.1."""
+    cos, sin = plain.rope_tables(torch.tensor([1]), 4, 10000.0)
+    got = plain.apply_rope(torch.tensor([[[1.0, 2.0, 3.0, 4.0]]]), cos, sin)[0, 0]
+    torch.testing.assert_close(got, torch.tensor([-1.9841107, 1.9599007, 2.4623779, 4.0197997]), rtol=0, atol=2e-6)
+    # and at position 3 with d = 8, theta = 1e6 (the benchmark's theta): angle of pair (2, 6) is 3 * 1e6^(-4/8) = 0.003
+    cos, sin = plain.rope_tables(torch.tensor([3]), 8, 1e6)
+    x = torch.zeros(1, 1, 8)
+    x[0, 0, 2] = 1.0
+    got = plain.apply_rope(x, cos, sin)[0, 0]
+    want = torch.zeros(8)
+    want[2], want[6] = 0.9999955, 0.0029999955  # cos 0.003, sin 0.003: the unit vector of element 2 turns towards element 6
+    torch.testing.assert_close(got, want, rtol=0, atol=1e-7)
+
+
 def test_rope_scores_depend_on_distance_only():
     d = 32
     q, k = torch.randn(1, 1, d, dtype=torch.float64), torch.randn(1, 1, d, dtype=torch.float64)

@@ -37,6 +37,23 @@ def _sample(L, logits, temps, keys, static: bool):
     return out.cpu()
 
 
+def host_scores(logits_row, temperature: float, key: int):
+    """What the kernel maximises for a tempered row, from its definition and in float64: logit / max(t, 1e-5) + g_i with
+    g_i = -log(-log(u_i)), u_i = (top 32 bits of mix64(key ^ mix64(i)) + 0.5) / 2^32."""
+    import numpy as np
+
+    def mix64(z):
+        z = z + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+    with np.errstate(over="ignore"):
+        h = mix64(np.uint64(key & (2**64 - 1)) ^ mix64(np.arange(len(logits_row), dtype=np.uint64)))
+    u = np.minimum(((h >> np.uint64(32)).astype(np.float64) + 0.5) / 2.0**32, 0.99999994)
+    return logits_row.astype(np.float64) / max(temperature, 1e-5) - np.log(-np.log(u))
+
+
 def test_static_sampling_matches_the_workspace_entry_point_twice_in_a_row():
     L = _lib()
     gen = torch.Generator().manual_seed(5)
@@ -52,6 +69,11 @@ def test_static_sampling_matches_the_workspace_entry_point_twice_in_a_row():
         assert torch.equal(got, want), (rows, vocab)
         greedy = [i for i in range(rows) if not tempered or i % 3 == 0]
         assert torch.equal(got[greedy].long(), logits.cpu().argmax(-1)[greedy])
+        if tempered:  # the tempered rows against the definition of the draw, worked out on the host
+            for i in [i for i in range(rows) if i % 3][:6]:
+                scores = host_scores(logits[i].cpu().numpy(), float(temps[i]), int(keys[i]))
+                assert scores[int(got[i])] >= scores.max() - 1e-4, (i, int(got[i]), int(scores.argmax()))
+                assert int(got[i]) != int(logits[i].argmax()) or scores.argmax() == int(got[i])
 
 
 def test_static_sampling_refuses_what_its_buffer_cannot_hold():
