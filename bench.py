@@ -8,8 +8,9 @@ the whole engine (schedule, step function from the cache, greedy sampling, postp
 line carries the 2,048-token prefill, the HBM roofline of the decode step, the host's phases of a
 step, the rates a probe kernel measures on this GPU, and under ``points``: decode at batch 1 and 64
 at that context, decode at batch 1/8/64 behind 2,048-token prompts with 256 generated tokens each,
-one float32 point, the reference's own two serving workloads, and the serving workloads of the 8B
-and 32B shapes. ``--shape 8b`` / ``--shape 32b`` print that shape's workload as a line of its own,
+decode at batch 8 behind 16,384 and 32,768 tokens, prompts of 8,192 and 32,704 tokens, one float32 point, the reference's
+own two serving workloads, the serving workloads of the 8B and 32B shapes, and decode steps (batch 1/8/64) and a prefill of
+the 1.7B, 8B and 32B shapes. ``--shape 8b`` / ``--shape 32b`` print that shape's workload as a line of its own,
 with its prefill and the roofline of its decode step.
 """
 
@@ -37,7 +38,12 @@ SHAPES = {
                tie_word_embeddings=False, max_position_embeddings=40960),
     "32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, intermediate_size=25600,
                 tie_word_embeddings=False, max_position_embeddings=40960),
+    # a shape between the measured ones (Qwen3-1.7B's layer sizes): its products fall between the thresholds of the kernel choice
+    "1.7b": dict(num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8, intermediate_size=6144,
+                 tie_word_embeddings=True, max_position_embeddings=40960),
 }
+SHAPE_NAMES = {"0.6b": "Qwen3-0.6B shape", "1.7b": "Qwen3-1.7B shape", "8b": "Qwen3-8B shape", "32b": "Qwen3-32B shape"}
+SHAPE_CONTEXT = {"1.7b": 2304, "8b": 2304, "32b": 640}  # near the context of the shape's serving workload
 
 
 def model_config(shape: str = "0.6b"):
@@ -289,20 +295,35 @@ def serving_workload(shape: str, dtype: str = "bfloat16") -> dict:
     return result
 
 
+def shape_points(shape: str, dtype: str, steps: int, warmup: int, prefill_tokens: int = 2048) -> dict:
+    """Decode steps at batch 64, 1 and 8 near the context of the shape's serving workload, and one prefill: what a
+    shape other than the headline's adds to a line. Returns the numbers of the batch-64 step beside the points."""
+    cfg = model_config(shape)
+    ctx = SHAPE_CONTEXT[shape]
+    bench = DecodeBench(cfg, dtype, max(ctx, prefill_tokens + 16), 64)
+    prefill = bench.prefill(prefill_tokens)
+
+    def decode(batch):  # the sequences reach `ctx` at the end of the timed steps, whatever the engine's limit is
+        return bench.decode(batch, steps, warmup, prompt_len=ctx - (steps + warmup + -(-batch * ctx // bench.budget) + 5))
+
+    tok_s, ms, gbs, _ = decode(64)
+    points, fracs = {"decode_b64": round(tok_s, 1)}, {"decode_b64": round(gbs / HBM_PEAK_GBS, 4)}
+    for b in (1, 8):
+        m = decode(b)
+        points[f"decode_b{b}"], fracs[f"decode_b{b}"] = round(m[0], 1), round(m[2] / HBM_PEAK_GBS, 4)
+    bench.engine = None
+    del bench
+    release()
+    return {"cfg": cfg, "ctx": ctx, "prefill": prefill, "ms": ms, "gbs": gbs, "points": points, "fracs": fracs}
+
+
 def shape_line(shape: str, args) -> dict:
     """The line of ``--shape 8b|32b``: the shape's serving workload as ``value``, plus the 2,048-token
     prefill and the HBM roofline of a decode step at batch 64 near that workload's context."""
-    cfg = model_config(shape)
     work = serving_workload(shape, args.dtype)
-    ctx = 2304 if shape == "8b" else 640
-    bench = DecodeBench(cfg, args.dtype, ctx, 64)
-    prefill = bench.prefill(min(args.prefill_tokens, ctx - 16))
-    tok_s, ms, gbs, _ = bench.decode(64, args.steps, args.warmup)
-    points, fracs = {"decode_b64": round(tok_s, 1)}, {"decode_b64": round(gbs / HBM_PEAK_GBS, 4)}
-    for b in (1, 8):
-        m = bench.decode(b, args.steps, args.warmup)
-        points[f"decode_b{b}"], fracs[f"decode_b{b}"] = round(m[0], 1), round(m[2] / HBM_PEAK_GBS, 4)
-    name = {"8b": "Qwen3-8B shape", "32b": "Qwen3-32B shape"}[shape]
+    sp = shape_points(shape, args.dtype, args.steps, args.warmup, args.prefill_tokens)
+    cfg, ctx, prefill, ms, gbs, points, fracs = (sp[k] for k in ("cfg", "ctx", "prefill", "ms", "gbs", "points", "fracs"))
+    name = SHAPE_NAMES[shape]
     what = {"8b": "64 requests, prompts uniform in [128, 2048], 128 output tokens, 8,192-token step budget",
             "32b": "64 requests of a shared 512-token prefix + 32 tokens, 64 output tokens, prefix cache warm"}[shape]
     return {
@@ -323,7 +344,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--shape", default="0.6b", choices=sorted(SHAPES))
+    ap.add_argument("--shape", default="0.6b", choices=["0.6b", "8b", "32b"])
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
@@ -369,6 +390,20 @@ def main() -> int:
             pts["shared_prefix_64x544in_64out"] = round(prefix, 1)
         bench.engine = None
         release()
+        # further contexts and prompt lengths of the headline shape: decode at batch 8 behind 16,384 and 32,768 tokens,
+        # whole prompts of 8,192 and 32,768 tokens
+        for ctx in (16384, 32768):
+            far = DecodeBench(cfg, args.dtype, ctx, args.batch)
+            m = far.decode(args.batch, 32, 4)
+            pts[f"decode_b{args.batch}_ctx{ctx}"] = round(m[0], 1)
+            pts_frac[f"decode_b{args.batch}_ctx{ctx}"] = round(m[2] / HBM_PEAK_GBS, 4)
+            if ctx == 32768:
+                for tokens in (8192, 32768 - 64):
+                    pf = far.prefill(tokens)
+                    pts[f"prefill_{tokens}_tok_s"], pts_frac[f"prefill_{tokens}"] = pf["value"], pf["frac"]
+            far.engine = None
+            del far
+            release()
         if args.dtype == "bfloat16":
             f32 = DecodeBench(cfg, "float32", args.context, args.batch)
             m = f32.decode(args.batch, 8, 2)
@@ -383,6 +418,15 @@ def main() -> int:
             pts[f"serving_{shape}_steps"] = work["steps"]
             pts[f"serving_{shape}_preemptions"] = work["preemptions"]
             pts[f"serving_{shape}_cached_tokens"] = work["cached_tokens"]
+        # the decode steps and the prefill of the other shapes (the in-between one, whose products fall between the
+        # thresholds of the kernel choice, and the two wide ones), near the contexts of their serving workloads
+        for shape in ("1.7b", "8b", "32b"):
+            sp = shape_points(shape, args.dtype, 32, 4, args.prefill_tokens)
+            for key, value in sp["points"].items():
+                pts[f"{key}_{shape}_ctx{sp['ctx']}"] = value
+                pts_frac[f"{key}_{shape}_ctx{sp['ctx']}"] = sp["fracs"][key]
+            pts[f"prefill_{sp['prefill']['tokens']}_{shape}_tok_s"] = sp["prefill"]["value"]
+            pts_frac[f"prefill_{sp['prefill']['tokens']}_{shape}"] = sp["prefill"]["frac"]
         extras["measured_peaks"] = measured_peaks()
     line = {
         "metric": f"decode tok/s at batch {args.batch} (Qwen3-0.6B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
