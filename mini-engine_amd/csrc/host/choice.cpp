@@ -65,7 +65,11 @@ bool streams(int m, int rows_of_w, int k) {
 // With each block's walk over k starting at a step of its own (what the kernel does for such k) the gated products stay ahead
 // up to 64 rows: 2 x 12,288 x 4,096 38-43 us against 48-50 at 17 to 64 rows, 2 x 14,336 x 4,096 45-48 against 58-65, 2 x 28,672
 // x 8,192 169-180 against 192-216; the plain 6,144 x 4,096 up to 32 (14.3 and 15.1 against 15.1 and 15.4; 19.4 against 17.6 at 64).
+// Plain products of weights between 16 and 32 MiB (the qkv of shapes between the narrow and the wide ones) stay with this
+// kernel up to 32 rows whatever their k: 4,096 x 2,048 at 24 and 32 rows 8.2 us against 9.3 and 9.4 from the library, 6,144 x
+// 2,560 10.5 and 11.3 against 11.6 and 11.9; from 48 rows on the two are level (9.6 and 9.4, 15.7 and 16.0).
 bool stream_serves_mid_rows(int m, int n, int k, bool gated, int units) {
+  if (!gated && m <= kStreamWholeRows && (int64_t)n * k < 2 * kStreamMinElements) return true;
   if (k % 2048 || m > (gated ? kSmallMaxRows : kStreamWholeRows)) return false;
   int plan[3] = {0, 0, 0};
   me_gemm_bf16_stream_plan(m, n, k, gated ? 1 : 0, 1, units, plan);

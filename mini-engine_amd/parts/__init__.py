@@ -2,6 +2,7 @@
 
 from . import attention, mlp, norm, rotary  # noqa: F401
 from .base import (
+    BLOCK_ARRANGEMENTS,
     FEED_FORWARDS,
     MIXERS,
     NORMS,
@@ -15,7 +16,7 @@ from .base import (
     StateBinding,
     StateNeed,
 )
-from .block import BLOCK_ARRANGEMENTS, PreNormBlock, build_block
+from .block import PreNormBlock, build_block
 from .decoder import Decoder
 
 __all__ = [

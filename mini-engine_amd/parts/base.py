@@ -134,17 +134,20 @@ class FeedForward(Part):
 
 
 class Registry:
-    def __init__(self, what: str):
-        self.what = what
+    """Kinds of one sort of part, by name. A spec names its kind in the attribute ``key`` (``kind`` for parts,
+    ``arrangement`` for the block that puts them together)."""
+
+    def __init__(self, what: str, key: str = "kind"):
+        self.what, self.key = what, key
         self._by_kind: dict[str, Callable[..., Part]] = {}
 
     def register(self, kind: str, factory: Callable[..., Part]) -> None:
         self._by_kind[kind] = factory
 
     def build(self, spec: Any, dtype: torch.dtype, device: torch.device) -> Part:
-        kind = getattr(spec, "kind", None)
+        kind = getattr(spec, self.key, None)
         if kind not in self._by_kind:
-            raise ValueError(f"no {self.what} registered for kind {kind!r}; known: {sorted(self._by_kind)}")
+            raise ValueError(f"no {self.what} registered for {self.key} {kind!r}; known: {sorted(self._by_kind)}")
         return self._by_kind[kind](spec, dtype, device)
 
     def kinds(self) -> list[str]:
@@ -155,3 +158,4 @@ MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
+BLOCK_ARRANGEMENTS = Registry("block arrangement", key="arrangement")

@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import kernels as K
-from .base import FEED_FORWARDS, MIXERS, NORMS
+from .base import BLOCK_ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS
 
 
 class PreNormBlock:
@@ -85,10 +85,8 @@ class PreNormBlock:
                     program.delta(out)
 
 
-BLOCK_ARRANGEMENTS = {"pre_norm": PreNormBlock}
+BLOCK_ARRANGEMENTS.register("pre_norm", PreNormBlock)
 
 
 def build_block(spec, dtype, device):
-    if spec.arrangement not in BLOCK_ARRANGEMENTS:
-        raise ValueError(f"unknown block arrangement {spec.arrangement!r}; known: {sorted(BLOCK_ARRANGEMENTS)}")
-    return BLOCK_ARRANGEMENTS[spec.arrangement](spec, dtype, device)
+    return BLOCK_ARRANGEMENTS.build(spec, dtype, device)
