@@ -120,7 +120,7 @@ class Run {
  public:
   Run(const Program& prog, const std::vector<Value>& values, const StepView& s, Arena& arena, int32_t* fed_tokens,
       hipStream_t stream)
-      : prog_(prog), s_(s), arena_(arena), fed_tokens_(fed_tokens), stream_(stream), dtype_(prog.dtype()),
+      : prog_(prog), values_(values), s_(s), arena_(arena), fed_tokens_(fed_tokens), stream_(stream), dtype_(prog.dtype()),
         elem_(prog.dtype() == kF32 ? 4 : 2), t_(s.lay.tokens), h_(prog.hidden()) {
     x_ = (float*)arena_.take((size_t)t_ * h_ * 4);
     spare_ = (float*)arena_.take((size_t)t_ * h_ * 4);
@@ -135,7 +135,7 @@ class Run {
       step(op);
       // the logits, the drawn tokens and partial sums that wait for the next norm outlive their operation;
       // an operation that used up waiting partial sums gives their memory back too
-      if (op.kind != kOpHead && op.kind != kOpSample && op.kind != kOpLinearDelta)
+      if (op.kind != kOpHead && op.kind != kOpHeadRows && op.kind != kOpSample && op.kind != kOpLinearDelta)
         arena_.used = released_to_ != (size_t)-1 ? released_to_ : mark;
     }
     return result_;
@@ -180,6 +180,18 @@ class Run {
         break;
       case kOpSample:
         sample();
+        break;
+      case kOpAdd:
+        if (pending_.any())
+          ok(me_residual_add(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, t_, h_, dtype_, stream_));
+        pending_ = Pending();
+        release_parts();
+        break;
+      case kOpCall:
+        call(op);
+        break;
+      case kOpHeadRows:
+        head_rows(op);
         break;
       default:
         throw Error(kBadValue, "unknown operation in a step program");
@@ -360,7 +372,7 @@ class Run {
 
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
   void head(const Op& op) {
-    const int rows = s_.lay.rows, vocab = prog_.vocab();
+    const int rows = s_.lay.rows;
     result_.rows = rows;
     if (rows == 0) {
       pending_ = Pending();
@@ -370,10 +382,40 @@ class Run {
     ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, (const float*)op.p[0], picked,
                       idx(s_.lay.want_rows), rows, h_, op.f[0], 0, dtype_, stream_));
     pending_ = Pending();
+    logits_of(picked, op);
+  }
+
+  // The head behind a final norm that a part computed itself: the value's first rows are the normed wanted rows.
+  void head_rows(const Op& op) {
+    result_.rows = s_.lay.rows;
+    if (s_.lay.rows == 0) return;
+    logits_of(bufs_[op.in], op);
+  }
+
+  void logits_of(const void* picked, const Op& op) {
+    const int rows = s_.lay.rows, vocab = prog_.vocab();
     float* logits = (float*)arena_.take((size_t)rows * vocab * 4);
     product(picked, op.p[1], vocab, h_, 0, kF32, logits, kRoleHead, rows);
     if (op.f[1] != 1.f) ok(me_scale_f32(logits, op.f[1], (long long)rows * vocab, stream_));
     result_.logits = logits;
+  }
+
+  // A part that brings its own code: it reads and writes values of the step and launches on the step's stream.
+  void call(const Op& op) {
+    CallFrame f{};
+    f.context = (void*)op.p[1];
+    f.in = op.in >= 0 ? bufs_[op.in] : nullptr;
+    f.out = op.out >= 0 ? bufs_[op.out] : nullptr;
+    f.x = x_;
+    f.in_cols = op.in >= 0 ? values_[op.in].cols : 0;
+    f.out_cols = op.out >= 0 ? values_[op.out].cols : 0;
+    f.in_elem = op.in >= 0 ? values_[op.in].elem : 0;
+    f.out_elem = op.out >= 0 ? values_[op.out].elem : 0;
+    f.tokens = t_;
+    f.rows = s_.lay.rows;
+    f.stream = stream_;
+    if (!op.p[0]) throw Error(kBadValue, "a called part needs its function");
+    if (((CallFn)op.p[0])(&f) != 0) throw Error(kBadState, "a part's own code failed in a step");
   }
 
   void sample() {
@@ -387,6 +429,7 @@ class Run {
   }
 
   const Program& prog_;
+  const std::vector<Value>& values_;
   const StepView& s_;
   Arena& arena_;
   int32_t* fed_tokens_;

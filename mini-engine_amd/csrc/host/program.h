@@ -33,7 +33,24 @@ enum OpKind {
   kOpHead = 7,        // p0 final norm weight, f0 eps, p1 head W [vocab, hidden], f1 the scale on the logits -> logits of the
                       // wanted rows
   kOpSample = 8,      // logits -> one token per wanted row
+  kOpAdd = 9,         // pending + x -> x, as a kernel of its own (before a norm that is no RMS norm)
+  kOpCall = 10,       // a part that brings its own code: p0 a function `int (const CallFrame*)`, p1 its context;
+                      // in (or -1), out (or -1): the values it reads and writes. It launches on the step's stream.
+  kOpHeadRows = 11,   // in: a value whose first rows are the normed wanted rows; p1 head W, f1 the scale on the logits
 };
+
+// What a called part is handed (kOpCall). Pointers are device memory of this step: they change from step to step.
+struct CallFrame {
+  void* context;
+  const void* in;   // [tokens, in_cols] or null
+  void* out;        // [tokens, out_cols] or null
+  float* x;         // the residual stream, float32 [tokens, hidden]
+  int64_t in_cols, out_cols;
+  int32_t in_elem, out_elem;  // bytes per element
+  int32_t tokens, rows;
+  hipStream_t stream;
+};
+typedef int (*CallFn)(const CallFrame*);
 
 struct Op {
   int kind = 0, in = -1, out = -1;

@@ -15,6 +15,8 @@ int me_embed_fed(void* x, const void* table, const int* ids, const int* fed_rows
 int me_scale_f32(float* x, float scale, long long count, hipStream_t stream);
 int me_add_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, const float* w,
                    void* h, const int* rows, int num_rows, int dim, float eps, int write_x, int dtype, hipStream_t stream);
+int me_residual_add(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, int num_rows, int dim,
+                    int dtype, hipStream_t stream);
 int me_rmsnorm(const void* in, const float* w, void* out, int num_rows, int dim, float eps, int dtype, hipStream_t stream);
 int me_swiglu(const void* gu, void* act, int num_tokens, int inter, int gate, int dtype, hipStream_t stream);
 int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table,

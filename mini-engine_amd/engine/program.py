@@ -1,11 +1,13 @@
 """Python face of the native step program (``csrc/host/program.cpp``, ``csrc/host/runner.cpp``).
 
-When a model is built, every part that can writes the operations of its forward pass into a
+When a model is built, every part writes the operations of its forward pass into a
 :class:`StepProgram` (a part's ``emit`` method; it says what the part computes, not which kernels
-run). A step of such a model then is one call into C++, which checks and packs the step that the
+run). A step of the model then is one call into C++, which checks and packs the step that the
 host core holds, uploads the indices, picks a kernel per operation for the step's size, launches
-them all and draws the next tokens. A model with a part that has no ``emit`` (a part defined
-outside the package, in Python) keeps the per-kernel path of :meth:`Decoder.forward`.
+them all and draws the next tokens. A part that has no ``emit`` (a part defined outside the package,
+with code of its own) enters the program as a *call*: the program hands its ``forward`` the step's
+values as tensors when the step reaches it, so such a part, with or without state of its own, runs in
+the same one pass as every other.
 
 Values are ``[tokens, columns]`` buffers of a step; parts get them from the program and the program
 hands a buffer out again once the scope that took it has ended, so a model of any depth needs the
@@ -16,6 +18,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import weakref
 
 import numpy as np
 import torch
@@ -25,8 +28,44 @@ from ..ops.library import lib
 _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
-EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE = range(9)
+EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS = range(12)
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
+
+
+class _RawFrame(ctypes.Structure):  # csrc/host/program.h: CallFrame
+    _fields_ = [("context", _vp), ("in_", _vp), ("out", _vp), ("x", _vp), ("in_cols", _i64), ("out_cols", _i64),
+                ("in_elem", _i32), ("out_elem", _i32), ("tokens", _i32), ("rows", _i32), ("stream", _vp)]
+
+
+_CALL_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.POINTER(_RawFrame))
+
+
+class Frame:
+    """What a called part sees of the step that has reached it: its input and output values and the residual
+    stream as tensors (views into the step's memory, valid during the call only) and the step's batch."""
+
+    def __init__(self, program: "StepProgram", raw: _RawFrame):
+        self.program, self.tokens, self.rows = program, int(raw.tokens), int(raw.rows)
+        dtype_of = {2: torch.bfloat16, 4: torch.float32}
+        arena = program.current_arena
+        self.input = view_in(arena, raw.in_, (self.tokens, int(raw.in_cols)), dtype_of[raw.in_elem]) if raw.in_ else None
+        self.output = view_in(arena, raw.out, (self.tokens, int(raw.out_cols)), dtype_of[raw.out_elem]) if raw.out else None
+        self.x = view_in(arena, raw.x, (self.tokens, program.hidden), torch.float32)
+
+    @property
+    def batch(self):
+        """The step's batch (:class:`~mini_engine_amd.engine.batch.StepBatch`), made once per step."""
+        return self.program.current_batch()
+
+    def write(self, result) -> None:
+        """A part's result into the output value: a tensor ``[tokens, columns]``, or partial sums over runs of k."""
+        from ..ops.kernels import PartialSums
+
+        if isinstance(result, PartialSums):
+            result = result.parts.sum(dim=0)
+        if tuple(result.shape) != tuple(self.output.shape):
+            raise ValueError(f"a part returned {tuple(result.shape)} where the step has {tuple(self.output.shape)}")
+        self.output.copy_(result)
 
 
 def _api():
@@ -78,6 +117,24 @@ class Normed:
         return self._value
 
 
+class CalledNorm:
+    """As :class:`Normed`, for a norm that is no RMS norm: the residual add as a kernel of its own, then the norm
+    part's ``forward`` on the residual stream. Parts get its value; nothing of it rides on their products."""
+
+    def __init__(self, program: "StepProgram", norm):
+        self.program, self.norm = program, norm
+        self.used = False
+        self._value: int | None = None
+
+    def value(self) -> int:
+        if self._value is None:
+            p, norm = self.program, self.norm
+            p.add()
+            self._value = p.call(lambda frame: frame.output.copy_(norm.forward(frame.x)), out_cols=p.hidden)
+            self.used = True
+        return self._value
+
+
 class StepProgram:
     def __init__(self, dtype: torch.dtype, hidden: int, vocab: int, max_positions: int):
         self._L = _api()
@@ -95,6 +152,12 @@ class StepProgram:
         self.num_ops = 0
         self.draws = False
         self.last_prefill_columns = 0  # query columns of the prefill attention's blocks in the last eager step (0: none ran)
+        # called parts: their C trampolines (kept alive), the memory and the batch of the step that is running,
+        # and the exception a call raised (raised again once the step's call into C++ has come back)
+        self._calls: list = []
+        self.current_arena: torch.Tensor | None = None
+        self.current_batch = lambda: None
+        self.call_error: BaseException | None = None
 
     def __del__(self):
         handle, self.handle = getattr(self, "handle", None), None
@@ -180,7 +243,7 @@ class StepProgram:
             x.used = True
             self.pending_consumed()
             return out
-        src = x.value() if isinstance(x, Normed) else x
+        src = x.value() if isinstance(x, (Normed, CalledNorm)) else x
         if self._value_kinds[src][0] != k:
             raise ValueError(f"the weight reads {k} columns, the value has {self._value_kinds[src][0]}")
         self.op(LINEAR, in_=src, out=out, ptrs=[None, weight], ints=[rows, k, gate])
@@ -221,6 +284,62 @@ class StepProgram:
                 ints=[heads, kv_heads, head_dim, rotary_dim, block_size, window, int(writes), group, covers],
                 floats=[eps, scale])
         return out
+
+    def add(self) -> None:
+        """The pending delta into the residual stream, as a kernel of its own (before a norm that is not RMS-shaped)."""
+        self.op(ADD)
+        self.pending_consumed()
+
+    def call(self, fn, in_: int = -1, out_cols: int | None = None, out_elem: int | None = None) -> int:
+        """A part with code of its own: when a step reaches this place, ``fn(frame)`` is called with a
+        :class:`Frame` (the value ``in_`` as ``frame.input``, a new value of ``out_cols`` columns as
+        ``frame.output``, the residual stream as ``frame.x``, the step's batch). It launches what it has to on the
+        current stream and returns nothing. Returns the output value (-1 without ``out_cols``)."""
+        out = self.take(out_cols, out_elem) if out_cols else -1
+        me = weakref.ref(self)  # (the program keeps the trampoline: no cycle through it)
+
+        def trampoline(raw):
+            program = me()
+            try:
+                fn(Frame(program, raw.contents))
+                return 0
+            except BaseException as e:  # an exception cannot cross the C frames in between: it is raised after the step
+                program.call_error = e
+                return 1
+
+        c_fn = _CALL_FN(trampoline)
+        self._calls.append(c_fn)
+        p = (ctypes.c_void_p * 6)()
+        p[0] = ctypes.cast(c_fn, ctypes.c_void_p).value
+        iv, fv = (ctypes.c_int64 * 10)(), (ctypes.c_float * 2)()
+        self.num_ops = _ok(self._L.me_runner_op(self.handle, CALL, in_, out, p, iv, fv))
+        return out
+
+    def call_part(self, part, h, extra=()) -> int:
+        """A mixer or feed-forward without ``emit``: its ``forward(h, batch, *extra)`` on the normed activations, its
+        result as a value ``[tokens, hidden]``."""
+        src = h.value()
+        return self.call(lambda frame: frame.write(part.forward(frame.input, frame.batch, *extra)), in_=src,
+                         out_cols=self.hidden)
+
+    def normed_by(self, norm) -> "CalledNorm":
+        """The add-and-norm before a part, for a norm part of any shape (its ``forward`` is called)."""
+        return CalledNorm(self, norm)
+
+    def head_by(self, norm, weight: torch.Tensor, logit_scale: float = 1.0) -> None:
+        """As :meth:`head`, for a final norm of any shape: the add, the norm part's ``forward`` on the wanted rows,
+        the head product."""
+        self._want(weight, self.dtype, (self.vocab, self.hidden), "head")
+        self.add()
+
+        def run(frame):
+            if frame.rows:
+                rows = frame.batch.want_rows[:frame.rows].long()
+                frame.output[:frame.rows].copy_(norm.forward(frame.x.index_select(0, rows)))
+
+        with self.scope():
+            picked = self.call(run, out_cols=self.hidden)
+            self.op(HEAD_ROWS, in_=picked, ptrs=[None, weight], floats=[0.0, logit_scale])
 
     def head(self, norm, weight: torch.Tensor, logit_scale: float = 1.0) -> None:
         """Final norm of the wanted rows, the head product, the logits times ``logit_scale``."""
@@ -281,11 +400,20 @@ def view_in(arena: torch.Tensor, address: int, shape: tuple[int, ...], dtype: to
     return arena[offset:offset + count].view(dtype).view(shape)
 
 
+def _after_calls(program: StepProgram, code: int) -> None:
+    """The step's call into C++ has come back: an exception that a called part raised on the way is raised now."""
+    error, program.call_error = program.call_error, None
+    if error is not None:
+        raise error
+    _ok(code)
+
+
 def run_step(program: StepProgram, memory: StepMemory, core) -> tuple[torch.Tensor | None, torch.Tensor | None, int]:
     """Run the step that ``core`` holds; (logits float32 [rows, vocab], drawn int32 [rows], rows)."""
     out = np.zeros(4, dtype=np.int64)
     stream = _vp(torch.cuda.current_stream().cuda_stream)
-    _ok(program._L.me_runner_step(program.handle, core._box, stream, _vp(out.ctypes.data)))
+    program.current_arena = memory.arena
+    _after_calls(program, program._L.me_runner_step(program.handle, core._box, stream, _vp(out.ctypes.data)))
     rows = int(out[1])
     program.last_prefill_columns = int(out[3])
     logits = view_in(memory.arena, int(out[0]), (rows, program.vocab), torch.float32) if out[0] else None
@@ -300,9 +428,11 @@ def run_static(program: StepProgram, arena: torch.Tensor, index: torch.Tensor, b
     out = np.zeros(4, dtype=np.int64)
     w = np.ascontiguousarray(widths, dtype=np.int32)
     stream = _vp(torch.cuda.current_stream().cuda_stream)
-    _ok(program._L.me_runner_static(program.handle, _vp(arena.data_ptr()), arena.numel(), _vp(index.data_ptr()), bucket,
-                                    _vp(w.ctypes.data), len(w), max_ctx, least_live,
-                                    _vp(None if drawn is None else drawn.data_ptr()), int(fed), stream, _vp(out.ctypes.data)))
+    program.current_arena = arena
+    _after_calls(program, program._L.me_runner_static(program.handle, _vp(arena.data_ptr()), arena.numel(), _vp(index.data_ptr()),
+                                                      bucket, _vp(w.ctypes.data), len(w), max_ctx, least_live,
+                                                      _vp(None if drawn is None else drawn.data_ptr()), int(fed), stream,
+                                                      _vp(out.ctypes.data)))
     logits = view_in(arena, int(out[0]), (bucket, program.vocab), torch.float32)
     tokens = drawn if drawn is not None else view_in(arena, int(out[2]), (bucket,), torch.int32)
     return logits, tokens

@@ -8,12 +8,15 @@ which every item is one decoded token can be replayed from a HIP graph captured 
 bucket (reference: ``src/mini_engine/cuda_graphs.py``): the graph reads its indices from one static
 buffer whose pinned source the core refills in place before each replay.
 
-A model whose parts all wrote their operations into a native step program runs a step as one call
-into C++ (check, pack, upload, every kernel, the draw of the next tokens); any other model runs
-:meth:`Decoder.forward`, one call per kernel, and draws with the sampler.
+Every model's forward pass is a native step program: a step is one call into C++ (check, pack, upload,
+every kernel, the draw of the next tokens), which calls back into a part's own ``forward`` where a part
+brings code of its own. (``native=False`` keeps the pass that launches kernel by kernel from Python,
+:meth:`Decoder.forward`, which the tests hold the program against.)
 """
 
 from __future__ import annotations
+
+import weakref
 
 import torch
 
@@ -27,6 +30,28 @@ from .core import HostCore, step_layout
 from .program import StepMemory, StepProgram, run_static, run_step
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+_capture_state_holder = None
+
+
+def _ordinary_capture_state(device) -> None:
+    """torch keeps the random generator's capture state in tensors that it makes at the first capture of a
+    process and updates in place at every later one, for as long as any graph lives. Steps run under inference
+    mode: made there, those tensors would refuse the update when someone captures a graph outside inference
+    mode while an engine's graphs are alive. A first small capture outside inference mode makes them ordinary
+    tensors, and its graph is kept so that they stay."""
+    global _capture_state_holder
+    if _capture_state_holder is None:
+        with torch.inference_mode(False):
+            cell = torch.zeros(1, device=device)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                cell += 1
+            torch.cuda.current_stream().wait_stream(side)
+        _capture_state_holder = (graph, cell)
 
 
 def batch_buckets(max_batch: int) -> list[int]:
@@ -56,12 +81,13 @@ class ModelRunner:
                              config.max_num_batched_tokens, config.max_model_len, eos_token_ids, config.seed)
         self.program: StepProgram | None = None
         self.memory: StepMemory | None = None
-        if native and not self.layout.has_state:
-            program = StepProgram(self.dtype, decoder.plan.hidden_size, decoder.plan.vocab_size, config.max_model_len)
-            if decoder.emit(program):
-                self.program = program
-                self.memory = StepMemory(program, self.device, [self.max_blocks_per_seq] * self.num_groups,
-                                         self.storage.spare_block, self.storage.spare_slot)
+        if native:
+            self.program = StepProgram(self.dtype, decoder.plan.hidden_size, decoder.plan.vocab_size, config.max_model_len)
+            decoder.emit(self.program)
+            batch_of_step = weakref.WeakMethod(self._batch_of_running_step)  # (no cycle: a dropped runner frees its graphs at once)
+            self.program.current_batch = lambda: batch_of_step()()
+            self.memory = StepMemory(self.program, self.device, [self.max_blocks_per_seq] * self.num_groups,
+                                     self.storage.spare_block, self.storage.spare_slot)
         self.sampler = Sampler()
         self.graph_safe = decoder.graph_safe()  # every part can be captured: decode steps may replay graphs
         self._graphs: dict[int, tuple] = {}
@@ -124,6 +150,10 @@ class ModelRunner:
             c = self.config
             self.memory.ensure(max(tokens, c.max_num_batched_tokens), max(items, c.max_num_seqs), max(rows, c.max_num_seqs),
                                max(ctx, c.max_model_len))
+            if self.layout.has_state:
+                core.step_check(self.decoder.plan.vocab_size, scan_pages=True)  # before anything is written
+                self._zero_fresh_state()
+            self.batch = None
             self._logits, self._drawn, _ = run_step(self.program, self.memory, core)
             if self._logits is None:
                 self._logits = torch.empty((0, self.decoder.plan.vocab_size), dtype=torch.float32, device=self.device)
@@ -133,6 +163,15 @@ class ModelRunner:
         self.batch = batch_from_core(core, self.device, self.storage.spare_block, self.storage.spare_slot)
         self._logits = self.decoder.forward(self.batch)
         return self._logits
+
+    def _batch_of_running_step(self) -> StepBatch:
+        """What a called part gets as the step's batch: views into the index buffer that the running step uploaded
+        (an eager step: made at the first call of the step) or the buffer a graph was captured on."""
+        if self.batch is None:
+            core, index = self.core, self.memory.index
+            _, starts, counts, _, slots = core.step_items()
+            self.batch = StepBatch(index, core.step_layout()).describe(starts, counts, slots)
+        return self.batch
 
     def _zero_fresh_state(self) -> None:
         """An item that starts at position 0 starts from a zero state, whoever held its slot before."""
@@ -160,10 +199,12 @@ class ModelRunner:
         """The launches of one decode step on a graph's static buffers: (logits, drawn or None)."""
         if self.program is None:
             return self.decoder.forward(batch), None
+        self.batch = batch  # what called parts see while the launches are recorded
         return run_static(self.program, self._static_arena, batch.buf, bucket, batch.widths, batch.max_ctx, batch.least_live,
                           drawn=self._fed, fed=True)
 
     def _capture(self, bucket: int):
+        _ordinary_capture_state(self.device)
         widths = [self.max_blocks_per_seq] * self.num_groups
         layout = step_layout(bucket, bucket, bucket, widths)
         host = torch.empty(layout["total"], dtype=torch.int32, pin_memory=True)

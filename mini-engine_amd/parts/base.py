@@ -17,6 +17,9 @@ A mixer or feed-forward class may set ``takes_normed_input = True``; its ``forwa
 to ``ops.kernels.linear`` as the input of its first matrix product, which fuses both into that
 product for decode-sized batches (``h.materialize()`` gives the tensor where it is needed).
 
+A part of the package also has ``emit(program, h, ...)``, which writes its operations into the step program that
+every step runs; a part without it enters that program as a call of its ``forward`` (``engine/program.py``).
+
 A part class that sets ``graph_safe = True`` promises that its ``forward`` can be captured into a graph for
 decode steps (see :class:`Part`); rows that pad a replayed batch carry the spare page and the spare state
 slot, which belong to no request.

@@ -69,16 +69,16 @@ class PreNormBlock:
 
 
     # ---- the native step program
-    def can_emit(self) -> bool:
-        """Whether every part of the block can write its operations into a step program."""
-        return (all(callable(getattr(p, "emit", None)) for p in (self.mixer, self.ffn))
-                and all(n.as_fused() is not None for n in (self.mixer_norm, self.ffn_norm)))
-
     def emit(self, program, cache=None) -> None:
+        """Write the block into a step program. A part with ``emit`` writes its own operations; any other part, and
+        any norm that is not RMS-shaped, enters as a call of its ``forward``."""
         for part, norm, extra in ((self.mixer, self.mixer_norm, (cache,)), (self.ffn, self.ffn_norm, ())):
             with program.scope():
-                h = program.normed(norm)
-                out = part.emit(program, h, *extra)
+                h = program.normed(norm) if norm.as_fused() is not None else program.normed_by(norm)
+                if callable(getattr(part, "emit", None)):
+                    out = part.emit(program, h, *extra)
+                else:
+                    out = program.call_part(part, h, extra)
                 if not h.used:  # the part never looked at its input: the add still has to happen
                     h.value()
                 if out is not None:

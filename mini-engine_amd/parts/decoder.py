@@ -93,20 +93,19 @@ class Decoder:
             x, spare, pending = self.blocks[i].forward(x, pending, batch, self.bindings[r], spare)
         return self.logits(x, pending, batch.want_rows)
 
-    def emit(self, program) -> bool:
-        """Write the model's forward pass and the draw of the next tokens into a native step program;
-        False (and nothing written) when a part cannot: a part without ``emit``, a norm that is not
-        RMS-shaped. The cache bindings have to be in place."""
+    def emit(self, program) -> None:
+        """Write the model's forward pass and the draw of the next tokens into a step program: what a step runs.
+        The cache bindings have to be in place."""
         if self.embed_table is None:
             raise RuntimeError("weights are not loaded")
-        if not all(self.blocks[i].can_emit() for i in set(self.plan.order)) or self.final_norm.as_fused() is None:
-            return False
         program.embed(self.embed_table, self.plan.embedding_multiplier or 1.0)
         for r, i in enumerate(self.plan.order):
             self.blocks[i].emit(program, self.bindings[r])
-        program.head(self.final_norm, self.head, self.plan.logit_scale or 1.0)
+        if self.final_norm.as_fused() is not None:
+            program.head(self.final_norm, self.head, self.plan.logit_scale or 1.0)
+        else:
+            program.head_by(self.final_norm, self.head, self.plan.logit_scale or 1.0)
         program.sample()
-        return True
 
     def logits(self, x: torch.Tensor, pending: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
         if rows.numel() == 0:

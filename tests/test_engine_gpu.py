@@ -450,3 +450,23 @@ def test_from_random_fills_every_tensor(tmp_path, name, dtype):
     th.assert_logits_close(got, want, dtype, f"from_random {name} {dtype}")
     if dtype == "float32":
         assert eng.generate([tokens[:9]], SamplingParams(max_tokens=6))[0] == plain.greedy_generate(w, pcfg, tokens[:9], 6)
+
+
+def test_someone_elses_graph_capture_beside_a_live_engine(peaked):
+    """An engine captures its decode graphs under inference mode; a capture that other code starts outside
+    inference mode while those graphs live must still work (torch updates the generator's capture state in place)."""
+    from mini_engine_amd import SamplingParams
+
+    eng = engine(peaked["A"][0], "A")
+    eng.generate(prompts_for("A", 3), SamplingParams(max_tokens=4))
+    assert eng.runner.graph_replays > 0
+    x = torch.zeros(4, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        x += 1
+    graph.replay()
+    torch.cuda.synchronize()
+    assert x.tolist() == [1.0] * 4  # (a capture records, it does not run)
+    assert eng.generate(prompts_for("A", 2), SamplingParams(max_tokens=3)) is not None

@@ -155,7 +155,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
     dec.load(Source())
     runner = ModelRunner(dec, EngineConfig(block_size=8, num_blocks=32, max_num_seqs=2, dtype="float32",
                                            max_model_len=128))
-    assert runner.layout.has_state and list(runner.layout.state_layers) == [0]
+    assert runner.layout.has_state and list(runner.layout.state_layers) == [0] and runner.program is not None
     bm = runner.new_block_manager()
     assert not bm.enable_prefix_caching  # state cannot be rebuilt from shared pages
 
@@ -461,7 +461,8 @@ def test_capturable_toy_parts_replay_from_graphs(graphs):
     dec.load(Source())
     runner = ModelRunner(dec, EngineConfig(block_size=8, num_blocks=32, max_num_seqs=3, dtype="float32", max_model_len=128,
                                            cuda_graphs=graphs))
-    assert runner.layout.has_state and runner.graph_safe and runner.program is None
+    # the model steps through the native program like any other: its own parts are calls in it
+    assert runner.layout.has_state and runner.graph_safe and runner.program is not None
     bm = runner.new_block_manager()
     g = torch.Generator().manual_seed(4)
     reqs = {k: torch.randint(0, 97, (n,), generator=g).tolist() for k, n in (("a", 20), ("b", 9), ("c", 7))}
