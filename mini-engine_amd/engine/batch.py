@@ -12,7 +12,6 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any
 
-import numpy as np
 import torch
 
 
@@ -72,12 +71,3 @@ class StepBatch:
         self.max_ctx = max(s + q for s, q in zip(starts, qlens))
         self.decode_only = self.max_qlen == 1
         return self
-
-
-def batch_from_core(core, device, spare_block: int = 0, spare_slot: int = 0) -> StepBatch:
-    """Pack the core's current step and upload it: the batch an eager step runs on."""
-    layout = core.step_layout()
-    arr = np.empty(layout["total"], dtype=np.int32)
-    core.step_pack(arr, None, 0, spare_block, spare_slot)
-    _, starts, counts, _, slots = core.step_items()
-    return StepBatch(torch.from_numpy(arr).to(device), layout).describe(starts, counts, slots)

@@ -10,8 +10,7 @@ buffer whose pinned source the core refills in place before each replay.
 
 Every model's forward pass is a native step program: a step is one call into C++ (check, pack, upload,
 every kernel, the draw of the next tokens), which calls back into a part's own ``forward`` where a part
-brings code of its own. (``native=False`` keeps the pass that launches kernel by kernel from Python,
-:meth:`Decoder.forward`, which the tests hold the program against.)
+brings code of its own.
 """
 
 from __future__ import annotations
@@ -25,7 +24,7 @@ from ..cache.storage import CacheStorage, plan_layout
 from ..config.engine_config import EngineConfig
 from ..parts.decoder import Decoder
 from ..sampling.sampler import Sampler
-from .batch import StepBatch, StepItem, batch_from_core
+from .batch import StepBatch, StepItem
 from .core import HostCore, step_layout
 from .program import StepMemory, StepProgram, run_static, run_step
 
@@ -63,7 +62,7 @@ def batch_buckets(max_batch: int) -> list[int]:
 
 
 class ModelRunner:
-    def __init__(self, decoder: Decoder, config: EngineConfig, eos_token_ids=(), native: bool = True):
+    def __init__(self, decoder: Decoder, config: EngineConfig, eos_token_ids=()):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible: this engine runs on the GPU only")
         self.decoder, self.config = decoder, config
@@ -79,22 +78,19 @@ class ModelRunner:
         self.core = HostCore(config.block_size, [(g.window, g.num_blocks or config.num_blocks) for g in self.layout.groups],
                              config.enable_prefix_caching, self.num_state_slots, self.layout.has_state, config.max_num_seqs,
                              config.max_num_batched_tokens, config.max_model_len, eos_token_ids, config.seed)
-        self.program: StepProgram | None = None
-        self.memory: StepMemory | None = None
-        if native:
-            self.program = StepProgram(self.dtype, decoder.plan.hidden_size, decoder.plan.vocab_size, config.max_model_len)
-            decoder.emit(self.program)
-            batch_of_step = weakref.WeakMethod(self._batch_of_running_step)  # (no cycle: a dropped runner frees its graphs at once)
-            self.program.current_batch = lambda: batch_of_step()()
-            self.memory = StepMemory(self.program, self.device, [self.max_blocks_per_seq] * self.num_groups,
-                                     self.storage.spare_block, self.storage.spare_slot)
+        self.program = StepProgram(self.dtype, decoder.plan.hidden_size, decoder.plan.vocab_size, config.max_model_len)
+        decoder.emit(self.program)
+        batch_of_step = weakref.WeakMethod(self._batch_of_running_step)  # (no cycle: a dropped runner frees its graphs at once)
+        self.program.current_batch = lambda: batch_of_step()()
+        self.memory = StepMemory(self.program, self.device, [self.max_blocks_per_seq] * self.num_groups,
+                                 self.storage.spare_block, self.storage.spare_slot)
         self.sampler = Sampler()
         self.graph_safe = decoder.graph_safe()  # every part can be captured: decode steps may replay graphs
         self._graphs: dict[int, tuple] = {}
         self._graph_pool = None
         self._static_arena: torch.Tensor | None = None
         self._copy_done: dict[int, torch.cuda.Event] = {}
-        self.batch: StepBatch | None = None  # the batch of the last step on the per-kernel path
+        self.batch: StepBatch | None = None  # the running step's batch, for parts that are called (made when first asked for)
         self._logits: torch.Tensor | None = None
         self._drawn: torch.Tensor | None = None  # what the native program drew for the last step's rows
         # Replayed steps of a native program draw into one buffer on the device, from which the next replay may
@@ -146,23 +142,22 @@ class ModelRunner:
             self._zero_fresh_state()
             return self._replay(items)
         self.eager_steps += 1
-        if self.program is not None:  # one call: check, pack, upload, every kernel, the draw
-            c = self.config
-            self.memory.ensure(max(tokens, c.max_num_batched_tokens), max(items, c.max_num_seqs), max(rows, c.max_num_seqs),
-                               max(ctx, c.max_model_len))
-            if self.layout.has_state:
-                core.step_check(self.decoder.plan.vocab_size, scan_pages=True)  # before anything is written
-                self._zero_fresh_state()
-            self.batch = None
-            self._logits, self._drawn, _ = run_step(self.program, self.memory, core)
-            if self._logits is None:
-                self._logits = torch.empty((0, self.decoder.plan.vocab_size), dtype=torch.float32, device=self.device)
-            return self._logits
-        core.step_check(self.decoder.plan.vocab_size, scan_pages=True)
-        self._zero_fresh_state()
-        self.batch = batch_from_core(core, self.device, self.storage.spare_block, self.storage.spare_slot)
-        self._logits = self.decoder.forward(self.batch)
+        self._logits = self._run_eager(tokens, items, rows, ctx)
         return self._logits
+
+    def _run_eager(self, tokens: int, items: int, rows: int, ctx: int) -> torch.Tensor:
+        """The step that the core holds as one call: check, pack, upload, every kernel, the draw."""
+        core, c = self.core, self.config
+        self.memory.ensure(max(tokens, c.max_num_batched_tokens), max(items, c.max_num_seqs), max(rows, c.max_num_seqs),
+                           max(ctx, c.max_model_len))
+        if self.layout.has_state:
+            core.step_check(self.decoder.plan.vocab_size, scan_pages=True)  # before anything is written
+            self._zero_fresh_state()
+        self.batch = None
+        logits, self._drawn, _ = run_step(self.program, self.memory, core)
+        if logits is None:
+            logits = torch.empty((0, self.decoder.plan.vocab_size), dtype=torch.float32, device=self.device)
+        return logits
 
     def _batch_of_running_step(self) -> StepBatch:
         """What a called part gets as the step's batch: views into the index buffer that the running step uploaded
@@ -180,9 +175,9 @@ class ModelRunner:
             self.storage.zero_state([s for s, p0 in zip(slots, starts) if p0 == 0 and s >= 0])
 
     def draw(self, rows: int, tempered: bool, replay: int | None = None):
-        """One token id per wanted row of a step (int32, on the host): what the native program drew
-        beside the logits, or the sampler's draw from them. ``replay`` names the pinned buffer of a
-        replayed step (``last_replay`` right after it was launched); without it the last step is meant."""
+        """One token id per wanted row of a step (int32, on the host): what the step program drew beside the
+        logits (a step without a draw of its own: the sampler's draw from them). ``replay`` names the pinned buffer
+        of a replayed step (``last_replay`` right after it was launched); without it the last step is meant."""
         if rows == 0:
             return self.sampler.draw(None, None, 0, False)
         if replay is None:
@@ -197,8 +192,6 @@ class ModelRunner:
     # ---------------------------------------------------------------------------------- graphs
     def _forward_static(self, batch: StepBatch, bucket: int):
         """The launches of one decode step on a graph's static buffers: (logits, drawn or None)."""
-        if self.program is None:
-            return self.decoder.forward(batch), None
         self.batch = batch  # what called parts see while the launches are recorded
         return run_static(self.program, self._static_arena, batch.buf, bucket, batch.widths, batch.max_ctx, batch.least_live,
                           drawn=self._fed, fed=True)
@@ -215,7 +208,7 @@ class ModelRunner:
         batch.max_ctx = self.config.max_model_len
         smaller = [b for b in batch_buckets(self.config.max_num_seqs) if b < bucket]
         batch.least_live = smaller[-1] + 1 if smaller else 1  # fewer items replay a smaller bucket's graph
-        if self.program is not None and self._static_arena is None:
+        if self._static_arena is None:
             most = self.config.max_num_seqs  # every bucket's graph works in the same memory: replays are serial
             self._static_arena = torch.empty(self.program.arena_need(most, most, most, self.config.max_model_len),
                                              dtype=torch.uint8, device=self.device)

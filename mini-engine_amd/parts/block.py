@@ -13,7 +13,6 @@ from __future__ import annotations
 
 import torch
 
-from ..ops import kernels as K
 from .base import BLOCK_ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS
 
 
@@ -40,33 +39,6 @@ class PreNormBlock:
         self.mixer.load(tensors, s.mixer_prefix)
         self.ffn_norm.load(tensors, s.ffn_norm_name)
         self.ffn.load(tensors, s.ffn_prefix)
-
-    def forward(self, x: torch.Tensor, pending: torch.Tensor | None, batch, cache=None, spare: torch.Tensor | None = None):
-        """``x`` float32 [T, H] is the residual stream, ``pending`` the previous block's output that
-        still has to be added, ``cache`` the binding of this run of the layer, ``spare`` a second
-        float32 buffer of x's shape. Returns ``(x, spare, pending)``: the buffer that now holds the
-        residual stream, the other one, and this block's own pending output.
-
-        A part whose class sets ``takes_normed_input`` is handed the add-and-norm unevaluated
-        (:class:`~mini_engine_amd.ops.kernels.NormedInput`) and may fuse it into its first matrix
-        product; any other part gets the normed activations."""
-        x, spare, a = self._run(self.mixer, self.mixer_norm, x, pending, spare, batch, (cache,))
-        return self._run(self.ffn, self.ffn_norm, x, a, spare, batch, ())
-
-    def _run(self, part, norm, x, pending, spare, batch, extra):
-        fused = norm.as_fused()
-        if fused is None:  # any other norm: the add as a kernel of its own, then the part
-            if pending is not None:
-                K.residual_add(x, pending)
-            return x, spare, part.forward(norm.forward(x), batch, *extra)
-        h = K.NormedInput(x, pending, fused[0], fused[1], self.dtype, spare)
-        out = part.forward(h if getattr(part, "takes_normed_input", False) else h.materialize(), batch, *extra)
-        if h.residual is None:  # the part never looked at its input: the add still has to happen
-            h.materialize()
-        if h.residual is not x:
-            x, spare = h.residual, x
-        return x, spare, out
-
 
     # ---- the native step program
     def emit(self, program, cache=None) -> None:

@@ -11,7 +11,6 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelPlan
-from ..ops import kernels as K
 from ..weights.loader import TensorWant, load_tensors
 from .base import NORMS
 from .block import build_block
@@ -81,18 +80,6 @@ class Decoder:
         return total
 
     # ---- step
-    def forward(self, batch) -> torch.Tensor:
-        """Run the batch's tokens through every layer of ``plan.order``; logits float32 [R, V] for
-        ``batch.want_rows``."""
-        if self.embed_table is None:
-            raise RuntimeError("weights are not loaded")
-        x = K.embed(batch.token_ids, self.embed_table, multiplier=self.plan.embedding_multiplier or 1.0)
-        spare = torch.empty_like(x)  # the residual stream alternates between two buffers
-        pending = None
-        for r, i in enumerate(self.plan.order):
-            x, spare, pending = self.blocks[i].forward(x, pending, batch, self.bindings[r], spare)
-        return self.logits(x, pending, batch.want_rows)
-
     def emit(self, program) -> None:
         """Write the model's forward pass and the draw of the next tokens into a step program: what a step runs.
         The cache bindings have to be in place."""
@@ -106,21 +93,6 @@ class Decoder:
         else:
             program.head_by(self.final_norm, self.head, self.plan.logit_scale or 1.0)
         program.sample()
-
-    def logits(self, x: torch.Tensor, pending: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
-        if rows.numel() == 0:
-            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
-        fused = self.final_norm.as_fused()
-        if fused is not None:
-            h = K.add_rmsnorm(x, pending, fused[0], fused[1], self.dtype, rows=rows, write_x=False)
-        else:
-            if pending is not None:
-                K.residual_add(x, pending)
-            h = self.final_norm.forward(x.index_select(0, rows.long()))
-        logits = K.linear(h, self.head, torch.float32, head=True)
-        if self.plan.logit_scale not in (None, 1.0):
-            K.scale_(logits, self.plan.logit_scale)
-        return logits
 
     def graph_safe(self) -> bool:
         """Whether a decode step of this model may be captured into a graph: every part says so

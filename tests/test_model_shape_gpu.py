@@ -49,18 +49,17 @@ def steps_for(reqs):
 
 @pytest.mark.parametrize("path", ["replayed", "eager", "per kernel"])
 def test_benchmark_layer_sizes_against_plain(model, path):
-    """The native step program, replayed and eager, and the per-kernel path that models with parts of their own take."""
+    """The step program, replayed and eager, and the same parts launched kernel by kernel from Python."""
     from types import SimpleNamespace
 
-    from mini_engine_amd.engine.runner import ModelRunner
+    from kernel_by_kernel import KernelByKernelRunner
     from mini_engine_amd.engine.trace import TraceSession, build_session
 
     folder, reqs, want = model
     steps = steps_for(reqs)
     engine = build_session(folder, "bfloat16", 4096, block_size=16, max_live=32, cuda_graphs=path == "replayed")
     if path == "per kernel":
-        runner = ModelRunner(engine.model, engine.config, native=False)
-        assert runner.program is None
+        runner = KernelByKernelRunner(engine.model, engine.config)
         engine = SimpleNamespace(runner=runner, core=runner.core, block_manager=runner.new_block_manager())
     session = TraceSession(engine)
     got = th.collect(steps, th.replay_in_process(session, steps))

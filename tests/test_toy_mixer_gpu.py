@@ -430,13 +430,15 @@ def plain_capturable(w, tokens):
     return 0.25 * (centered(x, "toy.norm") @ w["toy.head"].T)
 
 
+@pytest.mark.parametrize("kernel_by_kernel", [False, True])
 @pytest.mark.parametrize("graphs", [True, False])
-def test_capturable_toy_parts_replay_from_graphs(graphs):
+def test_capturable_toy_parts_replay_from_graphs(graphs, kernel_by_kernel):
     """A model of toy parts that say they can be captured: a mixer with state, a routed
     feed-forward, a norm with mean subtraction and bias (before a mixer, before a feed-forward and as
     the final norm), an embedding multiplier and a logit scale. Decode steps replay a graph; rows that
     pad the batch write the spare state slot; a request whose one-token prompt arrives in a decode
-    step starts from a zero state in a slot that another request has used."""
+    step starts from a zero state in a slot that another request has used. The parts run as calls inside
+    the engine's step program; the same parts launched kernel by kernel from Python give the same."""
     from mini_engine_amd import EngineConfig
     from mini_engine_amd.engine.batch import StepItem
     from mini_engine_amd.engine.runner import ModelRunner
@@ -459,6 +461,8 @@ def test_capturable_toy_parts_replay_from_graphs(graphs):
             return weights[n]
 
     dec.load(Source())
+    if kernel_by_kernel:
+        from kernel_by_kernel import KernelByKernelRunner as ModelRunner  # noqa: F811
     runner = ModelRunner(dec, EngineConfig(block_size=8, num_blocks=32, max_num_seqs=3, dtype="float32", max_model_len=128,
                                            cuda_graphs=graphs))
     # the model steps through the native program like any other: its own parts are calls in it

@@ -50,11 +50,11 @@ def steps_for(reqs):
 
 @pytest.mark.parametrize("path", ["replayed", "eager", "per kernel"])
 def test_wide_layers_against_plain(model, path):
-    """The native step program, replayed and eager, and the per-kernel path of models with parts of their own, whose
-    choice of kernel per product (``ops/kernels.py::linear``) mirrors the native one."""
+    """The step program, replayed and eager, and the same parts launched kernel by kernel from Python, whose products
+    (``ops/kernels.py::linear``) ask the same rule for their kernel."""
     from types import SimpleNamespace
 
-    from mini_engine_amd.engine.runner import ModelRunner
+    from kernel_by_kernel import KernelByKernelRunner
     from mini_engine_amd.engine.trace import TraceSession, build_session
     from mini_engine_amd.ops import kernels as K
 
@@ -71,8 +71,7 @@ def test_wide_layers_against_plain(model, path):
     steps = steps_for(reqs)
     engine = build_session(folder, "bfloat16", 64 * 40, block_size=16, max_live=40, cuda_graphs=path == "replayed")
     if path == "per kernel":
-        runner = ModelRunner(engine.model, engine.config, native=False)
-        assert runner.program is None
+        runner = KernelByKernelRunner(engine.model, engine.config)
         engine = SimpleNamespace(runner=runner, core=runner.core, block_manager=runner.new_block_manager())
     else:
         assert engine.runner.program is not None
