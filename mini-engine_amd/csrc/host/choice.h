@@ -1,5 +1,5 @@
 // Which kernel serves a matrix product of a step: the one table of thresholds in the tree. The native step program
-// (program.cpp) and the per-kernel Python path (ops/kernels.py::linear, through me_product_choice) both ask here, so
+// (program.cpp) and the Python entry point of the products (ops/kernels.py::linear, through me_product_choice) both ask here, so
 // the two cannot choose differently. Pure host code: sizes in, a kernel's code out.
 #pragma once
 
