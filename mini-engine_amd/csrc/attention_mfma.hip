@@ -159,7 +159,11 @@ struct DecodeFusedArgs {
   bf16_t* v_cache_w;
 };
 
-#define LONG_RUN 16  // tiles of a split from which on a wave fetches one tile at a time
+// Tiles of a split from which on a wave fetches one tile at a time, whatever DEPTH says: with five tiles and more of its own
+// a wave streams best without a tile requested ahead, since the other waves of its SIMD fill the gaps (measured with 16, 12,
+// 8, 4 and 1 here: batch 8 at contexts of 4,096 / 2,304 1.881 / 1.526 ms a step with 16, 1.851 / 1.505 with 4; batch 16 at
+// 1,024 1.538 -> 1.512; batch 64 at 512 2.047 -> 2.031; with 1, splits of two tiles lose: batch 1 1.040 -> 1.079).
+#define LONG_RUN 4
 
 // Most splits that one block takes on, a wave each. Heads beyond 128 need more than 256 registers a lane
 // with two tiles in flight, which only blocks of at most four waves (one per SIMD) may have.
