@@ -78,8 +78,8 @@ void destroy_plan(LibraryPlan& p) {
 // X [M, K] and W [N, K] bfloat16, C [M, N] bfloat16 or float32 (out_dtype), all contiguous. The first call
 // creates the library's handle and a workspace of 256 MB that lives as long as the process; the first call
 // for a shape must not come while a graph is being captured (it may load code), later ones may.
-extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype,
-                                    hipStream_t stream) {
+static int library_product(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype, bool accumulate,
+                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return me_fail("me_gemm_bf16_library: K=%d", K);
   if (!X || !W || !C) return me_fail("me_gemm_bf16_library: null operand");
@@ -116,9 +116,19 @@ extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M
     }
     plan = it->second;
   }
-  const float alpha = 1.f, beta = 0.f;
+  const float alpha = 1.f, beta = accumulate ? 1.f : 0.f;
   const hipblasStatus_t st = hipblasLtMatmul(g_handle, plan.desc, &alpha, W, plan.a, X, plan.b, &beta, C, plan.c, C, plan.c,
                                              &plan.algo, g_workspace, WORKSPACE_BYTES, stream);
   if (st != HIPBLAS_STATUS_SUCCESS) return me_fail("me_gemm_bf16_library: the product failed with status %d", (int)st);
   return 0;
+}
+
+extern "C" int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype,
+                                    hipStream_t stream) {
+  return library_product(X, W, C, M, N, K, out_dtype, false, stream);
+}
+
+// C[M, N] (float32) += X . W^T: the product added to what C holds, in the library's epilogue (a float32 sum per element).
+extern "C" int me_gemm_bf16_library_add(const void* X, const void* W, float* C, int M, int N, int K, hipStream_t stream) {
+  return library_product(X, W, C, M, N, K, ME_F32, true, stream);
 }

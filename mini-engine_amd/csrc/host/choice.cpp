@@ -89,7 +89,7 @@ ProductChoice choose_product(int dtype, int role, int m, int rows_of_w, int k, i
     return c;
   }
   const bool own = aligned && k % 8 == 0;  // what every kernel of this folder but the library's stand-ins needs
-  if (role == kRoleDelta && !gated) {
+  if ((role == kRoleDelta || role == kRoleDeltaInto) && !gated) {
     c.partial_sums = true;
     if (own && streams(m, rows_of_w, k)) {
       // float32 partial sums over runs of k (one run for short k): the next add-and-norm adds them up, and the delta is
@@ -98,7 +98,14 @@ ProductChoice choose_product(int dtype, int role, int m, int rows_of_w, int k, i
       c.runs = me_gemm_bf16_stream_splits(m, n, k, units);
       return c;
     }
-    c.kernel = kProductLibrary;  // more rows: the library's product with a float32 result, which stands as one partial sum
+    // More rows: the library's product with a float32 result. Where the caller can, the library adds it into the
+    // residual stream in its own epilogue (x += product, a float32 sum per element), so that the norm behind reads
+    // the stream alone and writes no new stream; else the result stands as one partial sum.
+    c.kernel = kProductLibrary;
+    if (role == kRoleDeltaInto && aligned && k % 8 == 0) {
+      c.partial_sums = false;
+      c.adds_into = true;
+    }
     return c;
   }
   if (role == kRoleHead) {
@@ -147,7 +154,7 @@ int choose_norm_fusion(int dtype, int m, int rows_of_w, int k, int pending, int 
 
 }  // namespace me
 
-// out: kernel, runs, partial_sums, gate_after
+// out: kernel, runs, partial_sums, gate_after, adds_into
 extern "C" void me_product_choice(int dtype, int role, int m, int rows_of_w, int k, int gated, int out_dtype, int units,
                                   int aligned, int* out) {
   const me::ProductChoice c = me::choose_product(dtype, role, m, rows_of_w, k, gated, out_dtype, units, aligned != 0);
@@ -155,6 +162,7 @@ extern "C" void me_product_choice(int dtype, int role, int m, int rows_of_w, int
   out[1] = c.runs;
   out[2] = c.partial_sums ? 1 : 0;
   out[3] = c.gate_after ? 1 : 0;
+  out[4] = c.adds_into ? 1 : 0;
 }
 
 extern "C" int me_norm_fusion_choice(int dtype, int m, int rows_of_w, int k, int pending, int units, int aligned) {

@@ -19,6 +19,7 @@ enum ProductRole {
   kRolePlain = 0,  // a projection inside a part
   kRoleDelta = 1,  // a product whose result only ever is the pending delta of the residual stream
   kRoleHead = 2,   // the logits of the wanted rows (float32 results)
+  kRoleDeltaInto = 3,  // as kRoleDelta, by a caller that can let the product add its result into the residual stream itself
 };
 
 struct ProductChoice {
@@ -26,6 +27,7 @@ struct ProductChoice {
   int runs = 1;             // runs of k whose float32 partial sums the next add-and-norm adds up (deltas only)
   bool partial_sums = false;  // the result is float32 [runs, m, n] whatever the model's dtype
   bool gate_after = false;    // the gate is a kernel of its own behind the product
+  bool adds_into = false;     // the product adds its result into the float32 residual stream (kRoleDeltaInto only)
 };
 
 enum NormFusion {

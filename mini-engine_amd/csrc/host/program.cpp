@@ -90,6 +90,19 @@ void library_product(const void* x, const void* w, void* out, int m, int n, int 
   ok(me_gemm_plain(x, w, out, m, n, k, kBF16, out_dtype, stream));
 }
 
+// x += a . w^T through the library; false (and nothing done) for sizes it has no algorithm for.
+bool library_adds(const void* a, const void* w, float* x, int m, int n, int k, hipStream_t stream) {
+  const auto shape = std::make_tuple(n, k, kF32);
+  {
+    std::lock_guard<std::mutex> hold(g_refused_mutex);
+    if (g_refused.count(shape)) return false;
+  }
+  if (me_gemm_bf16_library_add(a, w, x, m, n, k, stream) == 0) return true;
+  std::lock_guard<std::mutex> hold(g_refused_mutex);
+  g_refused.insert(shape);
+  return false;
+}
+
 // (keys per split, number of splits) of a decode launch: enough waves to fill the chip, splits of at least 64
 // keys, boundaries at multiples of 64.
 void decode_splits(int items, int kv_units, int max_ctx, int& split_keys, int& num_splits) {
@@ -283,7 +296,18 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
-    const ProductChoice c = choose_product(dtype_, kRoleDelta, t_, n, k, 0, dtype_, compute_units(), true);
+    const ProductChoice c = choose_product(dtype_, kRoleDeltaInto, t_, n, k, 0, dtype_, compute_units(), true);
+    if (c.adds_into) {  // x += product, in the library's epilogue: nothing stays pending
+      if (library_adds(x, op.p[1], x_, t_, n, k, stream_)) return;
+      // (a size the library has no algorithm for: the product as one partial sum, through this folder's kernels)
+      parts_mark_ = arena_.used;
+      float* sum = (float*)arena_.take((size_t)t_ * n * 4);
+      library_product(x, op.p[1], sum, t_, n, k, kF32, stream_);
+      pending_.parts = sum;
+      pending_.num_parts = 1;
+      pending_.stride = (long long)t_ * n;
+      return;
+    }
     if (c.partial_sums) {  // float32 sums over runs of k (or one whole sum) that wait for the next add-and-norm
       parts_mark_ = arena_.used;
       float* parts = (float*)arena_.take((size_t)c.runs * t_ * n * 4);

@@ -60,6 +60,7 @@ int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, const float* 
 int me_gemm_bf16_tiled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype, int shape,
                        hipStream_t stream);
 int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype, hipStream_t stream);
+int me_gemm_bf16_library_add(const void* X, const void* W, float* C, int M, int N, int K, hipStream_t stream);
 int me_sample_chunks(int vocab);
 int me_sample(const float* logits, int num_rows, int vocab, const float* temperatures, const uint64_t* keys, int* out,
               void* workspace, hipStream_t stream);

@@ -396,7 +396,7 @@ def product_choice(dtype: torch.dtype, role: int, rows: int, rows_of_w: int, k: 
                    units: int, aligned: bool = True) -> tuple[int, int, bool, bool]:
     """Which kernel serves a product: (kernel, runs of k, the result is float32 partial sums, the gate is a kernel of
     its own behind the product). The one rule of the tree, in ``csrc/host/choice.cpp``; no GPU is touched."""
-    out = (ctypes.c_int * 4)()
+    out = (ctypes.c_int * 5)()
     lib().me_product_choice(_i(_code(dtype)), _i(role), _i(rows), _i(rows_of_w), _i(k), _i(int(bool(gated))), _i(_code(out_dtype)),
                             _i(units), _i(int(aligned)), out)
     return int(out[0]), int(out[1]), bool(out[2]), bool(out[3])
