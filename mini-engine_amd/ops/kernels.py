@@ -389,7 +389,7 @@ class NormedInput:
 
 NORM_ALONE, NORM_IN_STREAM, NORM_IN_SMALL = 0, 1, 2  # csrc/host/choice.h: NormFusion
 PRODUCT_F32, PRODUCT_SMALL, PRODUCT_STREAM, PRODUCT_TILED, PRODUCT_LIBRARY = range(5)  # csrc/host/choice.h: ProductKernel
-ROLE_PLAIN, ROLE_DELTA, ROLE_HEAD = range(3)  # csrc/host/choice.h: ProductRole
+ROLE_PLAIN, ROLE_DELTA, ROLE_HEAD, ROLE_DELTA_INTO = range(4)  # csrc/host/choice.h: ProductRole
 
 
 def product_choice(dtype: torch.dtype, role: int, rows: int, rows_of_w: int, k: int, gated: bool, out_dtype: torch.dtype,
@@ -400,6 +400,16 @@ def product_choice(dtype: torch.dtype, role: int, rows: int, rows_of_w: int, k: 
     lib().me_product_choice(_i(_code(dtype)), _i(role), _i(rows), _i(rows_of_w), _i(k), _i(int(bool(gated))), _i(_code(out_dtype)),
                             _i(units), _i(int(aligned)), out)
     return int(out[0]), int(out[1]), bool(out[2]), bool(out[3])
+
+
+def delta_choice(rows: int, rows_of_w: int, k: int, units: int, aligned: bool = True) -> tuple[int, int, bool, bool]:
+    """How the step program takes a bfloat16 product that is a delta of the float32 residual stream and may be added
+    into it: (kernel, runs of k, the result is float32 partial sums, the kernel adds its product into the stream
+    itself). Exactly one of the last two holds."""
+    out = (ctypes.c_int * 5)()
+    lib().me_product_choice(_i(_code(torch.bfloat16)), _i(ROLE_DELTA_INTO), _i(rows), _i(rows_of_w), _i(k), _i(0),
+                            _i(_code(torch.bfloat16)), _i(units), _i(int(aligned)), out)
+    return int(out[0]), int(out[1]), bool(out[2]), bool(out[4])
 
 
 STREAM_MAX_ROWS = 256  # the weight-streaming product deals more than 64 rows to groups of blocks

@@ -81,3 +81,20 @@ def test_the_measured_rules_at_their_shapes():
     fusion = lambda rows, rows_of_w, k, pending: K.lib().me_norm_fusion_choice(1, rows, rows_of_w, k, pending, 256, 1)
     assert fusion(1, 4096, 1024, 2) == K.NORM_IN_STREAM and fusion(8, 4096, 1024, 1) == K.NORM_IN_SMALL
     assert fusion(8, 4096, 1024, 2) == K.NORM_ALONE and fusion(8, 6144, 4096, 1) == K.NORM_ALONE and fusion(17, 4096, 1024, 0) == K.NORM_ALONE
+
+
+@pytest.mark.parametrize("shape", sorted(SHAPES))
+def test_a_delta_is_added_into_the_stream_only_by_the_library(shape):
+    """Up to 64 rows the step program sums partial sums of runs of k; beyond, the library adds its one product into
+    the stream in its epilogue, and a shape the library is the fallback for stays one partial sum or the library's."""
+    for name, rows_of_w, k, gated, role in projections(shape):
+        if role != K.ROLE_DELTA:
+            continue
+        for rows in list(range(1, 301)) + [2048, 8192]:
+            kernel, runs, partial, adds = K.delta_choice(rows, rows_of_w, k, 256)
+            assert partial != adds, (name, rows)
+            assert adds == (kernel == K.PRODUCT_LIBRARY), (name, rows, kernel)
+            plain = K.product_choice(BF16, K.ROLE_DELTA, rows, rows_of_w, k, False, BF16, 256)
+            assert (kernel, runs) == plain[:2]  # the same kernel either way: only where the sum happens differs
+            if rows > 64:
+                assert adds
