@@ -681,116 +681,113 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
 // units (a short portion of a prompt over a long context), which is where the host does it.
 //
 // Keys and values are staged through LDS in tiles of 64 keys, double-buffered: while the waves
-// multiply tile i out of one buffer, the global loads of tile i+1 are in flight and are written to
-// the other buffer afterwards; one barrier per tile. Products use v_mfma_f32_16x16x32_bf16 (the
+// multiply tile i out of one buffer, the loads of tile i+1 fill the other, straight from the pages
+// (global_load_lds_dwordx4: no registers hold a tile and no LDS write instructions are issued; with the
+// tile in registers on its way a 2,048-token prompt took 38.6 us a layer, now 37.2, and 32,704 tokens
+// 161 ms in all, now 153); one barrier per tile. Products use v_mfma_f32_16x16x32_bf16 (the
 // full-rate bfloat16 instruction of gfx950; the 16x16x16 form runs at half its rate):
 //   S^T (16 keys x 16 columns) += K[16 keys, 32 d] . Q^T[32 d, 16 columns]
 //   O^T (16 d x 16 columns)   += V^T[16 d, 32 keys] . P^T[32 keys, 16 columns]
-// For the second product the 32 keys of a lane's B operand are the four keys it holds of each of two
-// 16-key score tiles (keys 4g..4g+3 and 16+4g..16+4g+3 of the 32); the value tile is stored in LDS in
-// that order, so the A operand is one 16-byte read and the contraction pairs up.
+// A lane holds four rows of every score tile. The rows of the four score tiles of a 64-key tile are dealt
+// to the keys so that these come to eight consecutive keys per 32 (PrefillLds below): the lane's B operand
+// of the second product then pairs with one 16-byte piece of a value row as it lies in its page.
 //
-// LDS rows are padded (keys and values: +16 elements) so that the 16-byte reads of a wave spread over
-// all banks. A 16-byte read is served in four groups of lanes
-// (0-3 with 12-15 and 20-27, 4-11 with 16-19 and 28-31, and the same in the upper half): with 16 rows
-// read by lane % 16 the groups are free of conflicts when the row stride is 32 bytes off a multiple
-// of 64 (measured: 5.3 cycles per wave instruction against 8 with a stride 16 bytes off).
+// A 16-byte LDS read is served in four groups of lanes (0-3 with 12-15 and 20-27, 4-11 with 16-19 and
+// 28-31, and the same in the upper half); the layouts below keep each group on distinct banks
+// (measured: 5.3 cycles per wave instruction against 8 with two lanes a bank).
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 
 #define PF_KT 64  // keys per LDS tile
-#define PF_PIECES(D, THREADS) ((8 * (D) + (THREADS) - 1) / (THREADS))  // 16-byte pieces of a tile per thread
 
+// One LDS buffer holds a 64-key tile as the global loads deliver it (a wave's load instruction writes 64
+// consecutive 16-byte pieces, one per lane, wherever in memory each lane reads): no rows can be padded, so
+// the key rows are swizzled instead.
+//   keys:   [64 keys][D/8 pieces]; the piece at physical column pc of key row k holds the eight dims from
+//           (pc ^ swizzle(k)) * 8. Row t*16.. of the first product's A operand is not key t*16 + r but
+//           key 32 (t/2) + 8 (r/4) + 4 (t%2) + r%4, so that a lane ends up with the scores of eight
+//           consecutive keys per 32 (four of score tile 2h, four of tile 2h+1): the B operand of the second
+//           product then pairs with eight consecutive keys of a value row, one 16-byte piece as it lies in
+//           the page. swizzle(k) = (k % 4) + 4 ((k / 8) % 4) is the row r that reads key k: with a row
+//           stride of 256 bytes (d = 128) the 16-byte reads of a wave's four groups of lanes hit every bank once.
+//   values: [4 sub-tiles of 16 keys][D dims][2 pieces]: the layout of a transposed page of 16 slots; rows 32
+//           bytes apart, read by lane % 16 with the piece chosen by the lane's upper bits, are free of conflicts as they are.
 template <int D>
 struct PrefillLds {
-  static constexpr int KROW = D + 16;       // elements per key row
-  static constexpr int VROW = PF_KT + 16;   // elements per value row (one d, 64 keys)
-  static constexpr int K_ELEMS = PF_KT * KROW;
-  static constexpr int V_ELEMS = D * VROW;
-  static constexpr int BUF_ELEMS = K_ELEMS + V_ELEMS;
-  static constexpr int BYTES = 2 * BUF_ELEMS * 2;
+  static constexpr int P = D / 8;                // 16-byte pieces per key row
+  static constexpr int REGION = PF_KT * D;       // elements of the keys of a tile, and of its values
+  static constexpr int BUF_ELEMS = 2 * REGION;
+  static constexpr int BUFFERS = 2;
+  static constexpr int BYTES = BUFFERS * BUF_ELEMS * 2;
+  static constexpr int LOW = (P & -P) < 16 ? (P & -P) : 16;  // the swizzle stays inside an aligned group of pieces that every row has
+  static constexpr int SWIZZLE_MASK = LOW - 1;
+  __device__ static constexpr int swizzle(int key) { return ((key & 3) | (((key >> 3) & 3) << 2)) & SWIZZLE_MASK; }
 };
 
-// Global loads of one 64-key tile into registers: thread `tid` of THREADS fetches 8D/THREADS
-// 16-byte pieces of keys and as many of values. Keys: piece c -> row c / (D/8), 8 elements at column
-// (c % (D/8)) * 8. Values: piece c -> 16-key sub-tile c / (2D), then d = (c % 2D) / 2, half = c % 2,
-// which walks a transposed value page front to back. The page size is a power of two.
-template <int D, int THREADS>
-struct PfPages {
-  int k[PF_PIECES(D, THREADS)], v[PF_PIECES(D, THREADS)];  // block-table entries, still per lane
+typedef __attribute__((address_space(1))) const void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// What a lane fetches of every tile: a wave's load instruction j of a region (j = wave, wave + WAVES, ...: D/8
+// instructions for the keys, as many for the values) brings pieces 64 j .. 64 j + 63 of the region. The pieces of
+// one instruction lie in one 16-key sub-tile, hence in one page: the page's address is scalar arithmetic and a
+// lane only adds its own offset, which is the same for every tile.
+template <int D, int WAVES>
+struct PfStage {
+  static constexpr int P = D / 8;
+  static constexpr int SLOTS = (P + WAVES - 1) / WAVES;
+  unsigned k_off[SLOTS], v_off[SLOTS];  // bytes from the sub-tile's first key (first slot) in its page
+  int page[SLOTS];                      // block-table entries of the tile to be fetched next: scalar
 };
 
-// Block-table entries of the pages that the wave's pieces of tile `key0` lie in. The loads are only
-// issued here; pf_load_tile waits for them, an iteration later, so their latency hides behind a
-// whole tile of work instead of standing at the head of every iteration.
-template <int D, int THREADS>
-__device__ __forceinline__ void pf_fetch_pages(PfPages<D, THREADS>& pages, int key0, int tid, const int* __restrict__ table,
-                                               int table_width, int bs_shift) {
-  const int wave_c0 = tid & ~(ME_WAVE - 1);
-#pragma unroll
-  for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
-    const int c_first = wave_c0 + i * THREADS;
-    const int key_k = key0 + ((c_first / (D / 8)) & ~15);
-    const int key_v = key0 + (c_first / (2 * D)) * 16;
-    pages.k[i] = table[min(key_k >> bs_shift, table_width - 1)];
-    pages.v[i] = table[min(key_v >> bs_shift, table_width - 1)];
-  }
-}
-
-template <int D, int THREADS>
-__device__ __forceinline__ void pf_load_tile(uint4v_t (&kreg)[PF_PIECES(D, THREADS)], uint4v_t (&vreg)[PF_PIECES(D, THREADS)], int key0,
-                                             int tid, const PfPages<D, THREADS>& pages, int bs_shift, int nkv, int kvh,
-                                             const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache) {
-  // The 64 lanes of a wave fetch pieces of one 16-key sub-tile (8D/64 consecutive pieces never
-  // straddle one), so the page of a piece is the same for the whole wave: it goes into a scalar
-  // register and the base address of the page is scalar arithmetic; a lane only adds its own offset.
-  const int bs_mask = (1 << bs_shift) - 1;
-  const int lane = tid & (ME_WAVE - 1), wave_c0 = tid - lane;
-#pragma unroll
-  for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
-    const int c_first = wave_c0 + i * THREADS;  // the wave's first piece of this round
-    if ((8 * D) % THREADS != 0 && c_first >= 8 * D) break;  // only the last round can be partial
-    const int c = c_first + lane;
-    {
-      const int key_w = key0 + ((c_first / (D / 8)) & ~15);  // first key of the wave's sub-tile
-      int page = __builtin_amdgcn_readfirstlane(pages.k[i]);
-      page = page < 0 ? 0 : page;
-      const bf16_t* base = k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + (key_w & bs_mask)) * D;
-      const int row = c / (D / 8) - (c_first / (D / 8) & ~15), col = c % (D / 8);
-      kreg[i] = *reinterpret_cast<const uint4v_t*>(base + row * D + col * 8);
-    }
-    {
-      const int sub = c_first / (2 * D);
-      const int key_w = key0 + sub * 16;
-      int page = __builtin_amdgcn_readfirstlane(pages.v[i]);
-      page = page < 0 ? 0 : page;
-      const bf16_t* base = v_cache + ((((size_t)page * nkv + kvh) * D) << bs_shift) + (key_w & bs_mask);
-      const int rem = c - sub * (2 * D);
-      const int d = rem >> 1, half = rem & 1;
-      vreg[i] = *reinterpret_cast<const uint4v_t*>(base + ((size_t)d << bs_shift) + half * 8);
-    }
-  }
-}
-
-template <int D, int THREADS>
-__device__ __forceinline__ void pf_store_tile(const uint4v_t (&kreg)[PF_PIECES(D, THREADS)], const uint4v_t (&vreg)[PF_PIECES(D, THREADS)],
-                                              bf16_t* ks, int tid) {
+template <int D, int WAVES>
+__device__ __forceinline__ void pf_stage_init(PfStage<D, WAVES>& st, int wave, int lane, int bs_shift) {
   using L = PrefillLds<D>;
-  bf16_t* vs = ks + L::K_ELEMS;
 #pragma unroll
-  for (int i = 0; i < PF_PIECES(D, THREADS); ++i) {
-    const int c = tid + i * THREADS;
-    if ((8 * D) % THREADS != 0 && c >= 8 * D) break;
-    const int row = c / (D / 8), col = c % (D / 8);
-    *reinterpret_cast<uint4v_t*>(ks + row * L::KROW + col * 8) = kreg[i];
-    const int sub = c / (2 * D), rem = c % (2 * D);
-    const int d = rem >> 1, half = rem & 1;
-    // Within a group of 32 keys the row holds, for g = 0..3, keys 4g..4g+3 and then keys 16+4g..16+4g+3:
-    // the eight keys a lane multiplies with its eight probabilities, as one 16-byte read.
-    uint2v_t* dst = reinterpret_cast<uint2v_t*>(vs + d * L::VROW + (sub >> 1) * 32 + half * 16 + (sub & 1) * 4);
-    dst[0] = (uint2v_t){vreg[i][0], vreg[i][1]};
-    dst[2] = (uint2v_t){vreg[i][2], vreg[i][3]};
+  for (int sl = 0; sl < PfStage<D, WAVES>::SLOTS; ++sl) {
+    const int n = 64 * (wave + sl * WAVES) + lane;  // piece of the region
+    const int key = (n / L::P) & (PF_KT - 1), pc = n % L::P;
+    st.k_off[sl] = (unsigned)(((key & 15) * D + ((pc ^ L::swizzle(key)) * 8)) * 2);
+    const int d = (n % (2 * D)) >> 1, piece = n & 1;
+    st.v_off[sl] = (((unsigned)d << bs_shift) * 2u) + (unsigned)piece * 16u;
+  }
+}
+
+// Block-table entries of the pages that the wave's instructions of tile `key0` read. Scalar loads, issued an
+// iteration before pf_issue_tile uses them.
+template <int D, int WAVES>
+__device__ __forceinline__ void pf_fetch_pages(PfStage<D, WAVES>& st, int key0, int wave, const int* __restrict__ table,
+                                               int table_width, int bs_shift) {
+  constexpr int P = D / 8;
+#pragma unroll
+  for (int sl = 0; sl < PfStage<D, WAVES>::SLOTS; ++sl) {
+    const int sub = min((wave + sl * WAVES) / (P / 4), 3);
+    st.page[sl] = table[min((key0 + 16 * sub) >> bs_shift, table_width - 1)];
+  }
+}
+
+// Requests tile `key0` from the pages straight into the LDS buffer `buf`; the data is there after the next
+// __syncthreads() (which waits for the wave's outstanding loads before the barrier).
+template <int D, int WAVES>
+__device__ __forceinline__ void pf_issue_tile(const PfStage<D, WAVES>& st, int key0, int wave, bf16_t* buf, int bs_shift, int nkv,
+                                              int kvh, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache) {
+  using L = PrefillLds<D>;
+  constexpr int P = D / 8;
+  const int bs_mask = (1 << bs_shift) - 1;
+  char* kdst = reinterpret_cast<char*>(buf);
+  char* vdst = reinterpret_cast<char*>(buf + L::REGION);
+#pragma unroll
+  for (int sl = 0; sl < PfStage<D, WAVES>::SLOTS; ++sl) {
+    const int j = wave + sl * WAVES;
+    if (P % WAVES != 0 && j >= P) break;  // the same for the whole wave
+    const int sub = j / (P / 4);
+    int page = st.page[sl];
+    page = page < 0 ? 0 : page;
+    const int off = (key0 + 16 * sub) & bs_mask;  // of the sub-tile's first key in its page
+    const char* kb = reinterpret_cast<const char*>(k_cache + ((((size_t)page * nkv + kvh) << bs_shift) + off) * D);
+    const char* vb = reinterpret_cast<const char*>(v_cache + ((((size_t)page * nkv + kvh) * D) << bs_shift) + off);
+    __builtin_amdgcn_global_load_lds((global_ptr_t)(kb + st.k_off[sl]), (lds_ptr_t)(kdst + j * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((global_ptr_t)(vb + st.v_off[sl]), (lds_ptr_t)(vdst + j * 1024), 16, 0, 0);
   }
 }
 
@@ -825,11 +822,13 @@ __device__ __forceinline__ void pf_scores64(const bf16_t* __restrict__ ks, int r
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int t = 0; t < 4; ++t) s[nb][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  const int key_r = 8 * (r >> 2) + (r & 3);  // the lane's key row of score tile 0; swizzle(key of any tile) = swizzle(key_r)
 #pragma unroll
   for (int c = 0; c < D / 32; ++c) {
+    const bf16_t* col = ks + key_r * D + ((c * 4 + g) ^ L::swizzle(key_r)) * 8;
     bf16x8_t kf[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) kf[t] = *reinterpret_cast<const bf16x8_t*>(ks + (t * 16 + r) * L::KROW + c * 32 + g * 8);
+    for (int t = 0; t < 4; ++t) kf[t] = *reinterpret_cast<const bf16x8_t*>(col + (32 * (t >> 1) + 4 * (t & 1)) * D);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -857,7 +856,7 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
     if (MASK) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int key = key_base + (i >> 2) * 16 + g * 4 + (i & 3);
+        const int key = key_base + (i >> 3) * 32 + g * 8 + ((i >> 2) & 1) * 4 + (i & 3);  // score tile i / 4, row 4g + i % 4
         if (key < lo_col[nb] || key > qpos[nb]) sv[i] = -INFINITY;
       }
     }
@@ -901,7 +900,7 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
   for (int h = 0; h < 2; ++h) {
 #pragma unroll
     for (int dt = 0; dt < D / 16; ++dt) {
-      const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r) * L::VROW + h * 32 + g * 8);
+      const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(vs + ((2 * h + (g >> 1)) * D + dt * 16 + r) * 16 + (g & 1) * 8);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
         acc[nb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[nb][h], acc[nb][dt], 0, 0, 0);
@@ -938,8 +937,11 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   using L = PrefillLds<D>;
   const int kvh = blockIdx.x % nkv;
   const int group = nh / nkv;
-  const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
+  const int tid = threadIdx.x, lane = tid & (ME_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / ME_WAVE);  // scalar: what a wave fetches follows from it
   const int r = lane & 15, g = lane >> 4;
+  PfStage<D, WAVES> stage;
+  pf_stage_init<D, WAVES>(stage, wave, lane, bs_shift);
   for (int wi = bundle_first[blockIdx.x / nkv];; ++wi) {
   const PrefillWork w = work[wi];  // the same for every lane: scalar loads
   const int item = w.item;
@@ -986,34 +988,26 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     for (int dt = 0; dt < D / 16; ++dt) acc[nb][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- global -> register -> LDS staging of 64-key tiles (pf_load_tile / pf_store_tile). While tile i
-  // is multiplied out of LDS buffer i % 2, tile i+1 waits in registers: it is written to the other buffer
-  // in the middle of the iteration, behind the first product, where the LDS writes and the global loads
-  // of tile i+2 that follow them overlap with the softmax arithmetic instead of standing between two
-  // barriers. The other buffer is free then: it was last read before the barrier that ended iteration i-1.
-  uint4v_t kreg[PF_PIECES(D, THREADS)], vreg[PF_PIECES(D, THREADS)];
+  // ---- staging of 64-key tiles: global memory -> LDS without a stop in registers (pf_issue_tile). While tile i
+  // is multiplied out of LDS buffer i % 2, the loads of tile i+1 fill the other buffer: it was last read
+  // before the barrier that ended iteration i-1, and the barrier that ends iteration i waits for the loads.
   const int first_tile = w.key_begin;
   const int last_key = w.key_last;
-  PfPages<D, THREADS> pages;
-  pf_fetch_pages<D, THREADS>(pages, first_tile, tid, table, table_width, bs_shift);
-  pf_load_tile<D, THREADS>(kreg, vreg, first_tile, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
-  pf_fetch_pages<D, THREADS>(pages, first_tile + PF_KT, tid, table, table_width, bs_shift);
-  pf_store_tile<D, THREADS>(kreg, vreg, lds, tid);
-  pf_load_tile<D, THREADS>(kreg, vreg, first_tile + PF_KT, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
-  pf_fetch_pages<D, THREADS>(pages, first_tile + 2 * PF_KT, tid, table, table_width, bs_shift);
+  pf_fetch_pages<D, WAVES>(stage, first_tile, wave, table, table_width, bs_shift);
+  pf_issue_tile<D, WAVES>(stage, first_tile, wave, lds, bs_shift, nkv, kvh, k_cache, v_cache);
+  pf_fetch_pages<D, WAVES>(stage, first_tile + PF_KT, wave, table, table_width, bs_shift);
   __syncthreads();
   int buf = 0;
   for (int key0 = first_tile; key0 <= last_key; key0 += PF_KT, buf ^= 1) {
     const bf16_t* ks = lds + (size_t)buf * L::BUF_ELEMS;
-    const bf16_t* vs = ks + L::K_ELEMS;
+    const bf16_t* vs = ks + L::REGION;
     const bool active = key0 <= wave_max_pos;  // else every column of the wave lies before this tile
+    // Tiles are fetched unconditionally (the page index is clamped to the table, so a tile past the last
+    // key reads valid memory that nobody uses).
+    pf_issue_tile<D, WAVES>(stage, key0 + PF_KT, wave, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, bs_shift, nkv, kvh, k_cache, v_cache);
+    pf_fetch_pages<D, WAVES>(stage, key0 + 2 * PF_KT, wave, table, table_width, bs_shift);  // for the next iteration
     float4_t s[NB][4];
     pf_scores64<D, NB>(ks, r, g, qf, s);  // also by a wave that will not use them: no control flow around s
-    // Tiles are fetched unconditionally (the page index is clamped to the table, so a tile past the last
-    // key reads valid memory that nobody uses): no control flow around the registers.
-    pf_store_tile<D, THREADS>(kreg, vreg, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, tid);
-    pf_load_tile<D, THREADS>(kreg, vreg, key0 + 2 * PF_KT, tid, pages, bs_shift, nkv, kvh, k_cache, v_cache);
-    pf_fetch_pages<D, THREADS>(pages, key0 + 3 * PF_KT, tid, table, table_width, bs_shift);  // for the next iteration
     if (active) {
       const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || window > 0;
       if (need_mask)

@@ -731,7 +731,7 @@ def test_temperature_sampling_is_keyed_repeatable_and_follows_softmax():
 
 # -------------------------------------------------------- matrix-core attention kernels (bfloat16)
 MFMA_SHAPES = [(4, 2, 32, 16), (6, 1, 32, 16), (16, 8, 128, 16), (8, 8, 64, 32), (16, 1, 64, 16), (3, 1, 96, 64),
-               (2, 2, 256, 16), (40, 2, 32, 16)]
+               (2, 2, 256, 16), (40, 2, 32, 16), (4, 2, 192, 16), (4, 4, 128, 128), (2, 1, 64, 256)]
 
 
 @pytest.mark.parametrize("nh,nkv,d,bs", MFMA_SHAPES)
