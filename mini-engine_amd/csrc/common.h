@@ -82,3 +82,48 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   for (int w = 0; w < nwaves; ++w) total += scratch[w];
   return total;
 }
+
+// ------------------------------------------------------------------ a norm carried from one product to the next
+// A product that is a delta of the float32 residual stream can add itself to the stream in its epilogue and leave,
+// for the RMS norm behind it, bf16(stream * w_norm) (not yet divided by the row's root mean square) and the sums of
+// squares of what its blocks added up, `blocks` partial sums a row. The product behind the norm multiplies its rows
+// by rsqrt(sum / dim + eps): a row's scale is a common factor of its products. No kernel of its own adds and norms.
+struct CarryOut {   // what the first product leaves (x == nullptr: an ordinary product)
+  float* x;         // [M, N] the residual stream, added to in place
+  bf16_t* h;        // [M, N] bf16(x * w_norm)
+  float* ss;        // [M, blocks] partial sums of squares of the rows of x
+  const float* w_norm;  // [N]
+  int blocks;
+};
+struct RowScale {   // what the second product reads (ss == nullptr: rows are not scaled)
+  const float* ss;  // [M, blocks]
+  int blocks;
+  float inv_dim, eps;
+};
+
+// scale[m] = rsqrt(sum_b ss[m, b] / dim + eps) for rows m < M, by the waves of a block in turn, in two halves: the loads
+// at a kernel's head (row_ss_fetch: wave w takes rows w, w + waves, ..; a lane sums every 64th partial sum), the rest
+// when the kernel's own work is done (row_scales_finish), so that the loads' latency hides behind it. The order of the
+// additions follows from the number of partial sums alone. The caller puts a barrier before it reads `scale`.
+template <int ROWS_PER_WAVE>
+__device__ __forceinline__ void row_ss_fetch(const RowScale& rs, int M, float (&part)[ROWS_PER_WAVE], int wave, int lane, int waves) {
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_WAVE; ++i) {
+    const int m = wave + i * waves;
+    // (one load per lane and row in the usual case, and nothing computed on it here: no wait at the kernel's head)
+    float s = m < M && lane < rs.blocks ? rs.ss[(size_t)m * rs.blocks + lane] : 0.f;
+    if (rs.blocks > ME_WAVE && m < M)
+      for (int b = lane + ME_WAVE; b < rs.blocks; b += ME_WAVE) s += rs.ss[(size_t)m * rs.blocks + b];
+    part[i] = s;
+  }
+}
+template <int ROWS_PER_WAVE>
+__device__ __forceinline__ void row_scales_finish(const RowScale& rs, int M, const float (&part)[ROWS_PER_WAVE], float* scale,
+                                                  int wave, int lane, int waves) {
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_WAVE; ++i) {
+    const int m = wave + i * waves;
+    const float s = wave_sum(part[i]);
+    if (m < M && lane == 0) scale[m] = rsqrtf(s * rs.inv_dim + rs.eps);
+  }
+}

@@ -14,6 +14,11 @@
 // deals the columns out in fours, as evenly as they go: the host picks arrangement, runs and blocks so that the launch
 // is whole rounds of the compute units where it can (plan_for_runs, plan_with_runs below).
 //
+// Two forms for a norm carried from a product to the next (common.h), instances of their own (AUX): a plain product of one
+// run of k that is a delta of the residual stream adds its columns to the stream in its epilogue and leaves bf16(x * w_norm)
+// and its part of the rows' sums of squares (me_gemm_bf16_stream_carry); a product multiplies its rows by
+// rsqrt(sum / dim + eps), with the sums read at its head and added up behind its loop (me_gemm_bf16_stream_scaled).
+//
 // Products use v_mfma_f32_16x16x32_bf16 in the transposed arrangement (C^T[n, m] = sum_k W[n, k] X[m, k]):
 // lane l feeds W[n0 + l % 16][8 k] and X[m0 + l % 16][8 k] (k = 32 c + 8 (l / 16) ..) and receives
 // C^T[4 (l / 16) .. +4][l % 16]. The SWIGLU form computes 16 gate columns and the 16 matching up columns per
@@ -34,10 +39,10 @@ constexpr int kMaxRows = 256;
 constexpr int kBufferFlags = 0x00020000;  // a raw buffer of 32-bit words (gfx9 family)
 constexpr int kRow = kStepK + 16;    // LDS row stride in elements: 288 bytes, 32 off a multiple of 64 (conflict-free 16-byte reads)
 
-template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int NT = 1>
+template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int NT = 1, bool AUX = false>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                           OutT* __restrict__ C, int rows, int N, int K, int steps_per_split, int gate,
-                                                          int rotate) {
+                                                          int rotate, RowScale rs, CarryOut carry) {
   static_assert(WN * WK == 4, "four waves per block");
   static_assert(NT == 1 || WK == 1, "waves with several tiles of columns do not cut k");
   // The grid's third dimension deals the rows out in groups of 16 MT; a block sees its group's rows only.
@@ -49,9 +54,15 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   constexpr int ACCS = (SWIGLU ? 2 : 1) * NT;  // tiles of 16 columns per wave: NT of them, gate and up of each in the gated form
   constexpr int XV = MT * 16 * (kStepK / 8) / 256;  // 16-byte vectors of x per thread and step
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][kRow];
+  __shared__ float row_scale[AUX ? MT * 16 : 1];  // with rs.ss: what the rows are multiplied by at the end
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int wn = wave % WN, wk = wave / WN;
   const int r = lane & 15, g = lane >> 4;
+  float ss_part[MT * 4];  // the rows whose scale this wave works out: loads here, the sums behind the loop over k
+  if (AUX && rs.ss) {
+    rs.ss += (size_t)blockIdx.z * (16 * MT) * rs.blocks;
+    row_ss_fetch<MT * 4>(rs, M, ss_part, wave, lane, 4);
+  }
   // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN NT) blocks gives every
   // block 16 WN NT columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
   const int fours = (N + 3) / 4;
@@ -144,6 +155,10 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     }
   }
 
+  if (AUX && rs.ss) {
+    row_scales_finish<MT * 4>(rs, M, ss_part, row_scale, wave, lane, 4);
+    __syncthreads();
+  }
   if (WK > 1) {  // the runs of k within a step: waves wk > 0 hand their sums to wave wk == 0 of their columns
     __syncthreads();
     float* red = reinterpret_cast<float*>(&xs[0][0][0]);  // [wk - 1][wn][t][a][j][lane]
@@ -172,6 +187,50 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     }
   }
   // lane (r, g) holds rows m = 16 t + r, columns 4 g .. +4 of each of its tiles
+  if constexpr (AUX && !SWIGLU && sizeof(OutT) == 4) {
+    if (carry.x) {
+      // The product is a delta of the residual stream and this block has all of k: x += delta, h = bf16(x * w_norm)
+      // and the sums of squares of the rows over the wave's columns, for the product behind the norm.
+      const size_t row0 = (size_t)blockIdx.z * (16 * MT);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r;
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+          const int nb = n0 + 16 * i + 4 * g;
+          if (m < M && nb < c1) {
+            float* xp = carry.x + (row0 + m) * N + nb;
+            bf16_t* hp = carry.h + (row0 + m) * N + nb;
+            if (nb + 3 < N && (N & 3) == 0) {
+              float4 v = *reinterpret_cast<const float4*>(xp);
+              const float4 wv = *reinterpret_cast<const float4*>(carry.w_norm + nb);
+              v.x += acc[t][i][0], v.y += acc[t][i][1], v.z += acc[t][i][2], v.w += acc[t][i][3];
+              *reinterpret_cast<float4*>(xp) = v;
+              uint2 packed;
+              packed.x = (uint32_t)f32_to_bf16_bits(v.x * wv.x) | ((uint32_t)f32_to_bf16_bits(v.y * wv.y) << 16);
+              packed.y = (uint32_t)f32_to_bf16_bits(v.z * wv.z) | ((uint32_t)f32_to_bf16_bits(v.w * wv.w) << 16);
+              *reinterpret_cast<uint2*>(hp) = packed;
+              sq = fmaf(v.x, v.x, sq), sq = fmaf(v.y, v.y, sq), sq = fmaf(v.z, v.z, sq), sq = fmaf(v.w, v.w, sq);
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if (nb + j < N) {
+                  const float v = xp[j] + acc[t][i][j];
+                  xp[j] = v;
+                  hp[j] = from_float<bf16_t>(v * carry.w_norm[nb + j]);
+                  sq = fmaf(v, v, sq);
+                }
+            }
+          }
+        }
+        sq += __shfl_xor(sq, 16, ME_WAVE);  // the four lanes of a row
+        sq += __shfl_xor(sq, 32, ME_WAVE);
+        if (g == 0 && m < M) carry.ss[(row0 + m) * carry.blocks + blockIdx.x * WN + wn] = sq;
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
     const int nb = n0 + 16 * i + 4 * g;
@@ -180,11 +239,12 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     for (int t = 0; t < MT; ++t) {
       const int m = t * 16 + r;
       if (m >= M) continue;
+      const float scale = AUX && rs.ss ? row_scale[m] : 1.f;
       float y[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        y[j] = acc[t][i][j];
-        if (SWIGLU) y[j] = gate_act(y[j], gate) * acc[t][NT + i][j];
+        y[j] = acc[t][i][j] * scale;
+        if (SWIGLU) y[j] = gate_act(y[j], gate) * (acc[t][NT + i][j] * scale);
       }
       OutT* dst = C + (size_t)m * N + nb;
       if (nb + 3 < N && (N & 3) == 0) {
@@ -448,6 +508,14 @@ StreamPlan plan_with_runs(int M, int N, int K, int compute_units) {
   return {1, 1, tiles, 1};  // (not reached)
 }
 
+// A delta that adds itself to the residual stream: every block walks all of k for a tile of 16 columns, four waves sharing k
+// within a step. (Narrower blocks, so that the launch goes round more compute units, are no faster: every block fetches all rows
+// of x whatever its width. 1,024 columns at 8 rows: 128 blocks of 8 columns as fast as 64 of 16, 256 of 4 slower.)
+StreamPlan plan_for_carry(int N, int compute_units) {
+  (void)compute_units;
+  return {1, 1, (N + 15) / 16, 1};
+}
+
 StreamPlan plan_of(int M, int N, int K, bool gated, int k_splits, int compute_units) {
   if (k_splits > 1) {
     const StreamPlan p = plan_with_runs(M, N, K, compute_units);
@@ -458,7 +526,7 @@ StreamPlan plan_of(int M, int N, int K, bool gated, int k_splits, int compute_un
 
 template <int MT, bool SWIGLU, typename OutT>
 void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int steps_per_split,
-                     int gate, hipStream_t stream) {
+                     int gate, RowScale rs, CarryOut carry, hipStream_t stream) {
   const dim3 grid(plan.grid, plan.splits, (M + kGroupRows - 1) / kGroupRows);
   const int wn = plan.wn;
   // Rows of W that lie a multiple of 4 KiB apart begin in the same memory channel: blocks that all start at k = 0 then
@@ -469,26 +537,36 @@ void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C,
   const int rotate = plan.splits == 1 && K % 2048 == 0;
   if constexpr (MT >= 3 && !SWIGLU && sizeof(OutT) == 4) {
     if (plan.nt == 2) {  // (two steps in flight: 3-15% ahead of three)
-      gemm_stream_kernel<MT, 4, 1, false, OutT, 2, 2><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
+      gemm_stream_kernel<MT, 4, 1, false, OutT, 2, 2><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
       return;
     }
   }
+  if (rs.ss || carry.x) {  // the forms that scale their rows or add into the residual stream: instances of their own
+    if (wn == 4)
+      gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3), 1, true><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
+    else if (wn == 2)
+      gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4), 1, true><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
+    else
+      // (more steps in flight gain nothing for a block that walks all of k: 8 and 12 stages measured slower than 6)
+      gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6), 1, true><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
+    return;
+  }
   if (wn == 4)
-    gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
+    gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
   else if (wn == 2)
-    gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
+    gemm_stream_kernel<MT, 2, 2, SWIGLU, OutT, (SWIGLU ? 3 : 4)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
   else
-    gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate);
+    gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
 }
 
 template <bool SWIGLU, typename OutT>
 void launch_rows(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int steps_per_split, int gate,
-                 hipStream_t stream) {
+                 RowScale rs, CarryOut carry, hipStream_t stream) {
   switch ((std::min(M, kGroupRows) + 15) / 16) {
-    case 1: launch_arranged<1, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
-    case 2: launch_arranged<2, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
-    case 3: launch_arranged<3, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
-    default: launch_arranged<4, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, stream); break;
+    case 1: launch_arranged<1, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, rs, carry, stream); break;
+    case 2: launch_arranged<2, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, rs, carry, stream); break;
+    case 3: launch_arranged<3, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, rs, carry, stream); break;
+    default: launch_arranged<4, SWIGLU, OutT>(plan, X, W, C, M, N, K, steps_per_split, gate, rs, carry, stream); break;
   }
 }
 
@@ -506,38 +584,75 @@ extern "C" void me_gemm_bf16_stream_plan(int M, int N, int K, int gated, int k_s
   out[0] = p.wn * p.nt, out[1] = p.splits, out[2] = p.grid;
 }
 
+static int stream_product(const char* who, const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
+                          int k_splits, int compute_units, RowScale rs, CarryOut carry, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("%s: unknown gate activation %d", who, swiglu);
+  if (M > kMaxRows) return me_fail("%s: M=%d exceeds %d rows", who, M, kMaxRows);
+  if (K <= 0 || K % 8) return me_fail("%s: K=%d must be a positive multiple of 8", who, K);
+  if (!X || !W || (!C && !carry.x)) return me_fail("%s: null operand", who);
+  if (((uintptr_t)X | (uintptr_t)W | (uintptr_t)C) & 15) return me_fail("%s: operands must be 16-byte aligned", who);
+  if (out_dtype != ME_BF16 && out_dtype != ME_F32) return me_fail("%s: output type %d", who, out_dtype);
+  if (k_splits < 1 || k_splits > 64) return me_fail("%s: %d splits of k", who, k_splits);
+  if (k_splits > 1 && (swiglu || out_dtype != ME_F32))
+    return me_fail("%s: partial sums over splits of k are plain float32 products", who);
+  if (swiglu && out_dtype != ME_BF16) return me_fail("%s: the gated form writes bfloat16", who);
+  if ((size_t)(swiglu ? 2 : 1) * N * K * 2 >= (1ull << 31) || (size_t)M * K * 2 >= (1ull << 31))
+    return me_fail("%s: operands of 2 GiB and more are not addressed by this kernel", who);
+  if (compute_units < 1) compute_units = 256;
+  const int steps = (K + kStepK - 1) / kStepK;
+  const int steps_per_split = (steps + k_splits - 1) / k_splits;
+  const int splits = (steps + steps_per_split - 1) / steps_per_split;  // no empty run
+  if (splits != k_splits) return me_fail("%s: K=%d cannot be cut into %d runs of whole steps", who, K, k_splits);
+  const StreamPlan plan = carry.x ? plan_for_carry(N, compute_units) : plan_of(M, N, K, swiglu != 0, splits, compute_units);
+  if (carry.x && carry.blocks != plan.grid * plan.wn * plan.nt)
+    return me_fail("%s: %d partial sums of squares a row, the launch writes %d", who, carry.blocks, plan.grid * plan.wn * plan.nt);
+  const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
+  if (swiglu)
+    launch_rows<true, bf16_t>(plan, x, w, (bf16_t*)C, M, N, K, steps_per_split, swiglu, rs, carry, stream);
+  else if (out_dtype == ME_F32)
+    launch_rows<false, float>(plan, x, w, (float*)C, M, N, K, steps_per_split, 0, rs, carry, stream);
+  else
+    launch_rows<false, bf16_t>(plan, x, w, (bf16_t*)C, M, N, K, steps_per_split, 0, rs, carry, stream);
+  return me_check_launch(who);
+}
+
 // C[M, N] = x . W^T (swiglu 1 or 2, a MeGate code: W is [2 N, K], gate rows then up rows, and C = act(gate) * up), X bfloat16 [M, K],
 // M <= 256, K % 8 == 0, pointers 16-byte aligned. out_dtype ME_BF16 or ME_F32. k_splits > 1 (plain float32
 // products only): C is [k_splits, M, N], partial sums over runs of k for the caller to add up.
 extern "C" int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
                                    int k_splits, int compute_units, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_stream: unknown gate activation %d", swiglu);
-  if (M > kMaxRows) return me_fail("me_gemm_bf16_stream: M=%d exceeds %d rows", M, kMaxRows);
-  if (K <= 0 || K % 8) return me_fail("me_gemm_bf16_stream: K=%d must be a positive multiple of 8", K);
-  if (!X || !W || !C) return me_fail("me_gemm_bf16_stream: null operand");
-  if (((uintptr_t)X | (uintptr_t)W | (uintptr_t)C) & 15) return me_fail("me_gemm_bf16_stream: operands must be 16-byte aligned");
-  if (out_dtype != ME_BF16 && out_dtype != ME_F32) return me_fail("me_gemm_bf16_stream: output type %d", out_dtype);
-  if (k_splits < 1 || k_splits > 64) return me_fail("me_gemm_bf16_stream: %d splits of k", k_splits);
-  if (k_splits > 1 && (swiglu || out_dtype != ME_F32))
-    return me_fail("me_gemm_bf16_stream: partial sums over splits of k are plain float32 products");
-  if (swiglu && out_dtype != ME_BF16) return me_fail("me_gemm_bf16_stream: the gated form writes bfloat16");
-  if ((size_t)(swiglu ? 2 : 1) * N * K * 2 >= (1ull << 31) || (size_t)M * K * 2 >= (1ull << 31))
-    return me_fail("me_gemm_bf16_stream: operands of 2 GiB and more are not addressed by this kernel");
-  if (compute_units < 1) compute_units = 256;
-  const int steps = (K + kStepK - 1) / kStepK;
-  const int steps_per_split = (steps + k_splits - 1) / k_splits;
-  const int splits = (steps + steps_per_split - 1) / steps_per_split;  // no empty run
-  if (splits != k_splits) return me_fail("me_gemm_bf16_stream: K=%d cannot be cut into %d runs of whole steps", K, k_splits);
-  const StreamPlan plan = plan_of(M, N, K, swiglu != 0, splits, compute_units);
-  const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
-  if (swiglu)
-    launch_rows<true, bf16_t>(plan, x, w, (bf16_t*)C, M, N, K, steps_per_split, swiglu, stream);
-  else if (out_dtype == ME_F32)
-    launch_rows<false, float>(plan, x, w, (float*)C, M, N, K, steps_per_split, 0, stream);
-  else
-    launch_rows<false, bf16_t>(plan, x, w, (bf16_t*)C, M, N, K, steps_per_split, 0, stream);
-  return me_check_launch("me_gemm_bf16_stream");
+  return stream_product("me_gemm_bf16_stream", X, W, C, M, N, K, swiglu, out_dtype, k_splits, compute_units, RowScale{}, CarryOut{},
+                        stream);
+}
+
+// The same product with its rows multiplied by rsqrt(sum_b row_ss[m, b] / ss_dim + eps) before the gate: the product
+// behind an RMS norm whose division was left to it (me_gemm_bf16_stream_carry wrote row_ss, float32 [M, ss_blocks]).
+extern "C" int me_gemm_bf16_stream_scaled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
+                                          int compute_units, const float* row_ss, int ss_blocks, int ss_dim, float eps,
+                                          hipStream_t stream) {
+  if (!row_ss || ss_blocks < 1 || ss_dim < 1) return me_fail("me_gemm_bf16_stream_scaled: no sums of squares");
+  return stream_product("me_gemm_bf16_stream_scaled", X, W, C, M, N, K, swiglu, out_dtype, 1, compute_units,
+                        RowScale{row_ss, ss_blocks, 1.f / (float)ss_dim, eps}, CarryOut{}, stream);
+}
+
+// Partial sums of squares a row that me_gemm_bf16_stream_carry writes for a product of these sizes.
+extern "C" int me_gemm_bf16_stream_carry_blocks(int M, int N, int K, int compute_units) {
+  (void)M, (void)K;
+  const StreamPlan p = plan_for_carry(N, compute_units < 1 ? 256 : compute_units);
+  return p.grid * p.wn * p.nt;
+}
+
+// x[M, N] += X . W^T in float32 (x the residual stream, X bfloat16 [M, K]), h[M, N] = bf16(x * w_norm) and
+// ss[M, blocks] = partial sums of squares of the new rows of x, blocks = me_gemm_bf16_stream_carry_blocks(M, N, K, units):
+// every block sums all of k for its columns, so nothing stays to be added up behind it.
+extern "C" int me_gemm_bf16_stream_carry(const void* X, const void* W, float* x, void* h, float* ss, const float* w_norm, int M,
+                                         int N, int K, int compute_units, hipStream_t stream) {
+  if (!x || !h || !ss || !w_norm) return me_fail("me_gemm_bf16_stream_carry: null operand");
+  if (((uintptr_t)x | (uintptr_t)w_norm) & 15 || (uintptr_t)h & 7) return me_fail("me_gemm_bf16_stream_carry: operands must be 16-byte aligned");
+  const int blocks = me_gemm_bf16_stream_carry_blocks(M, N, K, compute_units);
+  return stream_product("me_gemm_bf16_stream_carry", X, W, nullptr, M, N, K, 0, ME_F32, 1, compute_units, RowScale{},
+                        CarryOut{x, (bf16_t*)h, ss, w_norm, blocks}, stream);
 }
 
 namespace {

@@ -152,6 +152,25 @@ int choose_norm_fusion(int dtype, int m, int rows_of_w, int k, int pending, int 
   return kNormAlone;
 }
 
+// From three rows on the add-and-norm is a kernel of its own (above), one of eight launches a layer whose floors are what a
+// decode step of a few rows is made of. It goes away if the delta in front of it is summed over all of k by each block
+// (no runs of k across blocks: a fourth as many blocks, each with a longer walk), which then adds its columns to the stream,
+// writes bf16(x * w) and its part of the rows' sums of squares; the product behind the norm multiplies its rows by
+// rsqrt(mean + eps). Measured on the same GPU in turns, layers of 1,024 x 2,048 (o), 1,024 x 3,072 (down), 4,096 and
+// 2 x 3,072 x 1,024: the deltas take 6.7 us instead of 4.7 and the products behind them 0.6-0.9 more, the two add-and-norms
+// (4.6 each under the profiler, about 3 inside a graph) are gone: a step of 3 / 4 / 8 items 1.246 -> 1.198 / 1.435 -> 1.387 /
+// 1.781 -> 1.743 ms. With more rows the whole-k deltas cost more than the launches they save (16 items: 6,600 -> 6,570 tokens/s;
+// 24 and 32: 11,430 -> 10,300 and 12,290 -> 11,000), and so they do on weights that take longer to stream than a launch
+// costs (2,048 x 6,144 at 8 rows: 10.7 us against 7.3 in runs; a step of the 32B shape at batch 8, whose 320 blocks of 16
+// columns are a round and a quarter of the compute units, 12% slower): up to 8 rows, weights below 16 MiB.
+constexpr int kCarryMinRows = 3, kCarryMaxRows = 8;
+bool choose_carried_norm(int dtype, int m, int n, int k, int next_rows_of_w, int next_gated, int units, bool aligned) {
+  if (dtype != kBF16 || !aligned || m < kCarryMinRows || m > kCarryMaxRows || k % 8 || n % 8) return false;
+  if (!streams(m, n, k) || (int64_t)n * k >= kStreamMinElements) return false;
+  const ProductChoice next = choose_product(dtype, kRolePlain, m, next_rows_of_w, n, next_gated, dtype, units, aligned);
+  return !next.gate_after && (next.kernel == kProductSmall || next.kernel == kProductStream);
+}
+
 }  // namespace me
 
 // out: kernel, runs, partial_sums, gate_after, adds_into
@@ -167,4 +186,8 @@ extern "C" void me_product_choice(int dtype, int role, int m, int rows_of_w, int
 
 extern "C" int me_norm_fusion_choice(int dtype, int m, int rows_of_w, int k, int pending, int units, int aligned) {
   return me::choose_norm_fusion(dtype, m, rows_of_w, k, pending, units, aligned != 0);
+}
+
+extern "C" int me_carried_norm_choice(int dtype, int m, int n, int k, int next_rows_of_w, int next_gated, int units, int aligned) {
+  return me::choose_carried_norm(dtype, m, n, k, next_rows_of_w, next_gated, units, aligned != 0) ? 1 : 0;
 }

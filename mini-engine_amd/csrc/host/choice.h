@@ -43,6 +43,9 @@ enum PendingKind { kPendingNone = 0, kPendingTensor = 1, kPendingParts = 2 };
 ProductChoice choose_product(int dtype, int role, int m, int rows_of_w, int k, int gated, int out_dtype, int units,
                              bool aligned);
 int choose_norm_fusion(int dtype, int m, int rows_of_w, int k, int pending, int units, bool aligned);
+// Whether a delta of the residual stream (m rows, n = hidden columns, k) adds itself to the stream and leaves the norm
+// behind it to the product after the norm (next_rows_of_w rows of hidden, gated or not): no add-and-norm kernel between.
+bool choose_carried_norm(int dtype, int m, int n, int k, int next_rows_of_w, int next_gated, int units, bool aligned);
 
 // Limits that the rules above share with the arena's sizing.
 constexpr int kSmallMaxRows = 64;      // what the small matrix-core kernel accepts

@@ -42,7 +42,13 @@ struct Pending {
   const float* parts = nullptr;
   int num_parts = 0;
   long long stride = 0;
+  // A delta that has added itself to the stream and left the norm behind it half done: bf16(x * w) in the buffer of
+  // normed rows and the rows' sums of squares in `ss_blocks` partial sums, for the product behind the norm `carried_w`.
+  const float* ss = nullptr;
+  int ss_blocks = 0;
+  const void* carried_w = nullptr;
   bool any() const { return delta || parts; }
+  bool carried() const { return ss != nullptr; }
 };
 
 int compute_units() {
@@ -142,9 +148,14 @@ class Run {
   }
 
   RunResult go() {
-    for (const Op& op : prog_.ops()) {
+    const std::vector<Op>& ops = prog_.ops();
+    for (size_t at = 0; at < ops.size(); ++at) {
+      const Op& op = ops[at];
+      next_ = at + 1 < ops.size() ? &ops[at + 1] : nullptr;
       const size_t mark = arena_.used;
       released_to_ = (size_t)-1;
+      if (pending_.carried() && op.kind != kOpNormLinear)
+        throw Error(kBroken, "a norm was left to a product that does not follow");
       step(op);
       // the logits, the drawn tokens and partial sums that wait for the next norm outlive their operation;
       // an operation that used up waiting partial sums gives their memory back too
@@ -220,7 +231,7 @@ class Run {
   }
 
   void release_parts() {
-    if (parts_mark_ != (size_t)-1 && !pending_.parts) {
+    if (parts_mark_ != (size_t)-1 && !pending_.parts && !pending_.ss) {
       arena_.used = released_to_ = parts_mark_;
       parts_mark_ = (size_t)-1;
     }
@@ -232,6 +243,21 @@ class Run {
     const int gated = (int)op.i[2];  // 0, or the code of the gate's activation
     if (k != h_) throw Error(kBadValue, "a product behind a norm reads the hidden size");
     const int n = gated ? rows_of_w / 2 : rows_of_w;
+    if (pending_.carried()) {  // the add is done and the norm half done: this product multiplies its rows by the rest
+      if (op.p[0] != pending_.carried_w) throw Error(kBroken, "a norm was left to the product behind another norm");
+      const ProductChoice c = choose_product(dtype_, kRolePlain, t_, rows_of_w, k, gated, dtype_, compute_units(), true);
+      if (c.kernel == kProductSmall && !c.gate_after)
+        ok(me_gemm_bf16_small_scaled(normed_, op.p[1], bufs_[op.out], t_, n, k, gated, dtype_, pending_.ss, pending_.ss_blocks, k,
+                                     op.f[0], stream_));
+      else if (c.kernel == kProductStream && !c.gate_after)
+        ok(me_gemm_bf16_stream_scaled(normed_, op.p[1], bufs_[op.out], t_, n, k, gated, dtype_, compute_units(), pending_.ss,
+                                      pending_.ss_blocks, k, op.f[0], stream_));
+      else
+        throw Error(kBroken, "a norm was left to a product whose kernel does not scale its rows");
+      pending_ = Pending();
+      release_parts();
+      return;
+    }
     const int pending = pending_.parts ? kPendingParts : pending_.delta ? kPendingTensor : kPendingNone;
     // Where the add and the norm ride on the product the sum goes to the second residual buffer, since other blocks
     // of the kernel still read the first.
@@ -296,6 +322,18 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
+    if (next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ &&
+        choose_carried_norm(dtype_, t_, n, k, (int)next_->i[0], (int)next_->i[2], compute_units(), true)) {
+      // x += product in the product's epilogue, which also starts the norm behind it (choice.cpp)
+      const int blocks = me_gemm_bf16_stream_carry_blocks(t_, n, k, compute_units());
+      parts_mark_ = arena_.used;
+      float* ss = (float*)arena_.take((size_t)t_ * blocks * 4);
+      ok(me_gemm_bf16_stream_carry(x, op.p[1], x_, normed_, ss, (const float*)next_->p[0], t_, n, k, compute_units(), stream_));
+      pending_.ss = ss;
+      pending_.ss_blocks = blocks;
+      pending_.carried_w = next_->p[0];
+      return;
+    }
     const ProductChoice c = choose_product(dtype_, kRoleDeltaInto, t_, n, k, 0, dtype_, compute_units(), true);
     if (c.adds_into) {  // x += product, in the library's epilogue: nothing stays pending
       if (library_adds(x, op.p[1], x_, t_, n, k, stream_)) return;
@@ -463,6 +501,7 @@ class Run {
   void* normed_;
   std::vector<void*> bufs_;
   Pending pending_;
+  const Op* next_ = nullptr;  // the operation behind the one being run
   size_t parts_mark_ = (size_t)-1, released_to_ = (size_t)-1;
   RunResult result_;
 };

@@ -53,6 +53,13 @@ int me_gemm_bf16_stream_splits(int M, int N, int K, int compute_units);
 void me_gemm_bf16_stream_plan(int M, int N, int K, int gated, int k_splits, int compute_units, int* out);
 int me_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype, int k_splits,
                         int compute_units, hipStream_t stream);
+int me_gemm_bf16_stream_scaled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
+                               int compute_units, const float* row_ss, int ss_blocks, int ss_dim, float eps, hipStream_t stream);
+int me_gemm_bf16_stream_carry_blocks(int M, int N, int K, int compute_units);
+int me_gemm_bf16_stream_carry(const void* X, const void* W, float* x, void* h, float* ss, const float* w_norm, int M, int N, int K,
+                              int compute_units, hipStream_t stream);
+int me_gemm_bf16_small_scaled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
+                              const float* row_ss, int ss_blocks, int ss_dim, float eps, hipStream_t stream);
 int me_gemm_bf16_stream_norm_fits(int M, int K);
 int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, const float* parts, int num_parts, long long part_stride,
                              const float* w_norm, float eps, float* x_out, const void* W, void* C, int M, int N, int K,

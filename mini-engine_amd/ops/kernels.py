@@ -412,6 +412,15 @@ def delta_choice(rows: int, rows_of_w: int, k: int, units: int, aligned: bool = 
     return int(out[0]), int(out[1]), bool(out[2]), bool(out[4])
 
 
+def carried_norm_choice(dtype: torch.dtype, rows: int, n: int, k: int, next_rows_of_w: int, next_gated: bool, units: int,
+                        aligned: bool = True) -> bool:
+    """Whether the step program lets a delta of the residual stream (``rows`` x ``n`` = hidden, over ``k``) add itself to
+    the stream and leave the RMS norm behind it to the product after the norm (``next_rows_of_w`` rows of hidden): the
+    rule of ``csrc/host/choice.cpp``; no GPU is touched."""
+    return bool(lib().me_carried_norm_choice(_i(_code(dtype)), _i(rows), _i(n), _i(k), _i(next_rows_of_w), _i(int(bool(next_gated))),
+                                             _i(units), _i(int(aligned))))
+
+
 STREAM_MAX_ROWS = 256  # the weight-streaming product deals more than 64 rows to groups of blocks
 SMALL_MAX_ROWS = 64  # what the small matrix-core kernel accepts
 
@@ -459,6 +468,56 @@ def gemm_bf16_stream(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
     _want(out, "out", out_dtype, shape)
     check(lib().me_gemm_bf16_stream(_p(x), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
                                     _i(_code(out_dtype)), _i(k_splits), _i(compute_units(x.device)), _stream()))
+    return out
+
+
+def stream_carry_blocks(rows: int, n: int, k: int, device=None, units: int | None = None) -> int:
+    """Partial sums of squares a row that :func:`gemm_bf16_stream_carry` leaves for a product of these sizes."""
+    return int(lib().me_gemm_bf16_stream_carry_blocks(_i(rows), _i(n), _i(k), _i(units if units is not None else compute_units(device))))
+
+
+def gemm_bf16_stream_carry(a: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor
+                           ) -> tuple[torch.Tensor, torch.Tensor]:
+    """A product that is a delta of the float32 residual stream, added to the stream in its epilogue:
+    ``x += a @ weight.T`` in place; returns ``h = bf16(x * norm_weight)``, not yet divided by the rows' root mean
+    squares, and ``ss`` float32 ``[rows, blocks]``, partial sums of squares of the rows of the new ``x``. The product
+    behind the norm divides (:func:`gemm_bf16_scaled`)."""
+    _want(a, "a", torch.bfloat16, (None, None))
+    m, k = a.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0]
+    _want(x, "residual stream", torch.float32, (m, n))
+    _want(norm_weight, "norm weight", torch.float32, (n,))
+    if m > STREAM_MAX_ROWS:
+        raise ValueError(f"gemm_bf16_stream_carry takes at most {STREAM_MAX_ROWS} rows, got {m}")
+    blocks = stream_carry_blocks(m, n, k, a.device)
+    h = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    ss = torch.empty((m, blocks), dtype=torch.float32, device=a.device)
+    check(lib().me_gemm_bf16_stream_carry(_p(a), _p(weight), _p(x), _p(h), _p(ss), _p(norm_weight), _i(m), _i(n), _i(k),
+                                          _i(compute_units(a.device)), _stream()))
+    return h, ss
+
+
+def gemm_bf16_scaled(h: torch.Tensor, weight: torch.Tensor, ss: torch.Tensor, dim: int, eps: float, swiglu: bool = False,
+                     out_dtype: torch.dtype = torch.bfloat16, kernel: str = "small") -> torch.Tensor:
+    """``(h * rsqrt(ss.sum(1) / dim + eps)[:, None]) @ weight.T`` with the rows' scale applied to the product (before
+    the gate): the product behind an RMS norm whose division :func:`gemm_bf16_stream_carry` left to it. ``kernel``:
+    "small" (at most 64 rows) or "stream"."""
+    _want(h, "h", torch.bfloat16, (None, None))
+    m, k = h.shape
+    _want(weight, "weight", torch.bfloat16, (None, k))
+    n = weight.shape[0] // 2 if swiglu else weight.shape[0]
+    _want(ss, "sums of squares", torch.float32, (m, None))
+    out = torch.empty((m, n), dtype=out_dtype, device=h.device)
+    if kernel == "small":
+        check(lib().me_gemm_bf16_small_scaled(_p(h), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
+                                              _i(_code(out_dtype)), _p(ss), _i(ss.shape[1]), _i(dim), _f(eps), _stream()))
+    elif kernel == "stream":
+        check(lib().me_gemm_bf16_stream_scaled(_p(h), _p(weight), _p(out), _i(m), _i(n), _i(k), _i(gate_code(swiglu)),
+                                               _i(_code(out_dtype)), _i(compute_units(h.device)), _p(ss), _i(ss.shape[1]),
+                                               _i(dim), _f(eps), _stream()))
+    else:
+        raise ValueError(f"unknown kernel {kernel!r}")
     return out
 
 

@@ -301,6 +301,42 @@ def test_gemm_bf16_small_with_very_many_columns(m, n, k):
         assert (got - want).abs().max().item() <= tol_abs, (out_dtype, (got - want).abs().max().item(), scale)
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 1024, 2048), (8, 1024, 3072), (16, 1032, 520), (5, 104, 72), (33, 2048, 1000), (64, 4096, 264),
+                                   (70, 520, 136), (130, 1024, 1024)])
+def test_a_norm_carried_from_one_product_to_the_next(m, n, k):
+    """The delta of the residual stream added to it in the product's epilogue, with bf16(x * w) and partial sums of
+    squares left for the product behind the RMS norm, which multiplies its rows by rsqrt(mean + eps): against the
+    float32 add, norm and products, for both kernels that take the second product, gated and not. One row of the
+    stream is a thousand times the others, so that a scale taken from another row's sums shows."""
+    g = torch.Generator().manual_seed(m * 31 + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    x = torch.randn(m, n, generator=g)
+    x[m // 2] *= 1000.0
+    wn = 1.0 + 0.3 * torch.randn(n, generator=g)
+    eps = 1e-3
+    x_dev = dev(x.clone())
+    h, ss = K().gemm_bf16_stream_carry(dev(a), dev(w), x_dev, dev(wn))
+    want_x = x + a.float() @ w.float().T
+    assert (x_dev.cpu() - want_x).abs().max().item() <= 1e-4 * want_x.abs().max().item()
+    assert ss.shape == (m, K().stream_carry_blocks(m, n, k))
+    assert torch.allclose(ss.sum(1).cpu(), (want_x**2).sum(1), rtol=1e-4)
+    want_h = want_x * wn
+    assert ((h.float().cpu() - want_h).abs() <= 2**-7 * want_h.abs() + 1e-5 * want_x.abs().max()).all()  # one rounding to bfloat16
+    normed = plain.rms_norm(want_x, wn, eps)
+    for n2 in (96, 3 * 1024 + 8):
+        w2 = (torch.randn(2 * n2, n, generator=g) * 0.05).bfloat16()
+        y = normed @ w2.float().T
+        for gated in (False, True):
+            want = plain.silu(y[:, :n2]) * y[:, n2:] if gated else y
+            for kernel in ("small", "stream"):
+                if kernel == "small" and m > 64:
+                    continue
+                got = K().gemm_bf16_scaled(h, dev(w2), ss, n, eps, gated, torch.bfloat16, kernel).float().cpu()
+                assert got.shape == want.shape
+                assert ((got - want).abs().max(1).values <= 2**-6 * want.abs().max(1).values.clamp_min(1e-3)).all(), (n2, gated, kernel)
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 16, 128), (7, 100, 72), (16, 1040, 1000), (17, 4099, 1536), (33, 200, 2056), (48, 68, 8200),
                                    (64, 9000, 648), (64, 40, 136), (2, 3072, 264), (8, 6140, 128), (3, 6142, 136), (5, 1000, 3072),
                                    (64, 4096, 16384), (40, 2100, 24576), (33, 4098, 8704), (65, 520, 264), (130, 3072, 1024),

@@ -98,3 +98,38 @@ def test_a_delta_is_added_into_the_stream_only_by_the_library(shape):
             assert (kernel, runs) == plain[:2]  # the same kernel either way: only where the sum happens differs
             if rows > 64:
                 assert adds
+
+
+@pytest.mark.parametrize("shape", sorted(SHAPES))
+def test_a_norm_is_left_to_the_product_behind_it_only_where_that_product_scales_its_rows(shape):
+    """A delta adds itself to the stream and leaves the norm behind it half done for a few rows of a small weight,
+    and only in front of a product whose kernel multiplies its rows by the rest of the norm."""
+    proj = {name: (rows_of_w, k, gated) for name, rows_of_w, k, gated, _ in projections(shape)}
+    seen = set()
+    for delta, behind in (("o", "gate_up"), ("down", "qkv")):
+        n, k, _ = proj[delta]
+        next_rows, hidden, gated = proj[behind]
+        assert hidden == n
+        for rows in list(range(1, 301)) + [2048]:
+            carried = K.carried_norm_choice(BF16, rows, n, k, next_rows, gated, 256)
+            seen.add(carried)
+            if carried:
+                assert 3 <= rows <= 8 and n * k * 2 < 16 << 20
+                kernel, _, partial, gate_after = K.product_choice(BF16, K.ROLE_PLAIN, rows, next_rows, n, gated, BF16, 256)
+                assert kernel in (K.PRODUCT_SMALL, K.PRODUCT_STREAM) and not gate_after and not partial
+            assert not K.carried_norm_choice(F32, rows, n, k, next_rows, gated, 256)
+            assert not K.carried_norm_choice(BF16, rows, n, k, next_rows, gated, 256, aligned=False)
+    assert (True in seen) == (shape in ("0.6b", "1.7b"))
+
+
+def test_the_tiny_models_of_the_gpu_tests_leave_their_norms_to_the_products_behind():
+    """The GPU tests replay steps of three to eight tokens on these models: the carried norm is what they run there
+    (all but E, whose widths no kernel of this kind takes)."""
+    from conftest import tiny_configs
+
+    for name, cfg in tiny_configs().items():
+        hidden, inter, width = cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads * cfg.head_dim
+        qkv_rows = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
+        for rows in (3, 8):
+            assert K.carried_norm_choice(BF16, rows, hidden, width, 2 * inter, True, 256) == (name != "E"), name
+            assert K.carried_norm_choice(BF16, rows, hidden, inter, qkv_rows, False, 256) == (name != "E"), name
