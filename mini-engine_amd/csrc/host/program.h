@@ -5,7 +5,9 @@
 //
 // State that the operations share: the residual stream x (float32 [tokens, hidden]) in one of two
 // buffers, and a pending delta (a part's output that the next norm adds to x while it norms): nothing,
-// a buffer in the compute dtype, or partial sums over runs of k that the add sums up.
+// a buffer in the compute dtype, partial sums over runs of k that the add sums up, or, where the delta's
+// product has added itself to x already, the first half of the norm behind it (the rows times the norm's
+// weight, and their sums of squares) for the product after the norm to finish.
 #pragma once
 
 #include <hip/hip_runtime_api.h>
