@@ -75,11 +75,19 @@ struct KvTile {
   short4_t vf[D / 16];
 };
 
-template <int D>
+template <int D, bool STREAMED>
 __device__ __forceinline__ void load_tile(KvTile<D>& t, const bf16_t* __restrict__ kbase,
                                           const bf16_t* __restrict__ vbase, int bs) {
   const int lane = threadIdx.x & (ME_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
+  if constexpr (STREAMED) {  // non-temporal loads: for launches that stream hundreds of megabytes once (the host decides)
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) t.kf[c].u = stream_load16(kbase + (size_t)r * D + c * 32 + g * 8);
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt)
+      t.vf[dt] = __builtin_bit_cast(short4_t, stream_load8(vbase + (size_t)(dt * 16 + r) * bs + g * 4));
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < D / 32; ++c) t.kf[c].u = *reinterpret_cast<const uint4*>(kbase + (size_t)r * D + c * 32 + g * 8);
 #pragma unroll
@@ -169,7 +177,7 @@ struct DecodeFusedArgs {
 // with two tiles in flight, which only blocks of at most four waves (one per SIMD) may have.
 #define DECODE_BLOCK_WAVES(D) ((D) <= 128 ? 8 : 4)
 
-template <int D, bool FUSED, int DEPTH>
+template <int D, bool FUSED, int DEPTH, bool STREAMED>
 __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
@@ -193,8 +201,8 @@ __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_k
     int page = table[min(key0 >> bs_shift, table_width - 1)];
     page = page < 0 ? 0 : page;
     const int off = key0 & (bs - 1);
-    load_tile<D>(t, k_cache + (((size_t)page * nkv + kvh) * bs + off) * D,
-                 v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
+    load_tile<D, STREAMED>(t, k_cache + (((size_t)page * nkv + kvh) * bs + off) * D,
+                           v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
   };
   KvTile<D> t[DEPTH];
   // The keys of an item, from its window's first (rounded down to a tile of 16) to its newest, are dealt
@@ -509,17 +517,24 @@ template <int D>
 static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* item_ctx, const int* table,
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
                           float scale_log2, int depth, int num_splits, int block_waves, bf16_t* out,
-                          const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, hipStream_t stream) {
+                          const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, int streamed, hipStream_t stream) {
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits / block_waves);  // num_splits is a multiple of block_waves
   const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
   const size_t lds = block_waves > 1 ? (size_t)block_waves * heads_most * (D + 2) * sizeof(float) : 0;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
-#define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                                                                         \
-  attention_decode_kernel<D, FUSED, DEPTH><<<grid, 64 * block_waves, lds, stream>>>(                                       \
+#define ME_DECODE_LAUNCH_AS(FUSED, DEPTH, STREAMED, ARGS)                                                                  \
+  attention_decode_kernel<D, FUSED, DEPTH, STREAMED><<<grid, 64 * block_waves, lds, stream>>>(                             \
       q, kc, vc, item_ctx, table, width, part_o, part_ml, out, nh, nkv, bs_shift, window, scale_log2, num_splits, chunks,  \
       ARGS, live_items, waves_wanted)
+#define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                \
+  do {                                                      \
+    if (streamed)                                           \
+      ME_DECODE_LAUNCH_AS(FUSED, DEPTH, true, ARGS);        \
+    else                                                    \
+      ME_DECODE_LAUNCH_AS(FUSED, DEPTH, false, ARGS);       \
+  } while (0)
   if constexpr (D % 64 == 0) {
     if (fused) {
       if (depth == 2)
@@ -533,6 +548,7 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
     ME_DECODE_LAUNCH(false, 2, DecodeFusedArgs{});
   else
     ME_DECODE_LAUNCH(false, 1, DecodeFusedArgs{});
+#undef ME_DECODE_LAUNCH_AS
 #undef ME_DECODE_LAUNCH
 }
 
@@ -644,12 +660,20 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
     const long long rounds = (blocks + cus - 1) / cus;
     if (blocks > cus && blocks * 10 < rounds * cus * 9) block_waves = 1;  // rounds that are less than nine tenths full
   }
+  // Keys and values pass through once: loaded as non-temporal they arrive faster where the launch streams hundreds of
+  // megabytes over a full chip (batch 64 at 4,096: 6.21 -> 5.97 ms a step; batch 8 and 16 at 16,384: 3.54 -> 3.41 and
+  // 6.0 -> 5.6), and no faster or slower where it does not (batch 8 at 4,096, 134 MB: level; 33 MB and less: 0.4-0.8% slower;
+  // 160 to 224 blocks of 5 to 7 waves on 256 compute units, batch 20 to 28: 1-5% slower). The size goes by the longest context
+  // the launch may hold. (An instance of the kernel of its own: as a branch inside one kernel it cost steps that do not take
+  // it up to 4%.)
+  const long long kv_bytes = (long long)items * max_ctx * nkv * d * 4;
+  const int streamed = kv_bytes >= (256ll << 20) && (block_waves == 1 || (long long)items * nkv * ((nh / nkv + 15) / 16) >= 256);
   const float sl = scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
 #define ME_DECODE_CASE(DD)                                                                                      \
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
-                      depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, stream);   \
+                      depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, streamed, stream);   \
     break;
   switch (d) {
     ME_DECODE_CASE(32)
