@@ -46,9 +46,11 @@ __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
 }
 
 // ------------------------------------------------------------------ loads of data that is read once
-// Keys and values of a decode step and the weights of a skinny product pass through once: loaded as non-temporal
-// (the `nt` bit) they stream at 7.1-7.2 TB/s where ordinary loads reach 6.1-6.5 (4 GiB read by 2,048 to 131,072
-// blocks of 256 lanes, 16 bytes a lane).
+// A buffer that a kernel reads once streams at 7.1-7.2 TB/s through non-temporal loads (the `nt` bit) where ordinary
+// loads reach 6.1-6.5 (4 GiB read by 2,048 to 131,072 blocks of 256 lanes, 16 bytes a lane). Decode attention takes
+// the keys and values of large launches that way. Weights do not gain: the head's 311 MB at one row and the
+// projections of the 8B and 32B shapes took 1-11% longer (what a step reads again the step after seems to be served
+// better by ordinary loads).
 typedef unsigned me_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned me_u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint4 stream_load16(const void* p) {
@@ -58,7 +60,6 @@ __device__ __forceinline__ uint4 stream_load16(const void* p) {
 __device__ __forceinline__ me_u32x2 stream_load8(const void* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const me_u32x2*>(p));
 }
-constexpr int kBufferStreamed = 2;  // the same bit in the `aux` argument of a raw buffer load
 
 // ------------------------------------------------------------------ the activation of a gated feed-forward
 // act(gate) * up: the codes that the entry points' `gated` arguments take (0: the product is not gated).
