@@ -178,11 +178,11 @@ struct DecodeFusedArgs {
 #define DECODE_BLOCK_WAVES(D) ((D) <= 128 ? 8 : 4)
 
 template <int D, bool FUSED, int DEPTH, bool STREAMED>
-__global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_kernel(
+__device__ __forceinline__ void attention_decode_body(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
     float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
-    int window, float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa,
+    int window, float scale_log2, int num_splits, int head_chunks, const DecodeFusedArgs& fa,
     const int* __restrict__ live_items, int waves_wanted) {
   extern __shared__ float decode_lds[];  // only with several waves a block: their results, to be added up
   const int bs = 1 << bs_shift;
@@ -429,6 +429,29 @@ __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_k
   }
 }
 
+// STREAMED: the launch is large enough for non-temporal loads of its keys and values to pay (the host decides by its
+// size). They pay where every item reads pages of its own; items that share their pages (a prefix served from the
+// cache) read them out of each other's cache lines, which ordinary loads keep: the step says which it is (bit 0 of
+// step_flags[0]), and the kernel holds both bodies.
+template <int D, bool FUSED, int DEPTH, bool STREAMED>
+__global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
+    float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
+    int window, float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa,
+    const int* __restrict__ live_items, int waves_wanted, const int* __restrict__ step_flags) {
+  if constexpr (STREAMED) {
+    if (!(step_flags && (step_flags[0] & 1))) {
+      attention_decode_body<D, FUSED, DEPTH, true>(q, k_cache, v_cache, item_ctx, block_table, table_width, part_o, part_ml, out, nh,
+                                                   nkv, bs_shift, window, scale_log2, num_splits, head_chunks, fa, live_items,
+                                                   waves_wanted);
+      return;
+    }
+  }
+  attention_decode_body<D, FUSED, DEPTH, false>(q, k_cache, v_cache, item_ctx, block_table, table_width, part_o, part_ml, out, nh, nkv,
+                                                bs_shift, window, scale_log2, num_splits, head_chunks, fa, live_items, waves_wanted);
+}
+
 // out[item, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One block of 256 threads per
 // (item, head): the weights of all splits first (every split's statistics are loaded at once), then
 // the weighted sum with thread -> (four output elements, one of 256 / (d/4) groups of splits), so
@@ -517,7 +540,8 @@ template <int D>
 static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const int* item_ctx, const int* table,
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
                           float scale_log2, int depth, int num_splits, int block_waves, bf16_t* out,
-                          const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, int streamed, hipStream_t stream) {
+                          const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, int streamed,
+                          const int* step_flags, hipStream_t stream) {
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits / block_waves);  // num_splits is a multiple of block_waves
   const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
@@ -527,7 +551,7 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
 #define ME_DECODE_LAUNCH_AS(FUSED, DEPTH, STREAMED, ARGS)                                                                  \
   attention_decode_kernel<D, FUSED, DEPTH, STREAMED><<<grid, 64 * block_waves, lds, stream>>>(                             \
       q, kc, vc, item_ctx, table, width, part_o, part_ml, out, nh, nkv, bs_shift, window, scale_log2, num_splits, chunks,  \
-      ARGS, live_items, waves_wanted)
+      ARGS, live_items, waves_wanted, step_flags)
 #define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                \
   do {                                                      \
     if (streamed)                                           \
@@ -569,17 +593,17 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, hipStream_t stream);
+                         int waves_wanted, const int* step_flags, hipStream_t stream);
 
 extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                                         const int* block_table, int table_width, void* out, float* part_o,
                                         float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
                                         float scale, int split_keys, int num_splits, int max_ctx,
                                         const int* live_items, int full_splits, int waves_wanted,
-                                        hipStream_t stream) {
+                                        const int* step_flags, hipStream_t stream) {
   return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
                        bs, window, scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted,
-                       stream);
+                       step_flags, stream);
 }
 
 // Head sizes and groupings for which the decode kernel can take the norm, the rotary encoding and
@@ -598,7 +622,7 @@ extern "C" int me_attention_decode_fused_bf16(const void* qkv, const float* q_w,
                                               float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
                                               float scale, int split_keys, int num_splits, int max_ctx,
                                               const int* live_items, int full_splits, int waves_wanted,
-                                              hipStream_t stream) {
+                                              const int* step_flags, hipStream_t stream) {
   if (nkv <= 0 || nh <= 0 || nh % nkv || !me_attention_decode_fused_supported(d, bs, rope_table ? rotary_dim : 0, nh / nkv))
     return me_fail("me_attention_decode_fused_bf16: head_dim=%d block_size=%d rotary_dim=%d heads=%d/%d not supported", d,
                    bs, rotary_dim, nh, nkv);
@@ -611,14 +635,15 @@ extern "C" int me_attention_decode_fused_bf16(const void* qkv, const float* q_w,
   fa.k_cache_w = (bf16_t*)k_cache;
   fa.v_cache_w = (bf16_t*)v_cache;
   return decode_common(qkv, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
-                       bs, window, scale, split_keys, num_splits, max_ctx, &fa, live_items, full_splits, waves_wanted, stream);
+                       bs, window, scale, split_keys, num_splits, max_ctx, &fa, live_items, full_splits, waves_wanted, step_flags,
+                       stream);
 }
 
 static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, hipStream_t stream) {
+                         int waves_wanted, const int* step_flags, hipStream_t stream) {
   if (items <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_decode_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
@@ -673,7 +698,8 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
 #define ME_DECODE_CASE(DD)                                                                                      \
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
-                      depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, streamed, stream);   \
+                      depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, streamed, step_flags, \
+                      stream);                                                                                  \
     break;
   switch (d) {
     ME_DECODE_CASE(32)

@@ -219,6 +219,7 @@ class Core {
   std::vector<StepItem>& step() { return step_; }
   void check_step(int vocab_size, bool scan_pages) const;
   StepLayout layout(const std::vector<int>* widths, int pad_items) const;
+  int step_flags() const;
   void pack(int32_t* dst, const StepLayout& lay, int spare_page, int spare_slot) const;
   void refill(int32_t* dst, const StepLayout& lay, std::vector<RowMemo>& rows, int spare_page, int spare_slot) const;
   uint64_t draw_key(const Request* r) const;

@@ -393,7 +393,7 @@ class Run {
       partials(sp, part_o, part_ml);
       ok(me_attention_decode_fused_bf16(qkv, q_w, k_w, rope, rd, eps, owns ? 1 : 0, kc, vc, idx(s_.lay.item_ctx), table, width, out,
                                         part_o, part_ml, items, nh, nkv, d, bs, window, scale, sp.split_keys, sp.num_splits,
-                                        s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves, stream_));
+                                        s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves, idx(s_.lay.live_items) + 1, stream_));
       return;
     }
     void* q = arena_.take((size_t)t_ * nh * d * elem_);
@@ -411,7 +411,7 @@ class Run {
       partials(sp, part_o, part_ml);
       ok(me_attention_decode_bf16(q, kc, vc, idx(s_.lay.item_ctx), table, width, out, part_o, part_ml, items, nh, nkv, d, bs, window,
                                   scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
-                                  stream_));
+                                  idx(s_.lay.live_items) + 1, stream_));
       return;
     }
     if (mfma) {

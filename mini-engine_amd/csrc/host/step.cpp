@@ -3,7 +3,7 @@
 //
 // Sections of the buffer, in order (T tokens, B items, R wanted rows, G groups of width W_g):
 //   token_ids[T] positions[T] token_item[T] want_rows[R] item_start[B+1] item_ctx[B] state_slots[B]
-//   live_items[1] temperatures[R] (float bits) sample_keys[R] (64 bits each, 8-byte aligned)
+//   live_items[2] (the live items; bit 0 of the second word: the items share pages) temperatures[R] (float bits) sample_keys[R] (64 bits each, 8-byte aligned)
 //   token_source[T] (-1: the token's id is token_ids[t]; r >= 0: it is the r-th token the step before drew,
 //   which is still on the device)
 //   block_table_0[B, W_0] ... block_table_{G-1}[B, W_{G-1}]
@@ -33,7 +33,7 @@ StepLayout StepLayout::make(int tokens, int items, int rows, const std::vector<i
   section(l.item_start, items + 1);
   section(l.item_ctx, items);
   section(l.state_slots, items);
-  section(l.live_items, 1);
+  section(l.live_items, 2);
   section(l.temperatures, rows);
   at += at & 1;  // the keys are read as 64-bit values
   section(l.sample_keys, 2 * rows);
@@ -123,6 +123,19 @@ StepLayout Core::layout(const std::vector<int>* widths, int pad_items) const {
   return StepLayout::make(tokens, (int)step_.size() + pad_items, rows, widths ? *widths : w);
 }
 
+// What the kernels of a step may want to know of it beside its indices. Bit 0: a quarter or more of the keys that the
+// step's items read lie in pages that came out of the prefix cache, pages that other items read too: decode attention
+// then loads keys and values so that they stay in the caches (ordinary loads), not as data that passes through once.
+int Core::step_flags() const {
+  long long cached = 0, keys = 0;
+  for (const StepItem& it : step_) {
+    const int ctx = it.start + it.count;
+    keys += ctx;
+    cached += std::min(it.request->num_cached, ctx);
+  }
+  return cached > 0 && 4 * cached >= keys ? 1 : 0;
+}
+
 void Core::pack(int32_t* dst, const StepLayout& lay, int spare_page, int spare_slot) const {
   std::fill(dst, dst + lay.total, 0);
   std::fill_n(dst + lay.token_source, lay.tokens, -1);
@@ -171,6 +184,7 @@ void Core::pack(int32_t* dst, const StepLayout& lay, int spare_page, int spare_s
   }
   dst[lay.item_start + lay.items] = cursor;
   dst[lay.live_items] = live;
+  dst[lay.live_items + 1] = step_flags();
 }
 
 // The indices of a decode-only step written into a buffer that still holds those of the last step
@@ -241,6 +255,7 @@ void Core::refill(int32_t* dst, const StepLayout& lay, std::vector<RowMemo>& row
     memo.written = written;
   }
   dst[lay.live_items] = live;
+  dst[lay.live_items + 1] = step_flags();
 }
 
 }  // namespace me

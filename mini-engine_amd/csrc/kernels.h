@@ -33,13 +33,14 @@ int me_attention_prefill_columns(int wide);
 int me_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                              const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                              int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
-                             int max_ctx, const int* live_items, int full_splits, int waves_wanted, hipStream_t stream);
+                             int max_ctx, const int* live_items, int full_splits, int waves_wanted, const int* step_flags,
+                             hipStream_t stream);
 int me_attention_decode_fused_bf16(const void* qkv, const float* q_w, const float* k_w, const float* rope_table,
                                    int rotary_dim, float eps, int write_kv, void* k_cache, void* v_cache, const int* item_ctx,
                                    const int* block_table, int table_width, void* out, float* part_o, float* part_ml,
                                    int items, int nh, int nkv, int d, int bs, int window, float scale, int split_keys,
                                    int num_splits, int max_ctx, const int* live_items, int full_splits, int waves_wanted,
-                                   hipStream_t stream);
+                                   const int* step_flags, hipStream_t stream);
 int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items, const int* block_table,
                               int table_width, void* out, const int* work, const int* bundle_first, int num_bundles,
                               float* part_o, float* part_ml, const int* token_chunks, int max_chunks, int num_tokens, int nh,

@@ -772,10 +772,11 @@ def _decode_split_plan(items: int, kv_units: int, max_ctx: int, live):
 
 
 def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: float, window: int, max_ctx: int,
-                          out: torch.Tensor | None = None, live=None) -> torch.Tensor:
+                          out: torch.Tensor | None = None, live=None, step_flags: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of one new token per item over its cached keys: q [items, nh, d] bfloat16,
     item_ctx int32 [items] (keys per item, the new one included, each <= max_ctx). ``live``: see
-    :func:`_decode_split_plan`."""
+    :func:`_decode_split_plan`. ``step_flags``: None, or a device int32 whose bit 0 says that the items share
+    pages (a large launch then loads keys and values with ordinary loads instead of non-temporal ones)."""
     _want(q, "q", torch.bfloat16, (None, None, None))
     items, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -794,7 +795,7 @@ def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: flo
     check(lib().me_attention_decode_bf16(
         _p(q), _p(k_cache), _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out),
         _p(part_o), _p(part_ml), _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys),
-        _i(num_splits), _i(max_ctx), _p(live_count), _i(full_splits), _i(DECODE_WAVES), _stream()))
+        _i(num_splits), _i(max_ctx), _p(live_count), _i(full_splits), _i(DECODE_WAVES), _p(step_flags), _stream()))
     return out
 
 
@@ -805,10 +806,12 @@ def attention_decode_fused_supported(head_dim: int, block_size: int, rotary_dim:
 
 def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write_kv: bool, k_cache, v_cache, item_ctx,
                                 block_table, num_heads: int, scale: float, window: int, max_ctx: int,
-                                out: torch.Tensor | None = None, live=None) -> torch.Tensor:
+                                out: torch.Tensor | None = None, live=None,
+                                step_flags: torch.Tensor | None = None) -> torch.Tensor:
     """One new token per item, from the raw q/k/v projection: what :func:`qk_norm_rope_scatter` followed
     by :func:`attention_decode_bf16` compute, in one launch. qkv [items, (nh + 2 nkv) d] bfloat16
-    (or [items, nh d] with ``write_kv`` off). ``live``: see :func:`_decode_split_plan`."""
+    (or [items, nh d] with ``write_kv`` off). ``live``: see :func:`_decode_split_plan`; ``step_flags`` as in
+    :func:`attention_decode_bf16`."""
     nkv, bs, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     nh = num_heads
     _want(qkv, "qkv", torch.bfloat16, (None, ((nh + 2 * nkv) if write_kv else nh) * d))
@@ -838,7 +841,7 @@ def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write
         _p(qkv), _p(q_weight), _p(k_weight), _p(rope), _i(rd), _f(eps), _i(1 if write_kv else 0), _p(k_cache),
         _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out), _p(part_o), _p(part_ml),
         _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys), _i(num_splits), _i(max_ctx),
-        _p(live_count), _i(full_splits), _i(DECODE_WAVES), _stream()))
+        _p(live_count), _i(full_splits), _i(DECODE_WAVES), _p(step_flags), _stream()))
     return out
 
 

@@ -22,7 +22,7 @@ class RawItem:
 
 
 def raw_layout(t: int, b: int, r: int, widths: list[int]) -> dict:
-    sizes = (t, t, t, r, b + 1, b, b, 1, r)
+    sizes = (t, t, t, r, b + 1, b, b, 2, r)  # live_items: the count, then the step's flags
     lay, at = {"tokens": t, "items": b, "rows": r, "widths": list(widths)}, 0
     for name, n in zip(SECTIONS, sizes):
         lay[name] = at

@@ -794,6 +794,33 @@ def test_attention_decode_mfma(nh, nkv, d, bs, window):
         assert_attention_close(out, want)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs,max_ctx", [(16, 8, 128, 16, 8192), (8, 8, 64, 32, 16384)])
+def test_attention_decode_of_a_launch_large_enough_to_stream(nh, nkv, d, bs, max_ctx):
+    """A launch whose items may hold 256 MB and more of keys and values loads them as data that passes through once,
+    unless the step's flags say that the items share pages: the same result either way, and as without flags."""
+    dtype = torch.bfloat16
+    ctxs = [1, 16, 17, 33, 100, 255, 64, 65, 700, 1000]
+    assert len(ctxs) * max_ctx * nkv * d * 4 >= 256 << 20
+    items = [(c - 1, 1) for c in ctxs]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=200)
+    fill_new(k_cache, v_cache, tables, ks, vs, items, bs)
+    g = torch.Generator().manual_seed(10)
+    qs = [torch.randn(1, nh, d, generator=g).to(dtype) for _ in items]
+    scale = d**-0.5
+    want = dense_reference(qs, ks, vs, items, scale, 0)
+    item_ctx = torch.tensor(ctxs, dtype=torch.int32)
+    wide = torch.zeros(len(items), max_ctx // bs, dtype=torch.int32)
+    wide[:, : table_t.shape[1]] = table_t
+    outs = []
+    for flags in (None, 0, 1):
+        word = None if flags is None else dev(torch.tensor([flags], dtype=torch.int32))
+        out = K().attention_decode_bf16(dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide), scale, 0,
+                                        max_ctx, step_flags=word)
+        assert_attention_close(out, want)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])  # the kind of load changes no bit
+
+
 @pytest.mark.parametrize("nh,nkv,d,bs", [(16, 8, 128, 16), (4, 2, 64, 16), (6, 1, 96, 32)])
 def test_attention_decode_with_fewer_live_items_than_the_grid_holds(nh, nkv, d, bs):
     """A launch laid out for as few as `least` live items (a replayed graph: the rest is padding) has

@@ -129,6 +129,36 @@ def test_prefix_hit_skips_cached_tokens():  # :121-129
     assert b.block_table[:2] == a.block_table[:2]
 
 
+def test_a_step_says_when_its_items_read_pages_out_of_the_prefix_cache():
+    """The second word of the packed ``live_items`` section: bit 0 is set when a quarter or more of the keys that the
+    step's items read came out of the prefix cache (decode attention then keeps to loads that stay in the caches)."""
+    import numpy as np
+
+    def flags(s: Scheduler) -> int:
+        lay = s.core.step_layout()
+        arr = np.zeros(lay["total"], dtype=np.int32)
+        s.core.step_pack(arr)
+        assert arr[lay["live_items"]] == lay["items"]
+        return int(arr[lay["live_items"] + 1])
+
+    s = make()
+    a = add(s, 9, max_tokens=8)
+    batch = s.schedule()
+    assert flags(s) == 0  # nothing cached yet
+    s.postprocess(batch, [0])
+    b = add(s, 11, max_tokens=8)
+    batch = s.schedule()  # a decodes, b brings the 3 tokens behind its 8 cached ones: 8 of 10 + 11 keys
+    assert b.num_cached_tokens == 8 and flags(s) == 1
+    s.postprocess(batch, [0, 0])
+    for _ in range(3):  # both decode: 8 cached of 11 + 12 keys and more
+        batch = s.schedule()
+        assert flags(s) == 1
+        s.postprocess(batch, [0, 0])
+    c = add(s, 30, max_tokens=2, first=500)  # a long request of its own: 8 of (15 + 15 + 30) keys are no quarter
+    batch = s.schedule()
+    assert c.num_cached_tokens == 0 and flags(s) == 0
+
+
 def test_rejects_requests_that_can_never_fit():  # :132-137
     s = make(num_blocks=2, max_model_len=64)
     with pytest.raises(ValueError, match="KV blocks"):
