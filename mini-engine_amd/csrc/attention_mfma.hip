@@ -673,15 +673,15 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   int block_waves = (num_splits > 1 && num_splits <= DECODE_BLOCK_WAVES(d)) ? num_splits : 1;
   const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
   if ((size_t)block_waves * heads_most * (d + 2) * sizeof(float) > 48 * 1024) block_waves = 1;  // LDS for the sum
+  static int cus = 0;
+  if (cus <= 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0)
+      cus = 256;
+  }
+  const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);  // with every split of an (item, kv head) in one block
   if (block_waves > 1) {
-    static int cus = 0;
-    if (cus <= 0) {
-      int dev = 0;
-      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-          cus <= 0)
-        cus = 256;
-    }
-    const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);
     const long long rounds = (blocks + cus - 1) / cus;
     if (blocks > cus && blocks * 10 < rounds * cus * 9) block_waves = 1;  // rounds that are less than nine tenths full
   }
@@ -689,10 +689,10 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   // megabytes over a full chip (batch 64 at 4,096: 6.21 -> 5.97 ms a step; batch 8 and 16 at 16,384: 3.54 -> 3.41 and
   // 6.0 -> 5.6), and no faster or slower where it does not (batch 8 at 4,096, 134 MB: level; 33 MB and less: 0.4-0.8% slower;
   // 160 to 224 blocks of 5 to 7 waves on 256 compute units, batch 20 to 28: 1-5% slower). The size goes by the longest context
-  // the launch may hold. (An instance of the kernel of its own: as a branch inside one kernel it cost steps that do not take
-  // it up to 4%.)
+  // the launch may hold. (Instances of the kernel of their own: as a branch around every load of one kernel it cost steps that
+  // do not take it up to 4%.)
   const long long kv_bytes = (long long)items * max_ctx * nkv * d * 4;
-  const int streamed = kv_bytes >= (256ll << 20) && (block_waves == 1 || (long long)items * nkv * ((nh / nkv + 15) / 16) >= 256);
+  const int streamed = kv_bytes >= (256ll << 20) && (block_waves == 1 || blocks >= cus);
   const float sl = scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
 #define ME_DECODE_CASE(DD)                                                                                      \
