@@ -159,11 +159,12 @@ int choose_norm_fusion(int dtype, int m, int rows_of_w, int k, int pending, int 
 // rsqrt(mean + eps). Measured on the same GPU in turns, layers of 1,024 x 2,048 (o), 1,024 x 3,072 (down), 4,096 and
 // 2 x 3,072 x 1,024: the deltas take 6.7 us instead of 4.7 and the products behind them 0.6-0.9 more, the two add-and-norms
 // (4.6 each under the profiler, about 3 inside a graph) are gone: a step of 3 / 4 / 8 items 1.246 -> 1.198 / 1.435 -> 1.387 /
-// 1.781 -> 1.743 ms. With more rows the whole-k deltas cost more than the launches they save (16 items: 6,600 -> 6,570 tokens/s;
-// 24 and 32: 11,430 -> 10,300 and 12,290 -> 11,000), and so they do on weights that take longer to stream than a launch
-// costs (2,048 x 6,144 at 8 rows: 10.7 us against 7.3 in runs; a step of the 32B shape at batch 8, whose 320 blocks of 16
-// columns are a round and a quarter of the compute units, 12% slower): up to 8 rows, weights below 16 MiB.
-constexpr int kCarryMinRows = 3, kCarryMaxRows = 8;
+// 1.778 -> 1.727 ms, of 10 / 12 / 16 items at a context of 2,048 1.604 -> 1.555 / 1.649 -> 1.599 / 1.844 -> 1.809. From 17 rows
+// on (two tiles of rows a block) the whole-k deltas cost more than the launches they save (20 / 24 / 32 items: 1.97 -> 2.09 /
+// 2.11 -> 2.24 / 1.81 -> 1.97 ms), and so they do on weights that take longer to stream than a launch costs (2,048 x 6,144 at 8
+// rows: 10.7 us against 7.3 in runs; a step of the 32B shape at batch 8, whose 320 blocks of 16 columns are a round and a
+// quarter of the compute units, 12% slower): up to 16 rows, weights below 16 MiB.
+constexpr int kCarryMinRows = 3, kCarryMaxRows = 16;
 bool choose_carried_norm(int dtype, int m, int n, int k, int next_rows_of_w, int next_gated, int units, bool aligned) {
   if (dtype != kBF16 || !aligned || m < kCarryMinRows || m > kCarryMaxRows || k % 8 || n % 8) return false;
   if (!streams(m, n, k) || (int64_t)n * k >= kStreamMinElements) return false;

@@ -114,7 +114,7 @@ def test_a_norm_is_left_to_the_product_behind_it_only_where_that_product_scales_
             carried = K.carried_norm_choice(BF16, rows, n, k, next_rows, gated, 256)
             seen.add(carried)
             if carried:
-                assert 3 <= rows <= 8 and n * k * 2 < 16 << 20
+                assert 3 <= rows <= 16 and n * k * 2 < 16 << 20
                 kernel, _, partial, gate_after = K.product_choice(BF16, K.ROLE_PLAIN, rows, next_rows, n, gated, BF16, 256)
                 assert kernel in (K.PRODUCT_SMALL, K.PRODUCT_STREAM) and not gate_after and not partial
             assert not K.carried_norm_choice(F32, rows, n, k, next_rows, gated, 256)
@@ -123,13 +123,13 @@ def test_a_norm_is_left_to_the_product_behind_it_only_where_that_product_scales_
 
 
 def test_the_tiny_models_of_the_gpu_tests_leave_their_norms_to_the_products_behind():
-    """The GPU tests replay steps of three to eight tokens on these models: the carried norm is what they run there
+    """The GPU tests replay steps of three to sixteen tokens on these models: the carried norm is what they run there
     (all but E, whose widths no kernel of this kind takes)."""
     from conftest import tiny_configs
 
     for name, cfg in tiny_configs().items():
         hidden, inter, width = cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads * cfg.head_dim
         qkv_rows = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
-        for rows in (3, 8):
+        for rows in (3, 8, 16):
             assert K.carried_norm_choice(BF16, rows, hidden, width, 2 * inter, True, 256) == (name != "E"), name
             assert K.carried_norm_choice(BF16, rows, hidden, inter, qkv_rows, False, 256) == (name != "E"), name
