@@ -121,7 +121,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const T* __restric
     T v[4];
   };
   const int nvec = dim / 4;
-  float4 s[4];
+  float4 s[4], wv[4];  // (the norm's weight is requested with the row, not behind the sum over the block: the tail waits for nothing)
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
@@ -129,6 +129,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const T* __restric
     s[it] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (v < nvec) {
       s[it] = *reinterpret_cast<const float4*>(xr + 4 * v);
+      wv[it] = *reinterpret_cast<const float4*>(w + 4 * v);
       if (dr) {
         const Pack d = *reinterpret_cast<const Pack*>(dr + 4 * v);
         s[it].x += to_float(d.v[0]), s[it].y += to_float(d.v[1]), s[it].z += to_float(d.v[2]), s[it].w += to_float(d.v[3]);
@@ -163,10 +164,9 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const T* __restric
   for (int it = 0; it < 4; ++it) {
     const int v = threadIdx.x + it * blockDim.x;
     if (v < nvec) {
-      const float4 wv = *reinterpret_cast<const float4*>(w + 4 * v);
       Pack o;
-      o.v[0] = from_float<T>(s[it].x * inv * wv.x), o.v[1] = from_float<T>(s[it].y * inv * wv.y);
-      o.v[2] = from_float<T>(s[it].z * inv * wv.z), o.v[3] = from_float<T>(s[it].w * inv * wv.w);
+      o.v[0] = from_float<T>(s[it].x * inv * wv[it].x), o.v[1] = from_float<T>(s[it].y * inv * wv[it].y);
+      o.v[2] = from_float<T>(s[it].z * inv * wv[it].z), o.v[3] = from_float<T>(s[it].w * inv * wv[it].w);
       *reinterpret_cast<Pack*>(hr + 4 * v) = o;
     }
   }

@@ -124,6 +124,25 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
       }
   };
 
+  // A delta that adds itself to the stream (carry.x): the elements of the stream and of the norm's weight that this lane
+  // will add to and multiply with at the end are requested here, ahead of everything, so that the kernel's tail does not
+  // wait for memory once more. (Whole groups of four columns only; a ragged edge is read at the end.)
+  float4 x_early[AUX ? MT : 1][AUX ? NT : 1], wn_early[AUX ? NT : 1];
+  if constexpr (AUX && !SWIGLU && sizeof(OutT) == 4) {
+    if (carry.x && wk == 0 && (N & 3) == 0) {
+      const size_t row0 = (size_t)blockIdx.z * (16 * MT);
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int nb = n0 + 16 * i + 4 * g;
+        if (nb < c1 && nb + 3 < N) {
+          wn_early[i] = *reinterpret_cast<const float4*>(carry.w_norm + nb);
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+            if (t * 16 + r < M) x_early[t][i] = *reinterpret_cast<const float4*>(carry.x + (row0 + t * 16 + r) * N + nb);
+        }
+      }
+    }
+  }
   // (the scheduling barriers keep the stages' loads in the order of their use: the waits count loads in flight)
 #pragma unroll
   for (int p = 0; p < STAGES; ++p) {
@@ -203,8 +222,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
             float* xp = carry.x + (row0 + m) * N + nb;
             bf16_t* hp = carry.h + (row0 + m) * N + nb;
             if (nb + 3 < N && (N & 3) == 0) {
-              float4 v = *reinterpret_cast<const float4*>(xp);
-              const float4 wv = *reinterpret_cast<const float4*>(carry.w_norm + nb);
+              float4 v = x_early[t][i];
+              const float4 wv = wn_early[i];
               v.x += acc[t][i][0], v.y += acc[t][i][1], v.z += acc[t][i][2], v.w += acc[t][i][3];
               *reinterpret_cast<float4*>(xp) = v;
               uint2 packed;
