@@ -589,6 +589,46 @@ extern "C" int me_attention_mfma_supported(int d, int bs) {
 // cover it. live_items (device, or null): how many of the items are live, for a launch whose grid was
 // laid out for fewer items than it holds; then full_splits is the number of splits of a step with every
 // item live and waves_wanted the number of waves that the live items' splits should come to.
+// How many splits one block of a decode launch takes on, a wave each (1: a wave a block, and a second kernel or the
+// product behind adds up the splits).
+// Few splits (a step of many items): one block takes all splits of its heads, a wave each, adds their
+// results up itself and writes the output; the second kernel is not needed then. Such a block is a whole
+// (item, kv head) of work and a compute unit takes in only so much per microsecond, so this pays only where the
+// blocks divide evenly among the compute units: 512 blocks on 256 units yes (batch 64: 5% ahead of one wave a
+// block and the second kernel), and up to 256 (a block a unit: 17 to 32 items, 3-7% ahead), but 320 or 384 no
+// (batch 40: 8,280 -> 8,850 tokens/s with a wave a block: a unit had one block or two, and the step waited for
+// the units with two).
+static int decode_compute_units() {
+  static int cus = 0;
+  if (cus <= 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0)
+      cus = 256;
+  }
+  return cus;
+}
+
+static int decode_block_waves(int items, int nh, int nkv, int d, int num_splits) {
+  int block_waves = (num_splits > 1 && num_splits <= DECODE_BLOCK_WAVES(d)) ? num_splits : 1;
+  const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
+  if ((size_t)block_waves * heads_most * (d + 2) * sizeof(float) > 48 * 1024) block_waves = 1;  // LDS for the sum
+  const int cus = decode_compute_units();
+  const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);  // with every split of an (item, kv head) in one block
+  if (block_waves > 1) {
+    const long long rounds = (blocks + cus - 1) / cus;
+    if (blocks > cus && blocks * 10 < rounds * cus * 9) block_waves = 1;  // rounds that are less than nine tenths full
+  }
+  return block_waves;
+}
+
+// Whether a decode launch of these sizes leaves one partial result per split in part_o / part_ml (which the second
+// kernel, or me_attention_out_product_bf16 in its place, adds up): the launches that may be given no `out`.
+extern "C" int me_attention_decode_leaves_parts(int items, int nh, int nkv, int d, int num_splits) {
+  if (items <= 0 || nh <= 0 || nkv <= 0 || nh % nkv) return 0;
+  return decode_block_waves(items, nh, nkv, d, num_splits) == 1;
+}
+
 static int decode_common(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
@@ -663,28 +703,11 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   const int run_keys = (((max_ctx + run_splits - 1) / run_splits + 15) / 16) * 16;
   const long long run_waves = (long long)items * nkv * ((nh / nkv + 15) / 16) * run_splits;
   const int depth = (run_keys <= 256 || run_waves <= 1024) ? 2 : 1;
-  // Few splits (a step of many items): one block takes all splits of its heads, a wave each, adds their
-  // results up itself and writes the output; the second kernel is not needed then. Such a block is a whole
-  // (item, kv head) of work and a compute unit takes in only so much per microsecond, so this pays only where the
-  // blocks divide evenly among the compute units: 512 blocks on 256 units yes (batch 64: 5% ahead of one wave a
-  // block and the second kernel), and up to 256 (a block a unit: 17 to 32 items, 3-7% ahead), but 320 or 384 no
-  // (batch 40: 8,280 -> 8,850 tokens/s with a wave a block: a unit had one block or two, and the step waited for
-  // the units with two).
-  int block_waves = (num_splits > 1 && num_splits <= DECODE_BLOCK_WAVES(d)) ? num_splits : 1;
-  const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
-  if ((size_t)block_waves * heads_most * (d + 2) * sizeof(float) > 48 * 1024) block_waves = 1;  // LDS for the sum
-  static int cus = 0;
-  if (cus <= 0) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        cus <= 0)
-      cus = 256;
-  }
-  const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);  // with every split of an (item, kv head) in one block
-  if (block_waves > 1) {
-    const long long rounds = (blocks + cus - 1) / cus;
-    if (blocks > cus && blocks * 10 < rounds * cus * 9) block_waves = 1;  // rounds that are less than nine tenths full
-  }
+  const int block_waves = decode_block_waves(items, nh, nkv, d, num_splits);
+  if (!out && block_waves > 1)
+    return me_fail("me_attention_decode_bf16: a launch whose blocks add up their splits themselves needs `out`");
+  const int cus = decode_compute_units();
+  const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);
   // Keys and values pass through once: loaded as non-temporal they arrive faster where the launch streams hundreds of
   // megabytes over a full chip (batch 64 at 4,096: 6.21 -> 5.97 ms a step; batch 8 and 16 at 16,384: 3.54 -> 3.41 and
   // 6.0 -> 5.6), and no faster or slower where it does not (batch 8 at 4,096, 134 MB: level; 33 MB and less: 0.4-0.8% slower;
@@ -712,6 +735,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
 #undef ME_DECODE_CASE
   if (me_check_launch("me_attention_decode_bf16")) return 1;
   if (block_waves > 1) return 0;  // the blocks held all splits of their heads and wrote the output themselves
+  if (!out) return 0;             // the caller adds up the splits (me_attention_out_product_bf16)
   attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d);
   return me_check_launch("me_attention_decode_combine");
 }
@@ -1229,4 +1253,202 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
     return me_check_launch("me_attention_prefill_combine");
   }
   return 0;
+}
+
+// ------------------------------------------------------------------------------------ the splits' sum inside the output projection
+// For steps of very few items: the output projection behind decode attention reads the splits' partial results itself,
+// so that the kernel that adds them up is not launched (a launch costs such a step more than the kernel's work). The
+// heads are dealt to runs of k (HPR heads a run); a block owns one run and 64 output columns, for all rows. It asks
+// for everything at its head (its weights, its heads' partial results, their statistics: one trip to memory), adds up
+// the splits of each (row, head) pair as attention_decode_combine_kernel does, rounds the result to bfloat16 as that
+// kernel's output is, and multiplies: parts[run][row][n] = sum over the run's k of out[row][k] W[n][k], float32, for the
+// next add-and-norm to add up in their order. Every block of a run adds up the run's heads again, so this pays for narrow
+// products only (measured on 16 heads of 128 and 1,024 columns, one row, 64 splits: 16 runs x 16 blocks of columns 2.8%
+// of a step ahead of the two kernels, 8 runs x 16 1.7%, 16 x 8 blocks of 128 columns 1.2%, 8 x 8 0.5% behind; with
+// two rows 1.4% behind at best).
+#define OUT_MAX_SPLITS 128  // splits a (row, head) pair may have here
+#define OUT_MAX_ROWS 4
+#define OUT_EARLY 16        // partial results a thread asks for before it knows their weights
+
+template <int D, int HPR>
+__global__ __launch_bounds__(256) void attention_out_product_kernel(const float* __restrict__ part_o,
+                                                                    const float* __restrict__ part_ml, int num_splits,
+                                                                    const bf16_t* __restrict__ W, float* __restrict__ parts,
+                                                                    int items, int nh, int N, int gpp) {
+  constexpr int QUADS = D / 4;         // threads across a head's outputs, four each
+  constexpr int GROUPS = 256 / QUADS;  // groups of such threads; gpp of them share the splits of one (row, head) pair
+  constexpr int XROW = HPR * D + 8;    // LDS row stride in elements: 16 bytes off a multiple of 128
+  __shared__ float2 ml[GROUPS][OUT_MAX_SPLITS];  // statistics by pair and split (pairs <= GROUPS)
+  __shared__ float red[8];                        // maxima of the half-waves
+  __shared__ float4_t partial[256];
+  __shared__ float pdenom[GROUPS];
+  __shared__ __attribute__((aligned(16))) uint16_t xs[OUT_MAX_ROWS][XROW];
+  const int run = blockIdx.x, head0 = run * HPR;
+  const int heads_here = min(HPR, nh - head0);
+  const int tid = threadIdx.x, lane = tid & (ME_WAVE - 1), wave = tid / ME_WAVE, r = lane & 15, g = lane >> 4;
+  const size_t K = (size_t)nh * D;
+  const int n0 = ((int)blockIdx.y * 4 + wave) * 16;
+
+  // ---- the wave's weights, as the first product operand: lane -> row n0 + r, eight k from 32 c + 8 g
+  bf16x8_t w[HPR][D / 32];
+#pragma unroll
+  for (int hl = 0; hl < HPR; ++hl)
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+      w[hl][c] = bf16x8_t{};
+      if (n0 + r < N && hl < heads_here)
+        w[hl][c] = *reinterpret_cast<const bf16x8_t*>(W + (size_t)(n0 + r) * K + (size_t)(head0 + hl) * D + c * 32 + g * 8);
+    }
+
+  // ---- this thread's (row, head) pair and its share of the pair's splits
+  const int qd = tid % QUADS, grp = tid / QUADS;
+  const int pair = grp / gpp, sub = grp % gpp;
+  const int row = pair / HPR, hl_own = pair % HPR;
+  const bool pair_ok = row < items && hl_own < heads_here;
+  const size_t unit = (size_t)row * nh + head0 + hl_own;
+  const float* po = part_o + unit * num_splits * D + qd * 4;
+  float4_t early[OUT_EARLY];
+#pragma unroll
+  for (int i = 0; i < OUT_EARLY; ++i) {
+    const int sp = sub + i * gpp;
+    early[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    if (pair_ok && sp < num_splits) early[i] = *reinterpret_cast<const float4_t*>(po + (size_t)sp * D);
+  }
+  // the statistics of the pair's splits, dealt to the pair's threads; their maximum over the pair
+  const int pair_threads = QUADS * gpp, in_pair = sub * QUADS + qd;  // 32 or more threads
+  float big = -INFINITY;
+  for (int sp = in_pair; sp < num_splits; sp += pair_threads) {
+    float2 st = make_float2(-INFINITY, 0.f);
+    if (pair_ok) st = *reinterpret_cast<const float2*>(part_ml + (unit * num_splits + sp) * 2);
+    ml[pair][sp] = st;
+    if (st.y > 0.f) big = fmaxf(big, st.x);  // an empty split has no weight
+  }
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) big = fmaxf(big, __shfl_xor(big, off, ME_WAVE));  // over the half-wave
+  if ((lane & 31) == 0) red[tid / 32] = big;
+  __syncthreads();
+  {
+    const int first = pair * pair_threads / 32;
+    big = red[first];
+    for (int i = 1; i < pair_threads / 32; ++i) big = fmaxf(big, red[first + i]);
+  }
+  float4_t accv = {0.f, 0.f, 0.f, 0.f};
+  float dsum = 0.f;
+  if (pair_ok) {
+#pragma unroll
+    for (int i = 0; i < OUT_EARLY; ++i) {
+      const int sp = sub + i * gpp;
+      if (sp < num_splits) {
+        const float2 st = ml[pair][sp];
+        const float wgt = st.y > 0.f ? fast_exp2(st.x - big) : 0.f;
+        dsum += wgt * st.y;
+        accv[0] += wgt * early[i][0];
+        accv[1] += wgt * early[i][1];
+        accv[2] += wgt * early[i][2];
+        accv[3] += wgt * early[i][3];
+      }
+    }
+    for (int sp = sub + OUT_EARLY * gpp; sp < num_splits; sp += gpp) {
+      const float2 st = ml[pair][sp];
+      const float wgt = st.y > 0.f ? fast_exp2(st.x - big) : 0.f;
+      const float4_t v = *reinterpret_cast<const float4_t*>(po + (size_t)sp * D);
+      dsum += wgt * st.y;
+      accv[0] += wgt * v[0];
+      accv[1] += wgt * v[1];
+      accv[2] += wgt * v[2];
+      accv[3] += wgt * v[3];
+    }
+  }
+  partial[tid] = accv;
+  if (qd == 0) pdenom[grp] = dsum;
+  __syncthreads();
+  if (pair_ok && sub == 0) {
+    float4_t total = accv;
+    float denom = dsum;
+    for (int i = 1; i < gpp; ++i) {
+      const float4_t v = partial[(grp + i) * QUADS + qd];
+      total[0] += v[0];
+      total[1] += v[1];
+      total[2] += v[2];
+      total[3] += v[3];
+      denom += pdenom[grp + i];
+    }
+    const float inv = denom > 0.f ? 1.f / denom : 0.f;  // no visible key at all: zeros, not NaN
+    *reinterpret_cast<short4_t*>(&xs[row][hl_own * D + qd * 4]) =
+        pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
+  }
+  __syncthreads();
+
+  // ---- parts[run][m][n] = sum_k W[n][k] out[m][k]: lane -> out row r (rows beyond the items are zeros)
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int hl = 0; hl < HPR; ++hl) {
+    if (hl >= heads_here) break;
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+      bf16x8_t xf = bf16x8_t{};
+      if (r < items) xf = *reinterpret_cast<const bf16x8_t*>(&xs[r][hl * D + c * 32 + g * 8]);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[hl][c], xf, acc, 0, 0, 0);
+    }
+  }
+  if (r < items) {
+    const int n = n0 + g * 4;
+    if (n < N) *reinterpret_cast<float4_t*>(parts + ((size_t)run * items + r) * N + n) = acc;  // N is a multiple of 4
+  }
+}
+
+// Heads per run of k, for at most `OUT_RUNS` runs.
+#define OUT_RUNS 16
+static int out_heads_per_run(int nh) {
+  int hpr = 1;
+  while ((nh + hpr - 1) / hpr > OUT_RUNS) hpr *= 2;
+  return hpr;
+}
+
+// How many runs of k (float32 partial sums) me_attention_out_product_bf16 writes for nh heads.
+extern "C" int me_attention_out_product_runs(int nh) {
+  if (nh <= 0) return 0;
+  const int hpr = out_heads_per_run(nh);
+  return (nh + hpr - 1) / hpr;
+}
+
+// Sizes that me_attention_out_product_bf16 takes: up to 4 rows, heads of 64 or 128, up to 128 splits, a width that is
+// a multiple of 8, and at most 8 (row, head) pairs a block.
+extern "C" int me_attention_out_product_supported(int items, int nh, int d, int n, int num_splits) {
+  if (items <= 0 || items > OUT_MAX_ROWS || nh <= 0 || (d != 64 && d != 128) || n <= 0 || n % 8) return 0;
+  if (num_splits <= 0 || num_splits > OUT_MAX_SPLITS) return 0;
+  const int hpr = out_heads_per_run(nh);
+  if (hpr > 4) return 0;
+  int pairs = 1;
+  while (pairs < items * hpr) pairs *= 2;
+  return pairs <= 8;  // 32 threads or more a pair, whatever the head size
+}
+
+// part_o float [items * nh, num_splits, d], part_ml float [items * nh, num_splits, 2]: what a decode attention launch
+// without `out` left. W bf16 [n, nh * d]. parts float [runs, items, n] (runs: me_attention_out_product_runs(nh)).
+extern "C" int me_attention_out_product_bf16(const float* part_o, const float* part_ml, int num_splits, const void* W,
+                                             float* parts, int items, int nh, int d, int n, hipStream_t stream) {
+  if (!me_attention_out_product_supported(items, nh, d, n, num_splits))
+    return me_fail("me_attention_out_product_bf16: items=%d heads=%d head_dim=%d width=%d splits=%d not supported", items, nh,
+                   d, n, num_splits);
+  if (((uintptr_t)W | (uintptr_t)part_o | (uintptr_t)parts) & 15)
+    return me_fail("me_attention_out_product_bf16: operands must start at multiples of 16 bytes");
+  const int hpr = out_heads_per_run(nh);
+  const int runs = (nh + hpr - 1) / hpr;
+  int pairs = 1;
+  while (pairs < items * hpr) pairs *= 2;
+  const int groups = 256 / (d / 4);
+  const int gpp = groups / pairs;
+  dim3 grid(runs, (n + 63) / 64);
+  const bf16_t* w = (const bf16_t*)W;
+#define ME_OUT_CASE(DD, HH) \
+  if (d == DD && hpr == HH) attention_out_product_kernel<DD, HH><<<grid, 256, 0, stream>>>(part_o, part_ml, num_splits, w, parts, items, nh, n, gpp);
+  ME_OUT_CASE(64, 1)
+  ME_OUT_CASE(64, 2)
+  ME_OUT_CASE(64, 4)
+  ME_OUT_CASE(128, 1)
+  ME_OUT_CASE(128, 2)
+  ME_OUT_CASE(128, 4)
+#undef ME_OUT_CASE
+  return me_check_launch("me_attention_out_product_bf16");
 }

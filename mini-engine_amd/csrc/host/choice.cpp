@@ -172,6 +172,18 @@ bool choose_carried_norm(int dtype, int m, int n, int k, int next_rows_of_w, int
   return !next.gate_after && (next.kernel == kProductSmall || next.kernel == kProductStream);
 }
 
+// One item: a decode layer is six launches of about 5 us whose work is a fraction of that, and one of them only adds up the
+// splits of attention. The output projection can do that at its head (me_attention_out_product_bf16), once per block of 64
+// columns and run of heads: the splits' partial results are read as many times as the product has blocks of columns,
+// which a narrow product bears (1,024 columns, 16 heads of 128, contexts of 1,024 / 2,304 / 4,096 / 8,192: a step of
+// one item 1.027 -> 0.984 / 1.038 -> 1.001 / 1.042 -> 1.013 / 1.175 -> 1.106 ms; two items: 1.185 -> 1.202, the
+// second row doubles what every block reads). Wider products are left to the two kernels: their blocks of columns would read
+// more partial results than the product has weights.
+constexpr int kSplitSumMaxRows = 1, kSplitSumMaxColumns = 1024;
+bool choose_split_sum_in_product(int dtype, int m, int n, bool aligned) {
+  return dtype == kBF16 && aligned && m <= kSplitSumMaxRows && n <= kSplitSumMaxColumns && n % 8 == 0;
+}
+
 }  // namespace me
 
 // out: kernel, runs, partial_sums, gate_after, adds_into
@@ -191,4 +203,8 @@ extern "C" int me_norm_fusion_choice(int dtype, int m, int rows_of_w, int k, int
 
 extern "C" int me_carried_norm_choice(int dtype, int m, int n, int k, int next_rows_of_w, int next_gated, int units, int aligned) {
   return me::choose_carried_norm(dtype, m, n, k, next_rows_of_w, next_gated, units, aligned != 0) ? 1 : 0;
+}
+
+extern "C" int me_split_sum_choice(int dtype, int m, int n, int aligned) {
+  return me::choose_split_sum_in_product(dtype, m, n, aligned != 0) ? 1 : 0;
 }

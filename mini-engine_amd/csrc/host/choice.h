@@ -46,6 +46,9 @@ int choose_norm_fusion(int dtype, int m, int rows_of_w, int k, int pending, int 
 // Whether a delta of the residual stream (m rows, n = hidden columns, k) adds itself to the stream and leaves the norm
 // behind it to the product after the norm (next_rows_of_w rows of hidden, gated or not): no add-and-norm kernel between.
 bool choose_carried_norm(int dtype, int m, int n, int k, int next_rows_of_w, int next_gated, int units, bool aligned);
+// Whether the output projection behind a decode attention of m items (n = hidden columns) adds up the attention's splits
+// itself, so that no kernel of its own does (sizes that the kernel takes are its own matter: me_attention_out_product_supported).
+bool choose_split_sum_in_product(int dtype, int m, int n, bool aligned);
 
 // Limits that the rules above share with the arena's sizing.
 constexpr int kSmallMaxRows = 64;      // what the small matrix-core kernel accepts

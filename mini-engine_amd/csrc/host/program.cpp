@@ -322,6 +322,19 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     pending_ = Pending();
+    if (attn_parts_.o) {  // decode attention left its splits to this product
+      const AttnParts a = attn_parts_;
+      attn_parts_ = AttnParts();
+      if (a.value != op.in || k != a.nh * a.d) throw Error(kBroken, "attention left its splits to a product that does not follow");
+      const int runs = me_attention_out_product_runs(a.nh);
+      parts_mark_ = a.mark;
+      float* parts = (float*)arena_.take((size_t)runs * t_ * n * 4);
+      ok(me_attention_out_product_bf16(a.o, a.ml, a.splits, op.p[1], parts, t_, a.nh, a.d, n, stream_));
+      pending_.parts = parts;
+      pending_.num_parts = runs;
+      pending_.stride = (long long)t_ * n;
+      return;
+    }
     if (next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ &&
         choose_carried_norm(dtype_, t_, n, k, (int)next_->i[0], (int)next_->i[2], compute_units(), true)) {
       // x += product in the product's epilogue, which also starts the norm behind it (choice.cpp)
@@ -379,9 +392,28 @@ class Run {
     void* out = bufs_[op.out];
     const void* qkv = bufs_[op.in];
     const bool mfma = dtype_ == kBF16 && me_attention_mfma_supported(d, bs) && group <= 16;
+    const size_t mark = arena_.used;
     auto partials = [&](const SplitPlan& sp, float*& part_o, float*& part_ml) {
       part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * d * 4);
       part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
+    };
+    // A decode step of very few items leaves the splits' partial results to the output projection behind it: no kernel
+    // of its own adds them up.
+    auto leaves_to_product = [&](const SplitPlan& sp, float* part_o, float* part_ml) {
+      if (!(next_ && next_->kind == kOpLinearDelta && next_->in == op.out && next_->i[0] == h_ && next_->i[1] == (int64_t)nh * d &&
+            items == t_ && choose_split_sum_in_product(dtype_, items, h_, true) &&
+            me_attention_decode_leaves_parts(items, nh, nkv, d, sp.num_splits) &&
+            me_attention_out_product_supported(items, nh, d, h_, sp.num_splits)))
+        return false;
+      attn_parts_.o = part_o;
+      attn_parts_.ml = part_ml;
+      attn_parts_.splits = sp.num_splits;
+      attn_parts_.nh = nh;
+      attn_parts_.d = d;
+      attn_parts_.value = op.out;
+      attn_parts_.mark = mark;
+      released_to_ = arena_.used;  // the partial results outlive this operation
+      return true;
     };
     const int chunks = (group + 15) / 16;
     if (s_.decode_only && (long long)width * bs < s_.max_ctx && mfma)
@@ -391,6 +423,7 @@ class Run {
       const SplitPlan sp = split_plan(items, nkv * chunks, s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
       float *part_o, *part_ml;
       partials(sp, part_o, part_ml);
+      if (leaves_to_product(sp, part_o, part_ml)) out = nullptr;
       ok(me_attention_decode_fused_bf16(qkv, q_w, k_w, rope, rd, eps, owns ? 1 : 0, kc, vc, idx(s_.lay.item_ctx), table, width, out,
                                         part_o, part_ml, items, nh, nkv, d, bs, window, scale, sp.split_keys, sp.num_splits,
                                         s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves, idx(s_.lay.live_items) + 1, stream_));
@@ -409,6 +442,7 @@ class Run {
       const SplitPlan sp = split_plan(items, nkv * chunks, s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
       float *part_o, *part_ml;
       partials(sp, part_o, part_ml);
+      if (leaves_to_product(sp, part_o, part_ml)) out = nullptr;
       ok(me_attention_decode_bf16(q, kc, vc, idx(s_.lay.item_ctx), table, width, out, part_o, part_ml, items, nh, nkv, d, bs, window,
                                   scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
                                   idx(s_.lay.live_items) + 1, stream_));
@@ -501,6 +535,11 @@ class Run {
   void* normed_;
   std::vector<void*> bufs_;
   Pending pending_;
+  struct AttnParts {  // what a decode attention left for the output projection behind it
+    float *o = nullptr, *ml = nullptr;
+    int splits = 0, nh = 0, d = 0, value = -1;
+    size_t mark = 0;
+  } attn_parts_;
   const Op* next_ = nullptr;  // the operation behind the one being run
   size_t parts_mark_ = (size_t)-1, released_to_ = (size_t)-1;
   RunResult result_;

@@ -41,6 +41,13 @@ int me_attention_decode_fused_bf16(const void* qkv, const float* q_w, const floa
                                    int items, int nh, int nkv, int d, int bs, int window, float scale, int split_keys,
                                    int num_splits, int max_ctx, const int* live_items, int full_splits, int waves_wanted,
                                    const int* step_flags, hipStream_t stream);
+// Decode steps of very few items: the launch leaves its splits' partial results (out == nullptr) and the output
+// projection adds them up itself.
+int me_attention_decode_leaves_parts(int items, int nh, int nkv, int d, int num_splits);
+int me_attention_out_product_runs(int nh);
+int me_attention_out_product_supported(int items, int nh, int d, int n, int num_splits);
+int me_attention_out_product_bf16(const float* part_o, const float* part_ml, int num_splits, const void* W, float* parts,
+                                  int items, int nh, int d, int n, hipStream_t stream);
 int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items, const int* block_table,
                               int table_width, void* out, const int* work, const int* bundle_first, int num_bundles,
                               float* part_o, float* part_ml, const int* token_chunks, int max_chunks, int num_tokens, int nh,

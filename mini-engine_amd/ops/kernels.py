@@ -421,6 +421,13 @@ def carried_norm_choice(dtype: torch.dtype, rows: int, n: int, k: int, next_rows
                                              _i(units), _i(int(aligned))))
 
 
+def split_sum_choice(dtype: torch.dtype, rows: int, n: int, aligned: bool = True) -> bool:
+    """Whether the step program lets the output projection (``n`` = hidden columns) behind a decode attention of ``rows``
+    items add up the attention's splits itself (:func:`attention_out_product_bf16`): the rule of ``csrc/host/choice.cpp``;
+    no GPU is touched."""
+    return bool(lib().me_split_sum_choice(_i(_code(dtype)), _i(rows), _i(n), _i(int(aligned))))
+
+
 STREAM_MAX_ROWS = 256  # the weight-streaming product deals more than 64 rows to groups of blocks
 SMALL_MAX_ROWS = 64  # what the small matrix-core kernel accepts
 
@@ -771,12 +778,22 @@ def _decode_split_plan(items: int, kv_units: int, max_ctx: int, live):
     return keys, splits, count, min(full, splits)
 
 
+def attention_decode_leaves_parts(items: int, num_heads: int, num_kv_heads: int, head_dim: int, num_splits: int) -> bool:
+    """Whether a decode launch of these sizes leaves one partial result per split (which a second kernel, or
+    :func:`attention_out_product_bf16` in its place, adds up): the launches that may be asked to ``leave_parts``."""
+    return bool(lib().me_attention_decode_leaves_parts(_i(items), _i(num_heads), _i(num_kv_heads), _i(head_dim),
+                                                       _i(num_splits)))
+
+
 def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: float, window: int, max_ctx: int,
-                          out: torch.Tensor | None = None, live=None, step_flags: torch.Tensor | None = None) -> torch.Tensor:
+                          out: torch.Tensor | None = None, live=None, step_flags: torch.Tensor | None = None,
+                          leave_parts: bool = False):
     """Attention of one new token per item over its cached keys: q [items, nh, d] bfloat16,
     item_ctx int32 [items] (keys per item, the new one included, each <= max_ctx). ``live``: see
     :func:`_decode_split_plan`. ``step_flags``: None, or a device int32 whose bit 0 says that the items share
-    pages (a large launch then loads keys and values with ordinary loads instead of non-temporal ones)."""
+    pages (a large launch then loads keys and values with ordinary loads instead of non-temporal ones).
+    ``leave_parts``: the splits are not added up; the result is ``(part_o, part_ml, num_splits)`` for
+    :func:`attention_out_product_bf16` (only where :func:`attention_decode_leaves_parts` says so)."""
     _want(q, "q", torch.bfloat16, (None, None, None))
     items, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -789,14 +806,17 @@ def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: flo
     split_keys, num_splits, live_count, full_splits = _decode_split_plan(items, nkv * chunks, max_ctx, live)
     part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=q.device)
-    if out is None:
-        out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=q.device)
-    _want(out, "out", torch.bfloat16, (items, nh * d))
+    if leave_parts:
+        out = None
+    else:
+        if out is None:
+            out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=q.device)
+        _want(out, "out", torch.bfloat16, (items, nh * d))
     check(lib().me_attention_decode_bf16(
         _p(q), _p(k_cache), _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out),
         _p(part_o), _p(part_ml), _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys),
         _i(num_splits), _i(max_ctx), _p(live_count), _i(full_splits), _i(DECODE_WAVES), _p(step_flags), _stream()))
-    return out
+    return (part_o, part_ml, num_splits) if leave_parts else out
 
 
 def attention_decode_fused_supported(head_dim: int, block_size: int, rotary_dim: int, group: int) -> bool:
@@ -807,11 +827,11 @@ def attention_decode_fused_supported(head_dim: int, block_size: int, rotary_dim:
 def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write_kv: bool, k_cache, v_cache, item_ctx,
                                 block_table, num_heads: int, scale: float, window: int, max_ctx: int,
                                 out: torch.Tensor | None = None, live=None,
-                                step_flags: torch.Tensor | None = None) -> torch.Tensor:
+                                step_flags: torch.Tensor | None = None, leave_parts: bool = False):
     """One new token per item, from the raw q/k/v projection: what :func:`qk_norm_rope_scatter` followed
     by :func:`attention_decode_bf16` compute, in one launch. qkv [items, (nh + 2 nkv) d] bfloat16
-    (or [items, nh d] with ``write_kv`` off). ``live``: see :func:`_decode_split_plan`; ``step_flags`` as in
-    :func:`attention_decode_bf16`."""
+    (or [items, nh d] with ``write_kv`` off). ``live``: see :func:`_decode_split_plan`; ``step_flags`` and
+    ``leave_parts`` as in :func:`attention_decode_bf16`."""
     nkv, bs, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     nh = num_heads
     _want(qkv, "qkv", torch.bfloat16, (None, ((nh + 2 * nkv) if write_kv else nh) * d))
@@ -834,15 +854,42 @@ def attention_decode_fused_bf16(qkv, q_weight, k_weight, rope, eps: float, write
     split_keys, num_splits, live_count, full_splits = _decode_split_plan(items, nkv * chunks, max_ctx, live)
     part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=qkv.device)
     part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=qkv.device)
-    if out is None:
-        out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=qkv.device)
-    _want(out, "out", torch.bfloat16, (items, nh * d))
+    if leave_parts:
+        out = None
+    else:
+        if out is None:
+            out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=qkv.device)
+        _want(out, "out", torch.bfloat16, (items, nh * d))
     check(lib().me_attention_decode_fused_bf16(
         _p(qkv), _p(q_weight), _p(k_weight), _p(rope), _i(rd), _f(eps), _i(1 if write_kv else 0), _p(k_cache),
         _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out), _p(part_o), _p(part_ml),
         _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys), _i(num_splits), _i(max_ctx),
         _p(live_count), _i(full_splits), _i(DECODE_WAVES), _p(step_flags), _stream()))
-    return out
+    return (part_o, part_ml, num_splits) if leave_parts else out
+
+
+def attention_out_product_supported(items: int, num_heads: int, head_dim: int, width: int, num_splits: int) -> bool:
+    """Whether :func:`attention_out_product_bf16` takes these sizes."""
+    return bool(lib().me_attention_out_product_supported(_i(items), _i(num_heads), _i(head_dim), _i(width), _i(num_splits)))
+
+
+def attention_out_product_bf16(part_o, part_ml, num_splits: int, weight, items: int, num_heads: int) -> torch.Tensor:
+    """The output projection of a decode step of very few items, from the partial results that a decode attention
+    launch left (``leave_parts``): the splits are added up and rounded to bfloat16 as the second attention kernel
+    does, and multiplied with weight [n, nh d]. The result is float32 [runs, items, n]: sums over runs of k that the
+    next add-and-norm adds up."""
+    _want(weight, "weight", torch.bfloat16, (None, None))
+    n, k = weight.shape
+    if k % num_heads:
+        raise ValueError(f"a weight of {k} columns does not hold {num_heads} heads")
+    d = k // num_heads
+    _want(part_o, "part_o", torch.float32, (items * num_heads * num_splits * d,))
+    _want(part_ml, "part_ml", torch.float32, (items * num_heads * num_splits * 2,))
+    runs = lib().me_attention_out_product_runs(_i(num_heads))
+    parts = torch.empty((runs, items, n), dtype=torch.float32, device=weight.device)
+    check(lib().me_attention_out_product_bf16(_p(part_o), _p(part_ml), _i(num_splits), _p(weight), _p(parts), _i(items),
+                                              _i(num_heads), _i(d), _i(n), _stream()))
+    return parts
 
 
 class PrefillPlan:

@@ -821,6 +821,45 @@ def test_attention_decode_of_a_launch_large_enough_to_stream(nh, nkv, d, bs, max
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])  # the kind of load changes no bit
 
 
+@pytest.mark.parametrize("nh,nkv,d,width", [(16, 8, 128, 1024), (32, 8, 128, 4096), (6, 2, 64, 200), (64, 8, 128, 5120),
+                                            (3, 1, 64, 72)])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4])
+def test_output_projection_that_adds_up_the_splits_of_decode_attention(nh, nkv, d, width, rows):
+    """A decode step of very few items leaves the splits' partial results to its output projection: the product equals
+    the one of the finished attention output (the second kernel's, rounded to bfloat16) with the same weight, summed
+    over its runs of k; a far key that dominates lies in another split than the rest."""
+    dtype = torch.bfloat16
+    bs, max_ctx = 16, 4096
+    ctxs = [700, 3000, 65, 4096][:rows]
+    items = [(c - 1, 1) for c in ctxs]
+    k_cache, v_cache, tables, table_t, positions, token_item, ks, vs = make_paged(items, nkv, d, bs, dtype, num_pages=520)
+    g = torch.Generator().manual_seed(21)
+    qs = [torch.randn(1, nh, d, generator=g).to(dtype) for _ in items]
+    ks[0][5] = (qs[0][0, 0].float() * 3).to(dtype)  # one early key that the first head of item 0 finds among hundreds
+    fill_new(k_cache, v_cache, tables, ks, vs, [(0, c) for c in ctxs], bs)
+    scale = d**-0.5
+    item_ctx = torch.tensor(ctxs, dtype=torch.int32)
+    wide = torch.zeros(len(items), max_ctx // bs, dtype=torch.int32)
+    wide[:, : table_t.shape[1]] = table_t
+    weight = (torch.randn(width, nh * d, generator=g) * (nh * d) ** -0.5).to(dtype)
+    args = (dev(torch.cat(qs)), dev(k_cache), dev(v_cache), dev(item_ctx), dev(wide), scale, 0, max_ctx)
+    out = K().attention_decode_bf16(*args)
+    assert_attention_close(out, dense_reference(qs, ks, vs, items, scale, 0))
+    part_o, part_ml, splits = K().attention_decode_bf16(*args, leave_parts=True)
+    assert K().attention_decode_leaves_parts(rows, nh, nkv, d, splits)
+    if not K().attention_out_product_supported(rows, nh, d, width, splits):
+        from mini_engine_amd.ops.library import KernelError
+
+        with pytest.raises(KernelError, match="not supported"):
+            K().attention_out_product_bf16(part_o, part_ml, splits, dev(weight), rows, nh)
+        return  # (more (row, head) pairs than a block takes, or too many heads for a run of k)
+    parts = K().attention_out_product_bf16(part_o, part_ml, splits, dev(weight), rows, nh)
+    want = out.float().cpu() @ weight.float().T
+    got = parts.sum(0).cpu()
+    assert parts.shape[1:] == (rows, width)
+    torch.testing.assert_close(got, want, rtol=0, atol=2**-12 * float(want.abs().max()))
+
+
 @pytest.mark.parametrize("nh,nkv,d,bs", [(16, 8, 128, 16), (4, 2, 64, 16), (6, 1, 96, 32)])
 def test_attention_decode_with_fewer_live_items_than_the_grid_holds(nh, nkv, d, bs):
     """A launch laid out for as few as `least` live items (a replayed graph: the rest is padding) has

@@ -133,3 +133,19 @@ def test_the_tiny_models_of_the_gpu_tests_leave_their_norms_to_the_products_behi
         for rows in (3, 8, 16):
             assert K.carried_norm_choice(BF16, rows, hidden, width, 2 * inter, True, 256) == (name != "E"), name
             assert K.carried_norm_choice(BF16, rows, hidden, inter, qkv_rows, False, 256) == (name != "E"), name
+
+
+def test_the_output_projection_adds_up_the_splits_of_one_item_for_narrow_models_only():
+    """One item a step, up to 1,024 hidden columns: the output projection behind decode attention reads the splits'
+    partial results itself (the 0.6B shape and the tiny models C and D, whose head sizes its kernel takes); wider
+    models, more items and float32 keep the kernel that adds the splits up."""
+    from conftest import tiny_configs
+
+    for shape, (hidden, heads, kv, d, inter) in SHAPES.items():
+        for rows in (1, 2, 3, 8, 64):
+            assert K.split_sum_choice(BF16, rows, hidden) == (rows == 1 and shape == "0.6b"), (shape, rows)
+            assert not K.split_sum_choice(F32, rows, hidden)
+            assert not K.split_sum_choice(BF16, rows, hidden, aligned=False)
+    for name in ("C", "D"):
+        cfg = tiny_configs()[name]
+        assert K.split_sum_choice(BF16, 1, cfg.hidden_size) and not K.split_sum_choice(BF16, 2, cfg.hidden_size)

@@ -156,6 +156,27 @@ def test_long_contexts_in_portions_and_decoded(tiny_folders, name, dtype):
     assert not session.live
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_one_long_request_decoded_alone(tiny_folders, name):
+    """One item a step behind a context of 1,500: decode attention in two dozen splits, which the output projection
+    adds up itself at these widths (no kernel of its own does; tests/test_product_choice.py says that these models take
+    that path). The last twelve tokens one by one, every one's logits against the plain implementation."""
+    vocab = tiny_configs()[name].vocab_size
+    reqs = {"solo": random_prompt(1500, vocab, seed=33)}
+    from mini_engine_amd.engine.trace import TraceSession, build_session
+
+    session = TraceSession(build_session(tiny_folders[name], "bfloat16", 1536, block_size=BLOCK_SIZES[name]))
+    want = th.plain_logits(tiny_folders[name], reqs)
+    out = torch.from_numpy(session.run_step({"step": 0, "entries": [{"id": "solo", "tokens": reqs["solo"][:1488], "want": [1487]}],
+                                             "end": []}).copy())
+    th.assert_logits_close(out, want["solo"][[1487]], "bfloat16", f"{name} prompt")
+    for i in range(1488, 1500):
+        out = torch.from_numpy(session.run_step({"step": i, "entries": [{"id": "solo", "tokens": [reqs["solo"][i]], "want": [0]}],
+                                                 "end": ["solo"] if i == 1499 else []}).copy())
+        th.assert_logits_close(out, want["solo"][[i]], "bfloat16", f"{name} token {i}")
+    assert not session.live
+
+
 def test_first_tokens_of_a_sequence(tiny_folders):
     """Positions 0 and 1 alone: a one-token prompt, then its second token."""
     for name in ("A", "B"):
