@@ -752,11 +752,11 @@ def attention_mfma_supported(head_dim: int, block_size: int, group: int = 1) -> 
 
 def decode_splits(items: int, kv_units: int, max_ctx: int, target_waves: int = 1024) -> tuple[int, int]:
     """(keys per split, number of splits) for the decode kernel: enough waves to fill the chip,
-    splits of at least 64 keys, boundaries at multiples of 64."""
+    splits of at least 64 keys, whole tiles of 16."""
     units = max(1, items * kv_units)
     splits = max(1, min(-(-target_waves // units), max(max_ctx, 64) // 64))
     split_keys = -(-max_ctx // splits)
-    split_keys = -(-split_keys // 64) * 64
+    split_keys = -(-split_keys // 16) * 16
     return split_keys, -(-max_ctx // split_keys)
 
 
