@@ -106,8 +106,10 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
 
 // The same for rows whose length is a multiple of 4 and at most 16 elements per thread: a thread keeps its four
 // vectors of 4 sums in registers (one pass over memory), loads 16 bytes at a time and has the loads of four
-// partial sums in flight at once (a row of 5,120 with 7 partial sums: 41 -> 7 us).
-template <typename T>
+// partial sums in flight at once (a row of 5,120 with 7 partial sums: 41 -> 7 us). PB partial sums are requested
+// together (4, or 8 where there are more than 4: a trip to memory for all of them instead of one for four and one for
+// each of the rest); a run beyond the last reads the last one again and counts for nothing.
+template <typename T, int PB>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,
                                        int num_parts, size_t part_stride, const float* __restrict__ w, T* __restrict__ h,
                                        const int* __restrict__ rows, int dim, float eps, int write_x) {
@@ -137,20 +139,15 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const T* __restric
       if (pr) {  // in the order of the runs
         float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
         const float* at = pr + 4 * v;
-        int q = 0;
-        for (; q + 4 <= num_parts; q += 4) {
-          const float4 a = *reinterpret_cast<const float4*>(at + (size_t)q * part_stride);
-          const float4 b = *reinterpret_cast<const float4*>(at + (size_t)(q + 1) * part_stride);
-          const float4 c = *reinterpret_cast<const float4*>(at + (size_t)(q + 2) * part_stride);
-          const float4 e = *reinterpret_cast<const float4*>(at + (size_t)(q + 3) * part_stride);
-          d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
-          d.x += b.x, d.y += b.y, d.z += b.z, d.w += b.w;
-          d.x += c.x, d.y += c.y, d.z += c.z, d.w += c.w;
-          d.x += e.x, d.y += e.y, d.z += e.z, d.w += e.w;
-        }
-        for (; q < num_parts; ++q) {
-          const float4 a = *reinterpret_cast<const float4*>(at + (size_t)q * part_stride);
-          d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
+        for (int q = 0; q < num_parts; q += PB) {
+          float4 pv[PB];
+#pragma unroll
+          for (int i = 0; i < PB; ++i) pv[i] = *reinterpret_cast<const float4*>(at + (size_t)min(q + i, num_parts - 1) * part_stride);
+#pragma unroll
+          for (int i = 0; i < PB; ++i) {
+            const float on = q + i < num_parts ? 1.f : 0.f;
+            d.x += on * pv[i].x, d.y += on * pv[i].y, d.z += on * pv[i].z, d.w += on * pv[i].w;
+          }
         }
         s[it].x += d.x, s[it].y += d.y, s[it].z += d.z, s[it].w += d.w;
       }
@@ -185,8 +182,12 @@ static bool launch_add_rmsnorm_vec(float* x, const T* delta, const float* parts,
   // 4.1 against 9.8; 512 rows of 4,096 5.9 against 10.0; 2,048 rows of 1,024 5.5 against 6.2). A function of the row's
   // length alone: a row's sum of squares is added up in the same order whatever the number of rows.
   const int threads = nvec <= 64 ? 64 : (nvec <= 128 ? 128 : (nvec <= 256 ? 256 : (nvec <= 512 ? 512 : 1024)));
-  add_rmsnorm_vec_kernel<T><<<num_rows, threads, 0, stream>>>(x, delta, parts, num_parts, part_stride, w, h, rows, dim, eps,
-                                                              write_x);
+  if (parts && num_parts > 4)
+    add_rmsnorm_vec_kernel<T, 8><<<num_rows, threads, 0, stream>>>(x, delta, parts, num_parts, part_stride, w, h, rows, dim, eps,
+                                                                   write_x);
+  else
+    add_rmsnorm_vec_kernel<T, 4><<<num_rows, threads, 0, stream>>>(x, delta, parts, num_parts, part_stride, w, h, rows, dim, eps,
+                                                                   write_x);
   return true;
 }
 

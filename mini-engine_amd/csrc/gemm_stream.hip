@@ -284,6 +284,79 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   }
 }
 
+// The prologue of the kernel below works on ROWS rows at a time and on four consecutive elements of each per thread:
+// s = x_in + delta or + the partial sums, in the order of their runs. What it reads of the first PB runs is requested in
+// one go (norm_fetch), and for the thread's first elements before the kernel's first weights: loads complete in the order
+// of their issue, so a prologue that asked for its rows behind the weights waited for all of those, and one that asked
+// for four runs at a time and for one row after the other took a trip to memory for each (a second row cost the kernel
+// 2.3 us, sixteen runs instead of four 0.8). A run beyond the last reads the last one again and counts for nothing; so
+// does a row beyond the last.
+template <int ROWS, int PB>
+struct NormLoads {
+  float4 sv[ROWS], wv, pv[PB][ROWS];
+  uint2 dv[ROWS];
+};
+
+template <int ROWS, int PB>
+__device__ __forceinline__ void norm_fetch(NormLoads<ROWS, PB>& ld, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+                                           const float* __restrict__ parts, int num_parts, size_t part_stride,
+                                           const float* __restrict__ w_norm, int m0, int M, int K, int v) {
+#pragma unroll
+  for (int j = 0; j < ROWS; ++j) {
+    const size_t at = (size_t)min(m0 + j, M - 1) * K + 4 * v;
+    ld.sv[j] = *reinterpret_cast<const float4*>(x_in + at);
+    ld.dv[j] = make_uint2(0, 0);
+    if (delta) ld.dv[j] = *reinterpret_cast<const uint2*>(delta + at);
+  }
+  ld.wv = *reinterpret_cast<const float4*>(w_norm + 4 * v);
+  if (parts) {
+#pragma unroll
+    for (int i = 0; i < PB; ++i)
+#pragma unroll
+      for (int j = 0; j < ROWS; ++j)
+        ld.pv[i][j] = *reinterpret_cast<const float4*>(parts + (size_t)min(i, num_parts - 1) * part_stride +
+                                                       (size_t)min(m0 + j, M - 1) * K + 4 * v);
+  }
+}
+
+// The rows' sums from what norm_fetch brought (and from the runs beyond the first PB), their squares into ss, the sums
+// themselves to x_out if given, bf16(s * w_norm) into xn.
+template <int ROWS, int PB>
+__device__ __forceinline__ void norm_finish(const NormLoads<ROWS, PB>& ld, const bf16_t* __restrict__ delta,
+                                            const float* __restrict__ parts, int num_parts, size_t part_stride,
+                                            float* __restrict__ x_out, uint16_t* xn, float (&ss)[ROWS], int m0, int M, int K, int krow,
+                                            int v) {
+#pragma unroll
+  for (int j = 0; j < ROWS; ++j) {
+    if (m0 + j >= M) break;
+    const size_t at = (size_t)(m0 + j) * K + 4 * v;
+    float4 t = ld.sv[j];
+    if (delta) {
+      t.x += __uint_as_float(ld.dv[j].x << 16), t.y += __uint_as_float(ld.dv[j].x & 0xffff0000u);
+      t.z += __uint_as_float(ld.dv[j].y << 16), t.w += __uint_as_float(ld.dv[j].y & 0xffff0000u);
+    }
+    if (parts) {
+      float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int i = 0; i < PB; ++i) {
+        const float on = i < num_parts ? 1.f : 0.f;
+        d.x += on * ld.pv[i][j].x, d.y += on * ld.pv[i][j].y, d.z += on * ld.pv[i][j].z, d.w += on * ld.pv[i][j].w;
+      }
+      for (int q = PB; q < num_parts; ++q) {
+        const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)q * part_stride + at);
+        d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
+      }
+      t.x += d.x, t.y += d.y, t.z += d.z, t.w += d.w;
+    }
+    if (x_out) *reinterpret_cast<float4*>(x_out + at) = t;
+    ss[j] = fmaf(t.x, t.x, ss[j]), ss[j] = fmaf(t.y, t.y, ss[j]), ss[j] = fmaf(t.z, t.z, ss[j]), ss[j] = fmaf(t.w, t.w, ss[j]);
+    uint2 packed;
+    packed.x = (uint32_t)f32_to_bf16_bits(t.x * ld.wv.x) | ((uint32_t)f32_to_bf16_bits(t.y * ld.wv.y) << 16);
+    packed.y = (uint32_t)f32_to_bf16_bits(t.z * ld.wv.z) | ((uint32_t)f32_to_bf16_bits(t.w * ld.wv.w) << 16);
+    *reinterpret_cast<uint2*>(xn + (size_t)(m0 + j) * krow + 4 * v) = packed;
+  }
+}
+
 // The same product for a row or a few with the residual add and the RMSNorm in front of it as its prologue:
 // the input is the float32 residual stream x_in [M, K] plus a delta (a bfloat16 tensor, or float32 partial sums
 // of the product before, added in the order of their runs, or nothing). While the weights of the first steps
@@ -292,12 +365,12 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
 // rsqrt(mean(s^2) + eps) at the end (a row's scale is a common factor of its products). Block 0 writes s to
 // x_out, which must not alias x_in: the other blocks still read it. Every block reads all of x_in and the partial
 // sums, so this is for a row or two; no runs of k across blocks.
-template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES>
-__global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
-                                                               const float* __restrict__ parts, int num_parts, size_t part_stride,
-                                                               const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
-                                                               const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N,
-                                                               int K, int gate, int rotate) {
+template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int ROWS, int PB>
+__device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+                                                      const float* __restrict__ parts, int num_parts, size_t part_stride,
+                                                      const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
+                                                      const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N, int K,
+                                                      int gate, int rotate) {
   static_assert(WN * WK == 4, "four waves per block");
   constexpr int KC = kStepK / WK, CH = KC / 32, ACCS = SWIGLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char norm_lds[];
@@ -335,53 +408,33 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
         wd[a][c] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, k < K ? (int)(w_base[a] + (k0 + 32 * c) * 2) : (int)w_bytes, 0, 0);
       }
   };
+  // ---- the prologue: every row's sum, its squares, and bf16(s * w_norm) into LDS. What the thread's first elements need
+  // is asked for before the weights.
+  float* const x_to = blockIdx.x == 0 && (delta != nullptr || parts != nullptr) ? x_out : nullptr;
+  NormLoads<ROWS, PB> ld;
+  norm_fetch<ROWS, PB>(ld, x_in, delta, parts, num_parts, part_stride, w_norm, 0, M, K, min((int)threadIdx.x, K / 4 - 1));
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int p = 0; p < STAGES; ++p) {
     load_step(p, w[p]);
     __builtin_amdgcn_sched_barrier(0);
   }
-
-  // ---- the prologue: every row's sum, its squares, and bf16(s * w_norm) into LDS
-  const bool writes_x = blockIdx.x == 0 && (delta != nullptr || parts != nullptr);
-  for (int m = 0; m < M; ++m) {
-    float ss = 0.f;
+  bool fetched = true;
+  for (int m0 = 0; m0 < M; m0 += ROWS) {
+    float ss[ROWS];
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) ss[j] = 0.f;
     for (int v = threadIdx.x; v < K / 4; v += 256) {
-      const size_t at = (size_t)m * K + 4 * v;
-      float4 sv = *reinterpret_cast<const float4*>(x_in + at);
-      if (delta) {
-        const uint2 dv = *reinterpret_cast<const uint2*>(delta + at);
-        sv.x += __uint_as_float(dv.x << 16), sv.y += __uint_as_float(dv.x & 0xffff0000u);
-        sv.z += __uint_as_float(dv.y << 16), sv.w += __uint_as_float(dv.y & 0xffff0000u);
-      }
-      if (parts) {  // in the order of the runs
-        float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
-        int q = 0;
-        for (; q + 4 <= num_parts; q += 4) {
-          const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)q * part_stride + at);
-          const float4 b = *reinterpret_cast<const float4*>(parts + (size_t)(q + 1) * part_stride + at);
-          const float4 c = *reinterpret_cast<const float4*>(parts + (size_t)(q + 2) * part_stride + at);
-          const float4 e = *reinterpret_cast<const float4*>(parts + (size_t)(q + 3) * part_stride + at);
-          d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
-          d.x += b.x, d.y += b.y, d.z += b.z, d.w += b.w;
-          d.x += c.x, d.y += c.y, d.z += c.z, d.w += c.w;
-          d.x += e.x, d.y += e.y, d.z += e.z, d.w += e.w;
-        }
-        for (; q < num_parts; ++q) {
-          const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)q * part_stride + at);
-          d.x += a.x, d.y += a.y, d.z += a.z, d.w += a.w;
-        }
-        sv.x += d.x, sv.y += d.y, sv.z += d.z, sv.w += d.w;
-      }
-      if (writes_x) *reinterpret_cast<float4*>(x_out + at) = sv;
-      ss = fmaf(sv.x, sv.x, ss), ss = fmaf(sv.y, sv.y, ss), ss = fmaf(sv.z, sv.z, ss), ss = fmaf(sv.w, sv.w, ss);
-      const float4 wv = *reinterpret_cast<const float4*>(w_norm + 4 * v);
-      uint2 packed;
-      packed.x = (uint32_t)f32_to_bf16_bits(sv.x * wv.x) | ((uint32_t)f32_to_bf16_bits(sv.y * wv.y) << 16);
-      packed.y = (uint32_t)f32_to_bf16_bits(sv.z * wv.z) | ((uint32_t)f32_to_bf16_bits(sv.w * wv.w) << 16);
-      *reinterpret_cast<uint2*>(xn + (size_t)m * krow + 4 * v) = packed;
+      if (!fetched) norm_fetch<ROWS, PB>(ld, x_in, delta, parts, num_parts, part_stride, w_norm, m0, M, K, v);
+      fetched = false;
+      norm_finish<ROWS, PB>(ld, delta, parts, num_parts, part_stride, x_to, xn, ss, m0, M, K, krow, v);
     }
-    ss = wave_sum(ss);
-    if (lane == 0) sums[m * 4 + wave] = ss;
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) {
+      if (m0 + j >= M) break;
+      const float total = wave_sum(ss[j]);
+      if (lane == 0) sums[(m0 + j) * 4 + wave] = total;
+    }
   }
   __syncthreads();
   // rows beyond M read row M - 1 and count for nothing: their results are never stored
@@ -459,6 +512,29 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
     for (int j = 0; j < 4; ++j)
       if (nb + j < N) dst[j] = from_float<OutT>(y[j]);
   }
+}
+
+// One row: up to sixteen runs of partial sums in the prologue's first request; more rows: two at a time, eight runs.
+template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES>
+__global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+                                                               const float* __restrict__ parts, int num_parts, size_t part_stride,
+                                                               const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
+                                                               const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N,
+                                                               int K, int gate, int rotate) {
+#define ME_NORM_BODY(ROWS, PB)                                                                                                  \
+  gemm_stream_norm_body<WN, WK, SWIGLU, OutT, STAGES, ROWS, PB>(x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, \
+                                                                M, N, K, gate, rotate)
+  if (M == 1) {
+    if (num_parts <= 4)
+      ME_NORM_BODY(1, 4);
+    else if (num_parts <= 8)
+      ME_NORM_BODY(1, 8);
+    else
+      ME_NORM_BODY(1, 16);
+  } else {
+    ME_NORM_BODY(2, 8);
+  }
+#undef ME_NORM_BODY
 }
 
 // How a product is laid over the chip: the waves' arrangement (wn groups of 16 columns, 4 / wn runs of k within a
