@@ -142,7 +142,9 @@ ProductChoice choose_product(int dtype, int role, int m, int rows_of_w, int k, i
 // buffer, since other blocks of the kernel still read the first.
 // A row or two: the weight-streaming kernel adds and norms the rows itself while its first weights are on their way,
 // whatever the delta is (one row: 857 -> 967 tokens/s, two: 1,605 -> 1,700; from four rows on every block's reads of
-// the partial sums cost more than the launch they save: 2,749 -> 2,668).
+// the partial sums cost more than the launch they save: 2,749 -> 2,668; measured again with the prologue's loads requested
+// together, against the carried norm below: three rows 1.289 -> 1.332 ms a step, four 1.371 -> 1.440; and the carried norm
+// at two rows against this prologue: 1.157 -> 1.177).
 // Up to 16 rows with nothing, or a tensor, to add (the first layer's norm; parts of other kinds): the small kernel's prologue.
 int choose_norm_fusion(int dtype, int m, int rows_of_w, int k, int pending, int units, bool aligned) {
   (void)units;
