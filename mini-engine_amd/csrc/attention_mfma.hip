@@ -1431,8 +1431,9 @@ extern "C" int me_attention_out_product_bf16(const float* part_o, const float* p
   if (!me_attention_out_product_supported(items, nh, d, n, num_splits))
     return me_fail("me_attention_out_product_bf16: items=%d heads=%d head_dim=%d width=%d splits=%d not supported", items, nh,
                    d, n, num_splits);
-  if (((uintptr_t)W | (uintptr_t)part_o | (uintptr_t)parts) & 15)
-    return me_fail("me_attention_out_product_bf16: operands must start at multiples of 16 bytes");
+  if (!part_o || !part_ml || !W || !parts) return me_fail("me_attention_out_product_bf16: null operand");
+  if (((uintptr_t)W | (uintptr_t)part_o | (uintptr_t)parts) & 15 || (uintptr_t)part_ml & 7)
+    return me_fail("me_attention_out_product_bf16: operands must start at multiples of 16 bytes (the statistics: of 8)");
   const int hpr = out_heads_per_run(nh);
   const int runs = (nh + hpr - 1) / hpr;
   int pairs = 1;
