@@ -646,6 +646,8 @@ void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C,
       gemm_stream_kernel<MT, 1, 4, SWIGLU, OutT, (SWIGLU ? 4 : 6), 1, true><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
     return;
   }
+  // (64 rows, blocks of 64 columns: a step more in flight, 3 gated and 4 plain, is 0.6% of a decode step of the 8B shape at
+  // batch 64 slower and 1.3% of the 32B shape's)
   if (wn == 4)
     gemm_stream_kernel<MT, 4, 1, SWIGLU, OutT, (SWIGLU ? 2 : 3)><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
   else if (wn == 2)
