@@ -376,12 +376,13 @@ def test_gemm_bf16_stream(m, n, k, gated):
 
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 1024), (2, 100, 1000), (3, 1040, 72), (4, 68, 2056), (1, 16, 128), (2, 9000, 648),
                                    (1, 3072, 1024), (2, 6142, 264), (2, 520, 2048), (1, 100, 4096)])
-@pytest.mark.parametrize("delta", ["none", "tensor", "parts3", "parts6"])
+@pytest.mark.parametrize("delta", ["none", "tensor", "parts3", "parts6", "parts11", "parts16"])
 @pytest.mark.parametrize("gated", [False, "silu", "gelu_tanh"])
 def test_gemm_bf16_stream_norm(m, n, k, delta, gated):
     """Residual add, RMSNorm and product in one launch of the weight-streaming kernel, for a row or a few: every
     arrangement of a block's waves, k that is no multiple of a step, k of 2,048 and 4,096 (whose walk over k starts at
-    another step in every block), each kind of delta (none, a tensor, partial sums in odd and even numbers), both output
+    another step in every block), each kind of delta (none, a tensor, partial sums in odd and even numbers: fewer than the
+    prologue requests at once, which are 4, 8 or 16 for one row and 8 for more, as many, and more), both output
     types and both gates; the sum goes to the second buffer and only there."""
     g = torch.Generator().manual_seed(m * 31 + n + k)
     x, wn = torch.randn(m, k, generator=g) * 2, 1 + 0.2 * torch.randn(k, generator=g)
