@@ -72,6 +72,12 @@ __device__ __forceinline__ float gate_act(float g, int code) {
   }
   return g / (1.f + expf(-g));  // silu
 }
+// The same for results that are rounded to bfloat16: the exponential and the reciprocal as one instruction each (a
+// correctly rounded division and expf are two dozen instructions at the tail of every gated product).
+__device__ __forceinline__ float gate_act_bf16(float g, int code) {
+  if (code == ME_GATE_GELU_TANH) return gate_act(g, code);
+  return g * __builtin_amdgcn_rcpf(1.f + __expf(-g));
+}
 
 // ------------------------------------------------------------------ wave and block reductions
 __device__ __forceinline__ float wave_sum(float v) {

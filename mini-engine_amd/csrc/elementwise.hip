@@ -307,7 +307,7 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int
 #pragma unroll
   for (int k = 0; k < VEC; ++k) {
     const float gf = to_float(g.v[k]);
-    o.v[k] = from_float<T>(gate_act(gf, gate) * to_float(u.v[k]));
+    o.v[k] = from_float<T>((sizeof(T) == 2 ? gate_act_bf16(gf, gate) : gate_act(gf, gate)) * to_float(u.v[k]));
   }
   *reinterpret_cast<Pack*>(act + t * inter + i) = o;
 }

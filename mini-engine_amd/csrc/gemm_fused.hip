@@ -161,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
         }
         v0 *= scale;
         float y = v0;
-        if (SWIGLU) y = gate_act(v0, gate) * (v1 * scale);
+        if (SWIGLU) y = gate_act_bf16(v0, gate) * (v1 * scale);
         const int col = nb + tile * 16 + j;
         if (col < N) C[(size_t)m * N + col] = from_float<OutT>(y);
       }

@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         y[j] = acc[t][i][j] * scale;
-        if (SWIGLU) y[j] = gate_act(y[j], gate) * (acc[t][NT + i][j] * scale);
+        if (SWIGLU) y[j] = gate_act_bf16(y[j], gate) * (acc[t][NT + i][j] * scale);
       }
       OutT* dst = C + (size_t)m * N + nb;
       if (nb + 3 < N && (N & 3) == 0) {
@@ -494,7 +494,7 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     y[j] = acc[0][j] * scale;
-    if (SWIGLU) y[j] = gate_act(y[j], gate) * (acc[1][j] * scale);
+    if (SWIGLU) y[j] = gate_act_bf16(y[j], gate) * (acc[1][j] * scale);
   }
   OutT* dst = C + (size_t)m * N + nb;
   if (nb >= c1) return;
