@@ -25,12 +25,9 @@ struct bf16_t {
 __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest, ties to even
-  return (uint16_t)(u >> 16);
-}
+// Round to nearest, ties to even; NaN stays NaN: the hardware's conversion (gfx950 has one; by integer arithmetic this
+// is six instructions a value, which the tails and inner loops of the small kernels feel).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 template <typename T>
 __device__ __forceinline__ T from_float(float f);
