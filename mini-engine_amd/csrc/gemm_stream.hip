@@ -37,12 +37,29 @@ constexpr int kStepK = 128;          // k per block and step
 constexpr int kGroupRows = 64;       // rows per block; more rows are dealt to groups of blocks (the grid's third dimension)
 constexpr int kMaxRows = 256;
 constexpr int kBufferFlags = 0x00020000;  // a raw buffer of 32-bit words (gfx9 family)
+// How the grid's first dimension deals the columns out, in fours, as evenly as they go: block b takes `q` fours, the first
+// `r` blocks one more. Worked out on the host: the same from blockIdx and gridDim by division cost every block some four
+// hundred scalar instructions before it could ask for its first weights. `rotate`: whether a block walks k from a step of
+// its own.
+struct ColumnDeal {
+  int q, r, rotate;
+};
+__device__ __forceinline__ int deal_first(const ColumnDeal& d, int b) { return (b * d.q + min(b, d.r)) * 4; }
+inline ColumnDeal deal_of(int N, int grid, bool rotate) {
+  const int fours = (N + 3) / 4;
+  return {fours / grid, fours % grid, rotate ? 1 : 0};
+}
+// (no division either: a multiplicative hash of the block's number, scaled to [0, steps))
+__device__ __forceinline__ int deal_turn(unsigned b, int steps) {
+  return (int)((((b * 0x9E3779B1u) >> 16) * (unsigned)steps) >> 16);
+}
+
 constexpr int kRow = kStepK + 16;    // LDS row stride in elements: 288 bytes, 32 off a multiple of 64 (conflict-free 16-byte reads)
 
 template <int MT, int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int NT = 1, bool AUX = false>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                           OutT* __restrict__ C, int rows, int N, int K, int steps_per_split, int gate,
-                                                          int rotate, RowScale rs, CarryOut carry) {
+                                                          ColumnDeal deal, RowScale rs, CarryOut carry) {
   static_assert(WN * WK == 4, "four waves per block");
   static_assert(NT == 1 || WK == 1, "waves with several tiles of columns do not cut k");
   // The grid's third dimension deals the rows out in groups of 16 MT; a block sees its group's rows only.
@@ -65,9 +82,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   }
   // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN NT) blocks gives every
   // block 16 WN NT columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
-  const int fours = (N + 3) / 4;
-  const int c0 = (int)((long long)blockIdx.x * fours / gridDim.x) * 4;
-  const int c1 = min(N, (int)((long long)(blockIdx.x + 1) * fours / gridDim.x) * 4);
+  const int c0 = deal_first(deal, blockIdx.x);
+  const int c1 = min(N, deal_first(deal, blockIdx.x + 1));
   const int n0 = c0 + wn * NT * 16;  // the wave's first tile; tile i begins 16 i columns on
 
   const int total_steps = (K + kStepK - 1) / kStepK;
@@ -107,7 +123,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   suint4_t w[STAGES][ACCS][CH], xreg[STAGES][XV];
   // With `rotate` a block walks its steps of k from a step of its own on, around the end of its run: the blocks that start
   // together then read different memory channels (rows of W that lie a multiple of 4 KiB apart begin in the same one).
-  const int rot = rotate ? (int)((blockIdx.x * 5u + blockIdx.z) % (unsigned)max(steps, 1)) : 0;
+  const int rot = deal.rotate ? deal_turn(blockIdx.x * 5u + blockIdx.z, steps) : 0;
   auto load_step = [&](int step, suint4_t (&wd)[ACCS][CH], suint4_t (&xd)[XV]) {
     int turned = step + rot;
     if (turned >= steps) turned -= steps;
@@ -370,7 +386,7 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
                                                       const float* __restrict__ parts, int num_parts, size_t part_stride,
                                                       const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
                                                       const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N, int K,
-                                                      int gate, int rotate) {
+                                                      int gate, ColumnDeal deal) {
   static_assert(WN * WK == 4, "four waves per block");
   constexpr int KC = kStepK / WK, CH = KC / 32, ACCS = SWIGLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char norm_lds[];
@@ -382,9 +398,8 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
   const int r = lane & 15, g = lane >> 4;
   // The block's columns: the grid deals N out in fours, as evenly as they go (a grid of N / (16 WN) blocks gives every
   // block 16 WN columns; a larger one gives each fewer, and the rest of its last tile of 16 is neither fetched nor stored).
-  const int fours = (N + 3) / 4;
-  const int c0 = (int)((long long)blockIdx.x * fours / gridDim.x) * 4;
-  const int c1 = min(N, (int)((long long)(blockIdx.x + 1) * fours / gridDim.x) * 4);
+  const int c0 = deal_first(deal, blockIdx.x);
+  const int c1 = min(N, deal_first(deal, blockIdx.x + 1));
   const int n0 = c0 + wn * 16;
   const int n = n0 + r;
   const int steps = (K + kStepK - 1) / kStepK;
@@ -396,7 +411,7 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
   for (int a = 0; a < ACCS; ++a) w_base[a] = n < c1 ? (uint32_t)(((SWIGLU && a ? N : 0) + n) * K + wk * KC + g * 8) * 2 : w_bytes;
   suint4_t w[STAGES][ACCS][CH];
   // (with `rotate` the block's walk over k starts at a step of its own and goes around the end, as in the kernel above)
-  const int rot = rotate ? (int)((blockIdx.x * 5u) % (unsigned)steps) : 0;
+  const int rot = deal.rotate ? deal_turn(blockIdx.x * 5u, steps) : 0;
   auto turned = [&](int step) { return step + rot < steps ? step + rot : step + rot - steps; };
   auto load_step = [&](int step, suint4_t (&wd)[ACCS][CH]) {
     const int k0 = (step < steps ? turned(step) : steps) * kStepK;  // (steps past the end: beyond K, nothing is fetched)
@@ -520,10 +535,10 @@ __global__ __launch_bounds__(256) void gemm_stream_norm_kernel(const float* __re
                                                                const float* __restrict__ parts, int num_parts, size_t part_stride,
                                                                const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
                                                                const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N,
-                                                               int K, int gate, int rotate) {
+                                                               int K, int gate, ColumnDeal deal) {
 #define ME_NORM_BODY(ROWS, PB)                                                                                                  \
   gemm_stream_norm_body<WN, WK, SWIGLU, OutT, STAGES, ROWS, PB>(x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, \
-                                                                M, N, K, gate, rotate)
+                                                                M, N, K, gate, deal)
   if (M == 1) {
     if (num_parts <= 4)
       ME_NORM_BODY(1, 4);
@@ -629,7 +644,7 @@ void launch_arranged(StreamPlan plan, const bf16_t* X, const bf16_t* W, OutT* C,
   // walk over k at a step of its own instead (39.4 us; at 1 and 8 rows 42.7 -> 40.5 and 43.1 -> 41.0; 6,144 x 4,096 at 32
   // rows 15.5 -> 14.3). Runs of k across blocks start at different k already, and other strides spread by themselves
   // (k = 5,120: no change either way), so those keep the plain walk.
-  const int rotate = plan.splits == 1 && K % 2048 == 0;
+  const ColumnDeal rotate = deal_of(N, plan.grid, plan.splits == 1 && K % 2048 == 0);
   if constexpr (MT >= 3 && !SWIGLU && sizeof(OutT) == 4) {
     if (plan.nt == 2) {  // (two steps in flight: 3-15% ahead of three)
       gemm_stream_kernel<MT, 4, 1, false, OutT, 2, 2><<<grid, 256, 0, stream>>>(X, W, C, M, N, K, steps_per_split, gate, rotate, rs, carry);
@@ -767,7 +782,7 @@ int launch_norm(StreamPlan plan, const float* x_in, const bf16_t* delta, const f
 #define ME_NORM_LAUNCH(WN, WK, STAGES)                                                                                   \
   gemm_stream_norm_kernel<WN, WK, SWIGLU, OutT, STAGES><<<grid, 256, lds, stream>>>(x_in, delta, parts, num_parts, part_stride, \
                                                                                     w_norm, eps, x_out, W, C, M, N, K, gate, \
-                                                                                    K % 2048 == 0)
+                                                                                    deal_of(N, plan.grid, K % 2048 == 0))
   if (wn == 4)
     ME_NORM_LAUNCH(4, 1, (SWIGLU ? 2 : 3));
   else if (wn == 2)
