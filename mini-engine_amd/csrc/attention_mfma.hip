@@ -127,6 +127,8 @@ __device__ __forceinline__ void compute_tile(const KvTile<D>& t, int key0, int l
     float p[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) p[i] = fast_exp2(sv[i] - m_ref);
+    // (the column's sum per tile: with the four lanes of a column keeping sums of their own until the split is done,
+    // as the prefill kernel does, steps at batch 1 and 64 are 0.5-0.9% longer and only long contexts gain)
     lsum[nb] = lsum[nb] * alpha + column_sum((p[0] + p[1]) + (p[2] + p[3]));
     m[nb] = m_new;
 #pragma unroll
@@ -947,7 +949,9 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
     for (int i = 0; i < 16; ++i) p[i] = fast_exp2(fmaf(sv[i], scale_log2, -m_ref));
     const float psum = (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))) +
                        (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
-    lsum[nb] = fmaf(lsum[nb], alpha, column_sum(psum));
+    // the lane's own keys: the four lanes of a column scale their sums alike (the maximum is the column's) and add them
+    // up once, behind the loop over keys (8,192 and 32,704 tokens 1.9% faster than with the column's sum per tile)
+    lsum[nb] = fmaf(lsum[nb], alpha, psum);
     m[nb] = m_new;
     // The running maximum rarely moves after the first tiles: the rescale of the accumulator is skipped
     // when no column of the wave needs it. The multiplication is written as instructions that work in
@@ -1091,6 +1095,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     }
     __syncthreads();
   }
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) lsum[nb] = column_sum(lsum[nb]);
   if (w.chunk >= 0) {
     // one range of several: the unnormalised sums and the statistics of every column
 #pragma unroll
