@@ -134,6 +134,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(
   }
   if (SCALED && rs.ss) row_scales_finish<SCALE_ROWS>(rs, M, ss_part, row_scale, wave, lane, WAVES);
   __syncthreads();
+  if constexpr (!NORM) {
+    // Every thread of the block adds up one output element over the waves (thread -> tile t, lane l, element j: row
+    // m = 16 t + l % 16, column n0 + 4 (l / 16) + j): eight or sixteen reads of LDS in a row instead of the 32 or 64
+    // that a thread had with one wave doing the whole tail.
+    for (int e = threadIdx.x; e < MT * 256; e += WAVES * 64) {
+      const int t = e >> 8, l = (e >> 2) & 63, j = e & 3;
+      const int m = t * 16 + (l & 15);
+      if (m >= M) continue;
+      const float scale = SCALED && rs.ss ? row_scale[m] : 1.f;
+#pragma unroll
+      for (int tile = 0; tile < (SWIGLU ? 1 : NT); ++tile) {
+        float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+          v0 += red[w][t * ACCS + tile][l][j];
+          if (SWIGLU) v1 += red[w][t * ACCS + 1][l][j];
+        }
+        v0 *= scale;
+        float y = v0;
+        if (SWIGLU) y = gate_act_bf16(v0, gate) * (v1 * scale);
+        const int col = n0 + (l >> 4) * 4 + tile * 16 + j;
+        if (col < N) C[(size_t)m * N + col] = from_float<OutT>(y);
+      }
+    }
+    return;
+  }
   // thread -> (tile t, lane l): row m = 16 t + l % 16, columns n0 + 4 (l / 16) .. +4
   for (int idx = threadIdx.x; idx < MT * 64; idx += WAVES * 64) {
     const int t = idx / 64, l = idx % 64;
