@@ -194,7 +194,37 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     row_scales_finish<MT * 4>(rs, M, ss_part, row_scale, wave, lane, 4);
     __syncthreads();
   }
-  if (WK > 1) {  // the runs of k within a step: waves wk > 0 hand their sums to wave wk == 0 of their columns
+  // With as many tiles of rows as runs of k within a step (or a multiple), every wave finishes the tiles t with
+  // t % WK == wk: it hands the sums of the other tiles to their waves and adds up what they hand to it, so that the
+  // sums, the gate and the stores of a block of 64 rows are four waves' work and not one's.
+  constexpr bool SHARE_TAIL = WK > 1 && MT > 1 && MT % WK == 0;
+  if constexpr (SHARE_TAIL) {
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(&xs[0][0][0]);  // [wk][wn][t][a][j][lane]
+    constexpr int PER_WAVE = MT * ACCS * 4 * 64;
+    static_assert(WK * WN * PER_WAVE * 4 <= (int)sizeof(xs), "the partial sums fit the x tiles' memory");
+    float* mine = red + (wk * WN + wn) * PER_WAVE;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      if (t % WK != wk)
+#pragma unroll
+        for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mine[((t * ACCS + a) * 4 + j) * 64 + lane] = acc[t][a][j];
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      if (t % WK == wk)
+#pragma unroll
+        for (int o = 0; o < WK; ++o)
+          if (o != wk) {
+            const float* theirs = red + (o * WN + wn) * PER_WAVE;
+#pragma unroll
+            for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) acc[t][a][j] += theirs[((t * ACCS + a) * 4 + j) * 64 + lane];
+          }
+  } else if (WK > 1) {  // the runs of k within a step: waves wk > 0 hand their sums to wave wk == 0 of their columns
     __syncthreads();
     float* red = reinterpret_cast<float*>(&xs[0][0][0]);  // [wk - 1][wn][t][a][j][lane]
     constexpr int PER_WAVE = MT * ACCS * 4 * 64;
@@ -229,6 +259,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
       const size_t row0 = (size_t)blockIdx.z * (16 * MT);
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
+        if (SHARE_TAIL && t % WK != wk) continue;
         const int m = t * 16 + r;
         float sq = 0.f;
 #pragma unroll
@@ -272,6 +303,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     if (nb >= c1) continue;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
+      if (SHARE_TAIL && t % WK != wk) continue;
       const int m = t * 16 + r;
       if (m >= M) continue;
       const float scale = AUX && rs.ss ? row_scale[m] : 1.f;
