@@ -143,9 +143,13 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   // A delta that adds itself to the stream (carry.x): the elements of the stream and of the norm's weight that this lane
   // will add to and multiply with at the end are requested here, ahead of everything, so that the kernel's tail does not
   // wait for memory once more. (Whole groups of four columns only; a ragged edge is read at the end.)
+  // With as many tiles of rows as runs of k within a step (or a multiple), every wave finishes the tiles t with
+  // t % WK == wk: it hands the sums of the other tiles to their waves and adds up what they hand to it, so that the
+  // sums, the gate and the stores of a block of 64 rows are four waves' work and not one's.
+  constexpr bool SHARE_TAIL = WK > 1 && MT > 1 && MT % WK == 0;
   float4 x_early[AUX ? MT : 1][AUX ? NT : 1], wn_early[AUX ? NT : 1];
   if constexpr (AUX && !SWIGLU && sizeof(OutT) == 4) {
-    if (carry.x && wk == 0 && (N & 3) == 0) {
+    if (carry.x && (SHARE_TAIL || wk == 0) && (N & 3) == 0) {
       const size_t row0 = (size_t)blockIdx.z * (16 * MT);
 #pragma unroll
       for (int i = 0; i < NT; ++i) {
@@ -154,7 +158,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
           wn_early[i] = *reinterpret_cast<const float4*>(carry.w_norm + nb);
 #pragma unroll
           for (int t = 0; t < MT; ++t)
-            if (t * 16 + r < M) x_early[t][i] = *reinterpret_cast<const float4*>(carry.x + (row0 + t * 16 + r) * N + nb);
+            if ((!SHARE_TAIL || t % WK == wk) && t * 16 + r < M)
+              x_early[t][i] = *reinterpret_cast<const float4*>(carry.x + (row0 + t * 16 + r) * N + nb);
         }
       }
     }
@@ -194,10 +199,6 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     row_scales_finish<MT * 4>(rs, M, ss_part, row_scale, wave, lane, 4);
     __syncthreads();
   }
-  // With as many tiles of rows as runs of k within a step (or a multiple), every wave finishes the tiles t with
-  // t % WK == wk: it hands the sums of the other tiles to their waves and adds up what they hand to it, so that the
-  // sums, the gate and the stores of a block of 64 rows are four waves' work and not one's.
-  constexpr bool SHARE_TAIL = WK > 1 && MT > 1 && MT % WK == 0;
   if constexpr (SHARE_TAIL) {
     __syncthreads();
     float* red = reinterpret_cast<float*>(&xs[0][0][0]);  // [wk][wn][t][a][j][lane]
